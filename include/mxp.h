@@ -1,0 +1,297 @@
+/*
+ * mxp.h - C ABI of the MI355X weight-placement engine (libmxplace.so).
+ *
+ * The library turns safetensors byte ranges on local storage into one serving rank's
+ * parameter buffers in HBM: host-staged ingest through a bounded ring of pinned
+ * buffers, then hand-written gfx950 kernels for tensor-parallel slicing, QKV / gate_up
+ * fusing, MoE expert stacking, fp32->bf16 refit casts, fp8 block-scale tile slicing and
+ * per-tensor checksums.
+ *
+ * The boundary is plain C: opaque handles, pointers and sizes.  Device pointers are
+ * ordinary HIP device addresses owned by the caller; a `stream` argument is a
+ * `hipStream_t` passed as `void*` (NULL = the default stream).  Every function
+ * returns MXP_OK (0) or a negative MXP_ERR_* class; the text of the last error on the
+ * calling thread is available from mxp_last_error().  Handles are not re-entrant: use
+ * one plan / engine from one thread at a time.
+ *
+ * Each entry point names the piece of the reference (ai-dynamo/modelexpress,
+ * modelexpress_client/python/modelexpress/...) whose behaviour it replaces.
+ */
+#ifndef MXP_H_
+#define MXP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MXP_ABI_VERSION 1
+
+/* ---- status codes -------------------------------------------------------- */
+#define MXP_OK 0
+#define MXP_ERR_IO (-1)          /* open / read failure, short file, offset past EOF     */
+#define MXP_ERR_FORMAT (-2)      /* malformed safetensors header or index                */
+#define MXP_ERR_UNSUPPORTED (-3) /* dtype outside the map, unsupported layout            */
+#define MXP_ERR_COVERAGE (-4)    /* unmapped tensor / uncovered parameter (fail closed)  */
+#define MXP_ERR_ARG (-5)         /* bad argument                                         */
+#define MXP_ERR_DEVICE (-6)      /* HIP runtime error                                    */
+#define MXP_ERR_STATE (-7)       /* call out of order                                    */
+#define MXP_ERR_VERIFY (-8)      /* checksum / digest mismatch                           */
+
+/* Text of the last error raised on the calling thread ("" if none). */
+const char* mxp_last_error(void);
+int mxp_abi_version(void);
+
+/* ---- dtypes: the safetensors dtype map of gds_loader.py:36-49 ------------- */
+#define MXP_DTYPE_F64 0
+#define MXP_DTYPE_F32 1
+#define MXP_DTYPE_F16 2
+#define MXP_DTYPE_BF16 3
+#define MXP_DTYPE_F8_E4M3 4
+#define MXP_DTYPE_F8_E5M2 5
+#define MXP_DTYPE_I64 6
+#define MXP_DTYPE_I32 7
+#define MXP_DTYPE_I16 8
+#define MXP_DTYPE_I8 9
+#define MXP_DTYPE_U8 10
+#define MXP_DTYPE_BOOL 11
+#define MXP_MAX_DIMS 8
+
+/* Bytes per element, or 0 for an unknown code. */
+int mxp_dtype_size(int dtype);
+/* "BF16" -> MXP_DTYPE_BF16; -1 when the string is not in the map. */
+int mxp_dtype_from_name(const char* safetensors_name);
+const char* mxp_dtype_name(int dtype);
+
+/* =========================================================================
+ * 1. Checkpoint: safetensors discovery and header parse
+ *    replaces MxGdsLoader._resolve_safetensors_files (gds_loader.py:189-243)
+ *    and MxGdsLoader._parse_safetensors_header (gds_loader.py:245-282).
+ * ========================================================================= */
+typedef struct mxp_ckpt mxp_ckpt;
+
+typedef struct mxp_tensor_info {
+  const char* name;   /* owned by the checkpoint handle */
+  int32_t dtype;      /* MXP_DTYPE_* */
+  int32_t ndim;
+  int64_t shape[MXP_MAX_DIMS];
+  int32_t file_index; /* which shard file */
+  int32_t reserved;
+  uint64_t file_offset; /* absolute: 8 + header_len + data_offsets[0] */
+  uint64_t nbytes;      /* data_offsets[1] - data_offsets[0] */
+} mxp_tensor_info;
+
+typedef struct mxp_file_info {
+  const char* path;
+  uint64_t file_size;
+  uint64_t data_start; /* 8 + header_len */
+  int64_t n_tensors;
+} mxp_file_info;
+
+/* `model_path` is a directory (model.safetensors.index.json, then model.safetensors,
+ * then *.safetensors in sorted order) or a single .safetensors file.  Rejects files
+ * shorter than 8 bytes, headers above 100 MiB, dtypes outside the map, data ranges
+ * that run past the end of the file. */
+int mxp_ckpt_open(const char* model_path, mxp_ckpt** out);
+void mxp_ckpt_close(mxp_ckpt* ckpt);
+int64_t mxp_ckpt_tensor_count(const mxp_ckpt* ckpt);
+int64_t mxp_ckpt_file_count(const mxp_ckpt* ckpt);
+/* Tensors are listed per file in ascending file offset (gds_loader.py:297-300). */
+int mxp_ckpt_tensor_info(const mxp_ckpt* ckpt, int64_t index, mxp_tensor_info* out);
+int mxp_ckpt_file_info(const mxp_ckpt* ckpt, int64_t index, mxp_file_info* out);
+/* Index of the tensor called `name`, or -1. */
+int64_t mxp_ckpt_find(const mxp_ckpt* ckpt, const char* name);
+
+/* =========================================================================
+ * 2. Placement plan: destination map for one rank
+ *    replaces MdlLoader._extend_dest_map / _resolve_write / _warm_load resolution
+ *    (engines/vllm/refit/installer.py:341-437,470-564), _tp_local_tensor (:292-317),
+ *    _tp_shape_compatible (:319-339), _fused_destinations (:566-616),
+ *    _premerged_destination / _premerged_writes (:629-693), _resolve_expert (:695-754),
+ *    _assert_loaderless_coverage (:219-251), _check_moe_swizzle (:833-843), and the
+ *    run decomposition of refit/reshard/slice_plan.py:259-294.
+ *
+ *    The caller describes the rank's parameters (what the serving engine allocated:
+ *    name, dtype, local shape), the stacked-parameter groups and the expert mapping,
+ *    exactly the three things MdlLoader reads off the model object.  mxp_plan_build
+ *    resolves EVERY checkpoint tensor to its destination box before anything is
+ *    written; any unmapped tensor or uncovered parameter fails the whole plan.
+ * ========================================================================= */
+typedef struct mxp_plan mxp_plan;
+
+#define MXP_PLAN_ALLOW_CAST_F32_BF16 0x1u /* F32 source into BF16 parameter (refit)       */
+#define MXP_PLAN_ALLOW_UNMAPPED 0x2u      /* skip checkpoint tensors with no destination  */
+#define MXP_PLAN_ALLOW_UNCOVERED 0x4u     /* allow parameters no tensor writes            */
+#define MXP_PLAN_NO_FP8_BLOCK_CHECK 0x8u  /* do not require 128-aligned fp8 scale slicing */
+
+int mxp_plan_create(const mxp_ckpt* ckpt, int32_t tp_size, int32_t tp_rank, uint32_t flags,
+                    mxp_plan** out);
+void mxp_plan_destroy(mxp_plan* plan);
+/* Returns the parameter index (>= 0) or a negative error. */
+int64_t mxp_plan_add_param(mxp_plan* plan, const char* name, int32_t dtype, int32_t ndim,
+                           const int64_t* shape);
+/* One (fused_suffix, member_suffix) pair of the model's stacked_params_mapping, in pack
+ * order.  With none added, the built-in groups apply: qkv_proj <- q_proj,k_proj,v_proj
+ * and gate_up_proj <- gate_proj,up_proj (installer.py:72-78,773-797). */
+int mxp_plan_add_stacked(mxp_plan* plan, const char* fused_suffix, const char* member_suffix);
+/* One row of the model's get_expert_mapping(): shard is "w1", "w2" or "w3";
+ * `local_expert_id` is the slot in the rank's stacked parameter, or -1 when the
+ * expert is not local to this rank (such tensors are then skipped, not an error). */
+int mxp_plan_add_expert(mxp_plan* plan, const char* param_prefix, const char* weight_prefix,
+                        int32_t expert_id, const char* shard, int32_t local_expert_id);
+/* Skip checkpoint tensors whose name starts with `prefix` (e.g. other pipeline stages). */
+int mxp_plan_add_skip_prefix(mxp_plan* plan, const char* prefix);
+int mxp_plan_build(mxp_plan* plan);
+
+#define MXP_WRITE_DIRECT 0
+#define MXP_WRITE_FUSED 1
+#define MXP_WRITE_EXPERT 2
+#define MXP_WRITE_PREMERGED 3
+
+typedef struct mxp_write_info {
+  int64_t tensor_index; /* source tensor in the checkpoint */
+  int64_t param_index;  /* destination parameter */
+  int32_t kind;         /* MXP_WRITE_* */
+  int32_t cast;         /* 1 when fp32 -> bf16 */
+  /* The write as a pitched box, in bytes of the respective dtype. */
+  uint64_t src_offset;  /* from the start of the source tensor's data */
+  uint64_t src_pitch;
+  uint64_t dst_offset;  /* from the start of the destination parameter */
+  uint64_t dst_pitch;
+  uint64_t rows;
+  uint64_t row_bytes;   /* destination bytes per row */
+  /* Number of maximal runs contiguous in both source and destination
+   * (what slice_plan.paired_runs would enumerate). */
+  uint64_t paired_runs;
+} mxp_write_info;
+
+typedef struct mxp_param_info {
+  const char* name;
+  int32_t dtype;
+  int32_t ndim;
+  int64_t shape[MXP_MAX_DIMS];
+  uint64_t nbytes;
+  uint64_t bytes_written; /* by the plan; == nbytes when fully covered */
+  int32_t n_writes;
+  int32_t reserved;
+} mxp_param_info;
+
+int64_t mxp_plan_param_count(const mxp_plan* plan);
+int64_t mxp_plan_write_count(const mxp_plan* plan);
+int mxp_plan_param_info(const mxp_plan* plan, int64_t index, mxp_param_info* out);
+int mxp_plan_write_info(const mxp_plan* plan, int64_t index, mxp_write_info* out);
+/* Bytes read from storage, bytes that cross PCIe and bytes placed, for one execute. */
+int mxp_plan_totals(const mxp_plan* plan, uint64_t* file_bytes, uint64_t* h2d_bytes,
+                    uint64_t* placed_bytes, uint64_t* kernel_algorithmic_bytes);
+
+/* =========================================================================
+ * 3. Engine: pinned ring, HIP streams, kernels
+ *    replaces the host-staged ingest of the ModelStreamer path
+ *    (VllmAdapter.build_model_streamer_weight_iter, engines/vllm/adapter.py:233-292 ->
+ *    runai-model-streamer reader threads -> per-tensor copy_ inside model.load_weights,
+ *    adapter.py:223-231) and the per-file batch load of gds_loader.py:284-331; the
+ *    device side replaces destination.copy_(source) (installer.py:419-424), the
+ *    narrow().contiguous() gather (installer.py:317), the staged re-slice and dtype
+ *    conversion of refit/reshard/receiver.py:919-971.
+ * ========================================================================= */
+typedef struct mxp_engine mxp_engine;
+
+typedef struct mxp_engine_options {
+  int32_t device;          /* HIP device ordinal */
+  int32_t ring_slots;      /* pinned host slots (each with a device bounce slot); 0 = default 8 */
+  uint64_t slot_bytes;     /* bytes per slot; 0 = default 64 MiB */
+  int32_t reader_threads;  /* pread workers; 0 = default 8 */
+  int32_t streams;         /* HIP streams for H2D + kernels; 0 = default 4 */
+  uint32_t tile_bytes;     /* destination bytes per workgroup; 0 = default 64 KiB */
+  uint16_t nan_bits;       /* bf16 image of every NaN in the cast; 0 = default 0x7FC0 */
+  uint16_t reserved0;
+  int32_t use_o_direct;    /* 1 = open files with O_DIRECT (falls back if unsupported) */
+} mxp_engine_options;
+
+typedef struct mxp_exec_stats {
+  double wall_seconds;     /* entry to last stream idle */
+  double read_seconds;     /* summed over reader threads */
+  double kernel_ms;        /* HIP-event time of placement kernels (resident mode) */
+  uint64_t file_bytes;     /* read from storage */
+  uint64_t h2d_bytes;      /* copied host -> device */
+  uint64_t placed_bytes;   /* written into parameter buffers */
+  uint64_t n_chunks;
+  uint64_t n_segments;
+  uint64_t n_workgroups;
+  uint64_t n_launches;
+  int32_t mutated;         /* 1 once any destination byte may have been written */
+  int32_t reserved;
+} mxp_exec_stats;
+
+int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out);
+void mxp_engine_destroy(mxp_engine* engine);
+
+/* Lowers `plan` to the engine's descriptor tables and chunk list without running it
+ * (mxp_execute does this on first use); afterwards mxp_plan_totals is complete. */
+int mxp_prepare(mxp_engine* engine, mxp_plan* plan);
+
+/* Ingest from storage: reader threads pread each planned byte range into a pinned
+ * slot, the slot is copied to its device bounce slot with hipMemcpyAsync on one of
+ * the engine's streams, and the placement kernel for that slot runs on the same
+ * stream.  `dst_ptrs[i]` is the device address of parameter i (16-byte aligned,
+ * mxp_plan_param_info().nbytes long).  Blocks until every stream is idle.  Per
+ * parameter checksums are left in the plan (mxp_plan_checksums). */
+int mxp_execute(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs, mxp_exec_stats* stats);
+
+/* Same placement with the checkpoint already staged in HBM: `file_dev_ptrs[f]` holds
+ * the complete bytes of shard file f (16-byte aligned).  One kernel launch on `stream`
+ * for the whole plan; asynchronous unless `stats` is non-NULL (then it synchronises and
+ * reports the HIP-event time of the launch in stats->kernel_ms). */
+int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* file_dev_ptrs,
+                         void* const* dst_ptrs, void* stream, mxp_exec_stats* stats);
+
+/* Checksums accumulated by the last execute, one per parameter (tensor_utils.py:27-44
+ * over the parameter's row-major bytes).  Synchronises the engine first. */
+int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_t n);
+
+/* =========================================================================
+ * 4. Stand-alone device operators (all batched: one launch for n tensors)
+ * ========================================================================= */
+/* safe_checksum (tensor_utils.py:27-44) of n device buffers:
+ *   out[k] = sum_i byte_i * ((i * 2654435761 + 1) mod 2^32) mod 2^32. */
+int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
+                   uint32_t* out, void* stream);
+/* tensor_digest (refit/reshard/verify.py:79-155) of n device buffers: 16 bytes each
+ * (blake2b-128 over the little-endian u64 scalars).  `scalars`, if not NULL, receives
+ * 7 u64 per tensor: n, sum_rows, sum_rows_weighted, sum_tail, sum_tail_weighted,
+ * sum_ragged, n % 4. */
+int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
+               uint8_t* out16, uint64_t* scalars, void* stream);
+/* fp32 -> bf16 round-to-nearest-even of `n_elems` contiguous elements (torch copy_ at
+ * modelexpress_rl/train/engines/fsdp/adapter.py:203-206, receiver.py:964-971), with the
+ * checksum of the bf16 bytes in *checksum when not NULL. */
+int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems,
+                      uint32_t* checksum, void* stream);
+/* Pitched 2-D byte gather, the device form of narrow(axis, r*n, n).contiguous()
+ * (installer.py:317) and of the as_strided re-slice (receiver.py:919-960). */
+int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* dst,
+                 uint64_t dst_pitch, uint64_t rows, uint64_t row_bytes, uint32_t* checksum,
+                 void* stream);
+/* Measured pinned host -> device bandwidth of this box in bytes per second
+ * (hipMemcpyAsync of `bytes` from a pinned buffer, best of `repeats`). */
+int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double* bytes_per_second);
+
+/* ---- host-only helpers ---------------------------------------------------- */
+/* blake2b-128 over the scalar list tensor_digest would hash (verify.py:152-155). */
+int mxp_digest_from_scalars(const uint64_t scalars[7], uint8_t out16[16]);
+
+/* Seeded synthetic contents (test and benchmark inputs; same bytes on host and device).
+ * kind: 0 ~N(0,0.02), 1 ones, 2 zeros, 3 normal with denormal/inf/NaN/tie edge cases at
+ * 1e-6 density, 4 fp8 bytes over the finite e4m3 codes, 5 fp32 scales in [1e-4,1e-2],
+ * 6 as 3 at 1/64 density. */
+int mxp_synth_host(void* dst, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed,
+                   int32_t threads);
+int mxp_synth_device(void* dst_dev, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed,
+                     void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MXP_H_ */

@@ -1,0 +1,85 @@
+// Internal (non-ABI) declarations shared by the HIP kernels and the host engine.
+//
+// Everything the device executes is driven by flat descriptor tables built on
+// the host: a "segment" is one pitched 2-D byte box (rows x row_bytes) moving
+// from a source buffer to a destination buffer, optionally through the
+// fp32->bf16 cast, with the position-weighted checksum of the bytes it writes
+// accumulated on the way.  A "work item" is one tile (a band of rows) of one
+// segment; one workgroup executes one work item, so one launch covers an
+// arbitrary mix of tensors with thousands of workgroups.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mxp {
+
+enum SegOp : uint32_t {
+  kOpCopy = 0,       // dst bytes = src bytes
+  kOpCastF32Bf16 = 1,  // src is fp32, dst is bf16 (round to nearest even)
+  kOpChecksumOnly = 2  // read src, write nothing, accumulate checksum at dst_off indices
+};
+
+// 80 bytes, 16-byte aligned; the index is workgroup-uniform, so the whole record
+// arrives through scalar loads.
+struct alignas(16) Seg {
+  uint64_t src_off;    // byte offset of the box inside source buffer `src_buf`
+  uint64_t dst_off;    // byte offset inside destination buffer `dst_buf`; also the
+                       // checksum position of the first byte
+  uint64_t src_pitch;  // bytes between consecutive rows in the source
+  uint64_t dst_pitch;  // bytes between consecutive rows in the destination
+  uint32_t rows;
+  uint32_t row_bytes;  // DESTINATION bytes per row (source bytes are 2x for the cast)
+  uint32_t src_buf;    // index into the source base-pointer table
+  uint32_t dst_buf;    // index into the destination base-pointer table
+  uint32_t op;         // SegOp
+  uint32_t unit;       // bytes per lane access on the destination side: 16, 4, 2 or 1
+  uint32_t rows_per_tile;
+  uint32_t csum_slot;  // index into the checksum accumulator array, ~0u = none
+  uint32_t units_per_row;  // row_bytes / unit
+  uint32_t div_magic;  // floor(2^32 / units_per_row) + 1, exact for n*d < 2^32
+  uint32_t pad0, pad1;
+};
+static_assert(sizeof(Seg) == 80, "Seg layout is part of the host<->device contract");
+
+struct WorkItem {
+  uint32_t seg;
+  uint32_t tile;
+};
+
+// One tensor to digest: `out` receives five u64 scalars
+// {sum_rows, sum_rows_weighted, sum_tail, sum_tail_weighted, sum_ragged}.
+struct alignas(16) DigestJob {
+  const uint8_t* ptr;
+  uint64_t nbytes;
+  uint64_t out_slot;  // index of the first of 5 u64 in the output array
+  uint64_t first_block;  // first workgroup index that belongs to this job
+};
+
+constexpr uint32_t kKnuth = 2654435761u;
+constexpr int kPlaceThreads = 256;
+constexpr uint32_t kDigestRowWords = 1024;   // 4 KiB rows
+constexpr uint32_t kDigestRowsPerBlock = 16; // 64 KiB per workgroup
+
+// ---- launch wrappers (mxp_kernels.hip) -------------------------------------
+hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
+                        const void* const* src_bases_dev, void* const* dst_bases_dev,
+                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream);
+hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
+                         unsigned long long* out_dev, hipStream_t stream);
+hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);
+
+// Synthetic-checkpoint generator (mxp_synth.hip), same arithmetic on host and device.
+enum SynthKind : uint32_t {
+  kSynthNormal = 0,   // ~N(0, 0.02): centred sum of four 16-bit uniforms times a constant
+  kSynthOnes = 1,
+  kSynthZeros = 2,
+  kSynthNormalEdge = 3,  // kSynthNormal with denormal / +-inf / NaN injected at 1e-6 density each
+  kSynthFp8Finite = 4,   // bytes uniform over the 254 finite e4m3 codes
+  kSynthScale = 5        // fp32 uniform in [1e-4, 1e-2]
+};
+hipError_t launch_synth(void* dst, uint64_t n_elems, uint32_t dtype_code, uint32_t kind,
+                        uint64_t seed, hipStream_t stream);
+void synth_host(void* dst, uint64_t n_elems, uint32_t dtype_code, uint32_t kind, uint64_t seed,
+                int threads);
+
+}  // namespace mxp

@@ -1,0 +1,829 @@
+// Engine: lowers a built plan to device descriptor tables and executes it, either by
+// ingesting the planned byte ranges from storage through a bounded ring of pinned host
+// slots (pread -> hipMemcpyAsync -> placement kernel, one HIP stream per slot group), or
+// from a checkpoint already staged in HBM (one launch for the whole plan).
+//
+// Ownership: the caller owns every destination buffer; the engine owns the pinned ring,
+// the device bounce slots, streams, events and descriptor tables.  All HIP work issued
+// by a call has completed when the call returns, unless documented otherwise.
+#include <fcntl.h>
+#include <hip/hip_runtime.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <chrono>
+#include <condition_variable>
+#include <cstring>
+#include <memory>
+#include <mutex>
+#include <thread>
+
+#include "mxp_blake2b.hpp"
+#include "mxp_internal.hpp"
+#include "mxp_lower.hpp"
+
+namespace mxp {
+namespace {
+
+#define HIP_OK(expr)                                                                          \
+  do {                                                                                        \
+    const hipError_t e_ = (expr);                                                             \
+    if (e_ != hipSuccess)                                                                     \
+      throw Error(MXP_ERR_DEVICE, std::string(#expr) + ": " + hipGetErrorString(e_));         \
+  } while (0)
+
+double now_s() {
+  return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
+}
+uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+template <typename T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t cap = 0;
+  void reserve(size_t n) {
+    if (n <= cap) return;
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    cap = 0;
+    HIP_OK(hipMalloc(reinterpret_cast<void**>(&p), n * sizeof(T)));
+    cap = n;
+  }
+  void upload(const T* host, size_t n) {
+    reserve(n ? n : 1);
+    if (n) HIP_OK(hipMemcpy(p, host, n * sizeof(T), hipMemcpyHostToDevice));
+  }
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+};
+
+struct Slot {
+  uint8_t* host = nullptr;  // pinned
+  uint8_t* dev = nullptr;   // bounce
+  hipEvent_t done = nullptr;
+  std::mutex mu;
+  std::condition_variable cv;
+  uint64_t submitted = 0;  // number of chunks this slot has carried to the GPU
+};
+
+}  // namespace mxp
+
+using namespace mxp;
+
+struct mxp_plan::Lowered {
+  uint64_t slot_bytes = 0;
+  uint32_t tile_bytes = 0;
+  // resident tables: source buffer index = shard file index
+  DevBuf<Seg> res_segs;
+  DevBuf<WorkItem> res_work;
+  uint32_t res_n_work = 0, res_n_segs = 0;
+  // ingest tables: source buffer index 0 = the chunk's bounce slot
+  std::vector<Chunk> chunks;
+  DevBuf<Seg> ing_segs;
+  DevBuf<WorkItem> ing_work;
+  uint32_t ing_n_segs = 0, ing_n_work = 0;
+  // per execute
+  DevBuf<void*> dst_bases;
+  DevBuf<const void*> src_bases;
+  DevBuf<uint32_t> sums;
+  std::vector<void*> dst_host;        // what dst_bases currently holds
+  std::vector<const void*> src_host;  // what src_bases currently holds
+  uint64_t file_bytes = 0, h2d_bytes = 0, placed_bytes = 0, algo_bytes = 0;
+};
+
+struct mxp_engine {
+  mxp_engine_options opt{};
+  std::vector<std::unique_ptr<Slot>> slots;
+  uint8_t* pinned_base = nullptr;
+  uint8_t* bounce_base = nullptr;
+  std::vector<hipStream_t> streams;
+  DevBuf<const void*> slot_ptrs;  // device table: slot i -> bounce address
+  // descriptor staging for the stand-alone operators
+  uint8_t* desc_host = nullptr;  // pinned
+  size_t desc_host_cap = 0;
+  DevBuf<uint8_t> desc_dev;
+  hipEvent_t ev_a = nullptr, ev_b = nullptr;
+
+  ~mxp_engine() {
+    for (auto s : streams) (void)hipStreamDestroy(s);
+    for (auto& s : slots)
+      if (s->done) (void)hipEventDestroy(s->done);
+    if (pinned_base) (void)hipHostFree(pinned_base);
+    if (bounce_base) (void)hipFree(bounce_base);
+    if (desc_host) (void)hipHostFree(desc_host);
+    if (ev_a) (void)hipEventDestroy(ev_a);
+    if (ev_b) (void)hipEventDestroy(ev_b);
+  }
+};
+
+namespace mxp {
+namespace {
+
+void free_lowered(mxp_plan::Lowered* l) { delete l; }
+
+// Splits every write into slot-sized pieces, packs their byte ranges into chunks in
+// (file, offset) order, and lowers both the ingest and the resident descriptor tables.
+void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
+  if (!pl.built) throw Error(MXP_ERR_STATE, "plan has not been built");
+  if (pl.lowered && pl.lowered->slot_bytes == eng.opt.slot_bytes && pl.lowered->tile_bytes == eng.opt.tile_bytes)
+    return;
+  if (pl.lowered) { free_lowered(pl.lowered); pl.lowered = nullptr; }
+  auto L = std::make_unique<mxp_plan::Lowered>();
+  L->slot_bytes = eng.opt.slot_bytes;
+  L->tile_bytes = eng.opt.tile_bytes;
+  LowerOptions lo;
+  lo.tile_bytes = eng.opt.tile_bytes;
+  const mxp_ckpt& ck = *pl.ckpt;
+
+  // ---- resident: one box per write, source = staged shard file ----
+  {
+    std::vector<Seg> segs;
+    std::vector<WorkItem> work;
+    for (const auto& w : pl.writes) {
+      const TensorRec& t = ck.tensors[w.tensor];
+      BoxCopy b;
+      b.src_buf = (uint32_t)t.file_index;
+      b.dst_buf = (uint32_t)w.param;
+      b.src_off = t.file_offset + w.src_offset;
+      b.dst_off = w.dst_offset;
+      b.src_pitch = w.src_pitch;
+      b.dst_pitch = w.dst_pitch;
+      b.rows = w.rows;
+      b.row_bytes = w.row_bytes;
+      b.op = w.cast ? kOpCastF32Bf16 : kOpCopy;
+      b.csum_slot = (uint32_t)w.param;
+      lower_box(b, lo, segs, work);
+      L->placed_bytes += w.rows * w.row_bytes;
+      L->algo_bytes += w.rows * w.row_bytes * (w.cast ? 3 : 2);
+    }
+    L->res_n_segs = (uint32_t)segs.size();
+    L->res_n_work = (uint32_t)work.size();
+    L->res_segs.upload(segs.data(), segs.size());
+    L->res_work.upload(work.data(), work.size());
+  }
+
+  // ---- ingest: pieces in file order ----
+  struct Piece {
+    int file;
+    uint64_t file_off, nbytes;  // byte range to read
+    BoxCopy box;                // src_off relative to the start of the range
+  };
+  std::vector<Piece> pieces;
+  const uint64_t slot = eng.opt.slot_bytes;
+  for (const auto& w : pl.writes) {
+    const TensorRec& t = ck.tensors[w.tensor];
+    const uint64_t sm = w.cast ? 2 : 1;
+    const uint64_t row_src = w.row_bytes * sm;
+    BoxCopy b;
+    b.src_buf = 0;
+    b.dst_buf = (uint32_t)w.param;
+    b.op = w.cast ? kOpCastF32Bf16 : kOpCopy;
+    b.csum_slot = (uint32_t)w.param;
+    const uint64_t t0 = t.file_offset + w.src_offset;
+    if (w.rows == 1 || (w.src_pitch == row_src && w.dst_pitch == w.row_bytes)) {
+      // contiguous run: split on 4 KiB multiples of destination bytes
+      const uint64_t total = w.rows * w.row_bytes;
+      const uint64_t max_dst = (slot / sm) / 4096 * 4096;
+      for (uint64_t done = 0; done < total; done += max_dst) {
+        const uint64_t n = std::min(max_dst, total - done);
+        Piece p{t.file_index, t0 + done * sm, n * sm, b};
+        p.box.src_off = 0;
+        p.box.dst_off = w.dst_offset + done;
+        p.box.rows = 1;
+        p.box.row_bytes = n;
+        p.box.src_pitch = n * sm;
+        p.box.dst_pitch = n;
+        pieces.push_back(p);
+      }
+    } else {
+      // strided source: stage whole row bands and gather on the device
+      if (w.src_pitch > slot || row_src > slot)
+        throw Error(MXP_ERR_UNSUPPORTED, "a source row of '" + t.name + "' does not fit a staging slot");
+      const uint64_t max_rows = (slot - row_src) / w.src_pitch + 1;
+      for (uint64_t r = 0; r < w.rows; r += max_rows) {
+        const uint64_t nr = std::min(max_rows, w.rows - r);
+        Piece p{t.file_index, t0 + r * w.src_pitch, (nr - 1) * w.src_pitch + row_src, b};
+        p.box.src_off = 0;
+        p.box.dst_off = w.dst_offset + r * w.dst_pitch;
+        p.box.rows = nr;
+        p.box.row_bytes = w.row_bytes;
+        p.box.src_pitch = w.src_pitch;
+        p.box.dst_pitch = w.dst_pitch;
+        pieces.push_back(p);
+      }
+    }
+  }
+  std::stable_sort(pieces.begin(), pieces.end(), [](const Piece& a, const Piece& b) {
+    return a.file != b.file ? a.file < b.file : a.file_off < b.file_off;
+  });
+  {
+    std::vector<Seg> segs;
+    std::vector<WorkItem> work;
+    Chunk cur;
+    auto close = [&] {
+      if (cur.ranges.empty()) return;
+      cur.seg_count = (uint32_t)segs.size() - cur.seg_begin;
+      cur.work_count = (uint32_t)work.size() - cur.work_begin;
+      L->h2d_bytes += cur.used_bytes;
+      L->chunks.push_back(cur);
+      cur = Chunk();
+    };
+    for (auto& p : pieces) {
+      uint64_t at = align_up(cur.used_bytes, 256);
+      if (!cur.ranges.empty() && at + p.nbytes > slot) {
+        close();
+        at = 0;
+      }
+      if (cur.ranges.empty()) {
+        cur.seg_begin = (uint32_t)segs.size();
+        cur.work_begin = (uint32_t)work.size();
+      }
+      cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at});
+      cur.used_bytes = at + p.nbytes;
+      L->file_bytes += p.nbytes;
+      p.box.src_off = at;
+      const size_t w0 = work.size();
+      lower_box(p.box, lo, segs, work);
+      // work items index segments relative to the chunk's first segment
+      for (size_t k = w0; k < work.size(); ++k) work[k].seg -= cur.seg_begin;
+    }
+    close();
+    L->ing_n_segs = (uint32_t)segs.size();
+    L->ing_n_work = (uint32_t)work.size();
+    L->ing_segs.upload(segs.data(), segs.size());
+    L->ing_work.upload(work.data(), work.size());
+  }
+  L->dst_bases.reserve(pl.params.size() ? pl.params.size() : 1);
+  L->src_bases.reserve(ck.files.size() ? ck.files.size() : 1);
+  L->sums.reserve(pl.params.size() ? pl.params.size() : 1);
+  pl.lowered = L.release();
+  pl.lowered_free = free_lowered;
+}
+
+void check_dst(const mxp_plan& pl, void* const* dst_ptrs) {
+  if (!dst_ptrs) throw Error(MXP_ERR_ARG, "dst_ptrs is null");
+  for (size_t i = 0; i < pl.params.size(); ++i) {
+    if (pl.params[i].n_writes == 0) continue;
+    if (!dst_ptrs[i]) throw Error(MXP_ERR_ARG, "destination of parameter '" + pl.params[i].name + "' is null");
+    if (reinterpret_cast<uintptr_t>(dst_ptrs[i]) & 15u)
+      throw Error(MXP_ERR_ARG, "destination of parameter '" + pl.params[i].name + "' is not 16-byte aligned");
+  }
+}
+
+// Pointer tables are re-sent only when the caller's pointers changed since the last call.
+void upload_dst(mxp_plan::Lowered& L, const mxp_plan& pl, void* const* dst_ptrs) {
+  const size_t n = pl.params.size();
+  if (L.dst_host.size() == n && std::equal(L.dst_host.begin(), L.dst_host.end(), dst_ptrs)) return;
+  L.dst_bases.upload(dst_ptrs, n);
+  L.dst_host.assign(dst_ptrs, dst_ptrs + n);
+}
+
+void pread_full(int fd, uint8_t* dst, uint64_t n, uint64_t off, const std::string& path) {
+  while (n) {
+    const ssize_t r = ::pread(fd, dst, (size_t)std::min<uint64_t>(n, 1ull << 30), (off_t)off);
+    if (r < 0) {
+      if (errno == EINTR) continue;
+      throw Error(MXP_ERR_IO, "read failed on " + path + ": " + std::strerror(errno));
+    }
+    if (r == 0) throw Error(MXP_ERR_IO, "unexpected end of file in " + path + " at offset " + std::to_string(off));
+    dst += r;
+    off += (uint64_t)r;
+    n -= (uint64_t)r;
+  }
+}
+
+void ensure_desc(mxp_engine& e, size_t bytes) {
+  if (bytes > e.desc_host_cap) {
+    if (e.desc_host) (void)hipHostFree(e.desc_host);
+    e.desc_host = nullptr;
+    e.desc_host_cap = 0;
+    const size_t cap = align_up(bytes * 2, 1 << 16);
+    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e.desc_host), cap, hipHostMallocDefault));
+    e.desc_host_cap = cap;
+  }
+  e.desc_dev.reserve(e.desc_host_cap);
+}
+
+// Runs a batch of boxes whose sources / destinations are raw device pointers.
+// Layout of the descriptor arena: [segs][work][src ptrs][dst ptrs][sums].
+void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vector<const void*>& srcs,
+               const std::vector<void*>& dsts, uint32_t n_sums, uint32_t* sums_out, hipStream_t stream) {
+  LowerOptions lo;
+  lo.tile_bytes = e.opt.tile_bytes;
+  std::vector<Seg> segs;
+  std::vector<WorkItem> work;
+  for (const auto& b : boxes) lower_box(b, lo, segs, work);
+  const size_t o_segs = 0;
+  const size_t o_work = align_up(o_segs + segs.size() * sizeof(Seg), 256);
+  const size_t o_src = align_up(o_work + work.size() * sizeof(WorkItem), 256);
+  const size_t o_dst = align_up(o_src + srcs.size() * sizeof(void*), 256);
+  const size_t o_sum = align_up(o_dst + dsts.size() * sizeof(void*), 256);
+  const size_t total = align_up(o_sum + (size_t)n_sums * 4, 256);
+  HIP_OK(hipStreamSynchronize(stream));  // the arena may still feed an earlier launch
+  ensure_desc(e, total);
+  std::memset(e.desc_host, 0, total);
+  if (!segs.empty()) std::memcpy(e.desc_host + o_segs, segs.data(), segs.size() * sizeof(Seg));
+  if (!work.empty()) std::memcpy(e.desc_host + o_work, work.data(), work.size() * sizeof(WorkItem));
+  if (!srcs.empty()) std::memcpy(e.desc_host + o_src, srcs.data(), srcs.size() * sizeof(void*));
+  if (!dsts.empty()) std::memcpy(e.desc_host + o_dst, dsts.data(), dsts.size() * sizeof(void*));
+  HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, total, hipMemcpyHostToDevice, stream));
+  uint8_t* d = e.desc_dev.p;
+  HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + o_segs), reinterpret_cast<const WorkItem*>(d + o_work),
+                      (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + o_src),
+                      reinterpret_cast<void* const*>(d + o_dst), reinterpret_cast<uint32_t*>(d + o_sum),
+                      e.opt.nan_bits, stream));
+  if (sums_out && n_sums) {
+    HIP_OK(hipMemcpyAsync(e.desc_host + o_sum, d + o_sum, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::memcpy(sums_out, e.desc_host + o_sum, (size_t)n_sums * 4);
+  } else {
+    // the pinned arena is read by the copy above; later calls synchronise before reuse
+  }
+}
+
+// Splits an arbitrary device pointer into a 16-byte aligned base and an offset, so the
+// lowering can pick the widest access the true address allows.
+inline void split_ptr(const void* p, const void*& base, uint64_t& off) {
+  const uintptr_t v = reinterpret_cast<uintptr_t>(p);
+  off = v & 15u;
+  base = reinterpret_cast<const void*>(v - off);
+}
+
+}  // namespace
+}  // namespace mxp
+
+extern "C" {
+
+int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
+  return guard([&] {
+    if (!out) throw Error(MXP_ERR_ARG, "mxp_engine_create: null out");
+    *out = nullptr;
+    auto e = std::make_unique<mxp_engine>();
+    if (opts) e->opt = *opts;
+    auto& o = e->opt;
+    if (o.ring_slots <= 0) o.ring_slots = 8;
+    if (o.slot_bytes == 0) o.slot_bytes = 64ull << 20;
+    if (o.reader_threads <= 0) o.reader_threads = 8;
+    if (o.streams <= 0) o.streams = 4;
+    if (o.tile_bytes == 0) o.tile_bytes = 64 * 1024;
+    if (o.nan_bits == 0) o.nan_bits = 0x7FC0;
+    if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
+    if (o.tile_bytes < 1024 || o.tile_bytes > (1u << 20)) throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 1 MiB]");
+    if (o.ring_slots > 256 || o.reader_threads > 256 || o.streams > 64) throw Error(MXP_ERR_ARG, "ring, thread or stream count too large");
+    int n_dev = 0;
+    HIP_OK(hipGetDeviceCount(&n_dev));
+    if (n_dev <= 0) throw Error(MXP_ERR_DEVICE, "no HIP device is visible");
+    if (o.device < 0 || o.device >= n_dev) throw Error(MXP_ERR_ARG, "device ordinal out of range");
+    HIP_OK(hipSetDevice(o.device));
+    for (int s = 0; s < o.streams; ++s) {
+      hipStream_t st;
+      HIP_OK(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+      e->streams.push_back(st);
+    }
+    HIP_OK(hipEventCreate(&e->ev_a));
+    HIP_OK(hipEventCreate(&e->ev_b));
+    *out = e.release();
+  });
+}
+
+void mxp_engine_destroy(mxp_engine* engine) {
+  if (!engine) return;
+  (void)hipSetDevice(engine->opt.device);
+  (void)hipDeviceSynchronize();
+  delete engine;
+}
+
+}  // extern "C"
+
+namespace mxp {
+namespace {
+
+// The ring is allocated on first ingest so that engines used only for resident
+// placement or the stand-alone operators hold no pinned memory.
+void ensure_ring(mxp_engine& e) {
+  if (!e.slots.empty()) return;
+  const auto& o = e.opt;
+  const size_t total = (size_t)o.ring_slots * o.slot_bytes;
+  HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e.pinned_base), total, hipHostMallocDefault));
+  HIP_OK(hipMalloc(reinterpret_cast<void**>(&e.bounce_base), total));
+  std::vector<const void*> ptrs;
+  for (int s = 0; s < o.ring_slots; ++s) {
+    auto sl = std::make_unique<Slot>();
+    sl->host = e.pinned_base + (size_t)s * o.slot_bytes;
+    sl->dev = e.bounce_base + (size_t)s * o.slot_bytes;
+    HIP_OK(hipEventCreateWithFlags(&sl->done, hipEventDisableTiming));
+    ptrs.push_back(sl->dev);
+    e.slots.push_back(std::move(sl));
+  }
+  e.slot_ptrs.upload(ptrs.data(), ptrs.size());
+}
+
+void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_stats* stats) {
+  const double t_start = now_s();
+  HIP_OK(hipSetDevice(e.opt.device));
+  check_dst(pl, dst_ptrs);
+  lower_plan(pl, e);
+  ensure_ring(e);
+  auto& L = *pl.lowered;
+  const mxp_ckpt& ck = *pl.ckpt;
+  if (stats) std::memset(stats, 0, sizeof *stats);
+
+  std::vector<int> fds(ck.files.size(), -1);
+  struct FdCloser {
+    std::vector<int>& f;
+    ~FdCloser() { for (int fd : f) if (fd >= 0) ::close(fd); }
+  } closer{fds};
+  for (size_t f = 0; f < ck.files.size(); ++f) {
+    int flags = O_RDONLY;
+#ifdef O_DIRECT
+    if (e.opt.use_o_direct) flags |= O_DIRECT;
+#endif
+    fds[f] = ::open(ck.files[f].path.c_str(), flags);
+    if (fds[f] < 0 && e.opt.use_o_direct) fds[f] = ::open(ck.files[f].path.c_str(), O_RDONLY);
+    if (fds[f] < 0) throw Error(MXP_ERR_IO, "cannot open " + ck.files[f].path + ": " + std::strerror(errno));
+  }
+
+  // Everything below may change destination bytes.
+  upload_dst(L, pl, dst_ptrs);
+  HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, e.streams[0]));
+  HIP_OK(hipStreamSynchronize(e.streams[0]));
+  for (auto& s : e.slots) s->submitted = 0;
+
+  std::atomic<size_t> next{0};
+  std::atomic<bool> abort{false};
+  std::atomic<int> mutated{0};
+  std::mutex err_mu;
+  std::unique_ptr<Error> first_err;
+  std::vector<double> read_s((size_t)e.opt.reader_threads, 0.0);
+  const size_t n_chunks = L.chunks.size();
+  const size_t n_slots = e.slots.size();
+
+  auto worker = [&](int tid) {
+    try {
+      HIP_OK(hipSetDevice(e.opt.device));
+      for (;;) {
+        const size_t c = next.fetch_add(1);
+        if (c >= n_chunks || abort.load()) break;
+        const Chunk& ch = L.chunks[c];
+        Slot& sl = *e.slots[c % n_slots];
+        const uint64_t turn = c / n_slots;
+        {
+          // Wait until the previous chunk carried by this slot has been submitted, then
+          // until the GPU has finished with it.
+          std::unique_lock<std::mutex> lk(sl.mu);
+          sl.cv.wait(lk, [&] { return sl.submitted == turn || abort.load(); });
+        }
+        if (abort.load()) break;
+        if (turn > 0) HIP_OK(hipEventSynchronize(sl.done));
+        const double t0 = now_s();
+        for (const auto& r : ch.ranges)
+          pread_full(fds[r.file], sl.host + r.slot_off, r.nbytes, r.file_off, ck.files[r.file].path);
+        read_s[tid] += now_s() - t0;
+        hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
+        HIP_OK(hipMemcpyAsync(sl.dev, sl.host, ch.used_bytes, hipMemcpyHostToDevice, st));
+        mutated.store(1);
+        HIP_OK(launch_place(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
+                            e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, e.opt.nan_bits, st));
+        HIP_OK(hipEventRecord(sl.done, st));
+        {
+          std::lock_guard<std::mutex> lk(sl.mu);
+          sl.submitted = turn + 1;
+        }
+        sl.cv.notify_all();
+      }
+    } catch (const Error& er) {
+      std::lock_guard<std::mutex> lk(err_mu);
+      if (!first_err) first_err = std::make_unique<Error>(er);
+      abort.store(true);
+      for (auto& s : e.slots) { { std::lock_guard<std::mutex> g(s->mu); } s->cv.notify_all(); }
+    } catch (const std::exception& ex) {
+      std::lock_guard<std::mutex> lk(err_mu);
+      if (!first_err) first_err = std::make_unique<Error>(MXP_ERR_STATE, ex.what());
+      abort.store(true);
+      for (auto& s : e.slots) { { std::lock_guard<std::mutex> g(s->mu); } s->cv.notify_all(); }
+    }
+  };
+  {
+    std::vector<std::thread> pool;
+    const int n_thr = (int)std::min<size_t>((size_t)e.opt.reader_threads, n_chunks ? n_chunks : 1);
+    for (int t = 0; t < n_thr; ++t) pool.emplace_back(worker, t);
+    for (auto& t : pool) t.join();
+  }
+  hipError_t sync_err = hipSuccess;
+  for (auto st : e.streams) {
+    const hipError_t r = hipStreamSynchronize(st);
+    if (r != hipSuccess) sync_err = r;
+  }
+  if (stats) {
+    stats->wall_seconds = now_s() - t_start;
+    for (double r : read_s) stats->read_seconds += r;
+    stats->file_bytes = L.file_bytes;
+    stats->h2d_bytes = L.h2d_bytes;
+    stats->placed_bytes = L.placed_bytes;
+    stats->n_chunks = n_chunks;
+    stats->n_segments = L.ing_n_segs;
+    stats->n_workgroups = L.ing_n_work;
+    stats->n_launches = n_chunks;
+    stats->mutated = mutated.load();
+  }
+  if (first_err) throw *first_err;
+  if (sync_err != hipSuccess) throw Error(MXP_ERR_DEVICE, std::string("stream synchronize: ") + hipGetErrorString(sync_err));
+}
+
+void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_dev_ptrs, void* const* dst_ptrs,
+                         hipStream_t stream, mxp_exec_stats* stats) {
+  HIP_OK(hipSetDevice(e.opt.device));
+  check_dst(pl, dst_ptrs);
+  if (!file_dev_ptrs) throw Error(MXP_ERR_ARG, "file_dev_ptrs is null");
+  const mxp_ckpt& ck = *pl.ckpt;
+  for (size_t f = 0; f < ck.files.size(); ++f)
+    if (!file_dev_ptrs[f] || (reinterpret_cast<uintptr_t>(file_dev_ptrs[f]) & 15u))
+      throw Error(MXP_ERR_ARG, "staged file pointer " + std::to_string(f) + " is null or not 16-byte aligned");
+  lower_plan(pl, e);
+  auto& L = *pl.lowered;
+  if (stats) std::memset(stats, 0, sizeof *stats);
+  // The pointer tables are small; plain synchronous copies keep them ordered before the launch.
+  upload_dst(L, pl, dst_ptrs);
+  if (L.src_host.size() != ck.files.size() || !std::equal(L.src_host.begin(), L.src_host.end(), file_dev_ptrs)) {
+    L.src_bases.upload(file_dev_ptrs, ck.files.size());
+    L.src_host.assign(file_dev_ptrs, file_dev_ptrs + ck.files.size());
+  }
+  HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, stream));
+  if (stats) HIP_OK(hipEventRecord(e.ev_a, stream));
+  HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
+                      e.opt.nan_bits, stream));
+  if (stats) {
+    HIP_OK(hipEventRecord(e.ev_b, stream));
+    HIP_OK(hipEventSynchronize(e.ev_b));
+    float ms = 0;
+    HIP_OK(hipEventElapsedTime(&ms, e.ev_a, e.ev_b));
+    stats->kernel_ms = ms;
+    stats->wall_seconds = ms * 1e-3;
+    stats->placed_bytes = L.placed_bytes;
+    stats->n_segments = L.res_n_segs;
+    stats->n_workgroups = L.res_n_work;
+    stats->n_launches = 1;
+    stats->mutated = 1;
+  }
+}
+
+}  // namespace
+}  // namespace mxp
+
+extern "C" {
+
+int mxp_execute(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs, mxp_exec_stats* stats) {
+  return guard([&] {
+    if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_execute: null handle");
+    do_execute(*engine, *plan, dst_ptrs, stats);
+  });
+}
+
+int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* file_dev_ptrs,
+                         void* const* dst_ptrs, void* stream, mxp_exec_stats* stats) {
+  return guard([&] {
+    if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_execute_resident: null handle");
+    do_execute_resident(*engine, *plan, file_dev_ptrs, dst_ptrs, static_cast<hipStream_t>(stream), stats);
+  });
+}
+
+int mxp_prepare(mxp_engine* engine, mxp_plan* plan) {
+  return guard([&] {
+    if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_prepare: null handle");
+    HIP_OK(hipSetDevice(engine->opt.device));
+    lower_plan(*plan, *engine);
+  });
+}
+
+int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_t n) {
+  return guard([&] {
+    if (!engine || !plan || !out) throw Error(MXP_ERR_ARG, "mxp_plan_checksums: null argument");
+    if (!plan->lowered) throw Error(MXP_ERR_STATE, "plan has not been executed");
+    if (n != (int64_t)plan->params.size()) throw Error(MXP_ERR_ARG, "mxp_plan_checksums: n must equal the parameter count");
+    HIP_OK(hipSetDevice(engine->opt.device));
+    HIP_OK(hipDeviceSynchronize());
+    if (n) HIP_OK(hipMemcpy(out, plan->lowered->sums.p, (size_t)n * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int mxp_plan_totals(const mxp_plan* plan, uint64_t* file_bytes, uint64_t* h2d_bytes, uint64_t* placed_bytes,
+                    uint64_t* kernel_algorithmic_bytes) {
+  return guard([&] {
+    if (!plan) throw Error(MXP_ERR_ARG, "mxp_plan_totals: null plan");
+    if (!plan->built) throw Error(MXP_ERR_STATE, "plan has not been built");
+    uint64_t placed = 0, algo = 0;
+    for (const auto& w : plan->writes) {
+      placed += w.rows * w.row_bytes;
+      algo += w.rows * w.row_bytes * (w.cast ? 3 : 2);
+    }
+    if (placed_bytes) *placed_bytes = placed;
+    if (kernel_algorithmic_bytes) *kernel_algorithmic_bytes = algo;
+    if (file_bytes) *file_bytes = plan->lowered ? plan->lowered->file_bytes : 0;
+    if (h2d_bytes) *h2d_bytes = plan->lowered ? plan->lowered->h2d_bytes : 0;
+  });
+}
+
+int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n, uint32_t* out,
+                   void* stream) {
+  return guard([&] {
+    if (!engine || !out || n < 0 || (n && (!ptrs || !nbytes))) throw Error(MXP_ERR_ARG, "mxp_checksum32: bad argument");
+    if (n == 0) return;
+    HIP_OK(hipSetDevice(engine->opt.device));
+    std::vector<BoxCopy> boxes;
+    std::vector<const void*> srcs;
+    for (int64_t k = 0; k < n; ++k) {
+      if (nbytes[k] && !ptrs[k]) throw Error(MXP_ERR_ARG, "mxp_checksum32: null pointer");
+      const void* base;
+      uint64_t off;
+      split_ptr(ptrs[k], base, off);
+      srcs.push_back(base);
+      // A misaligned start only narrows the access width the lowering picks.
+      BoxCopy b;
+      b.src_buf = (uint32_t)k;
+      b.src_off = off;
+      b.row_bytes = nbytes[k];
+      b.op = kOpChecksumOnly;
+      b.csum_slot = (uint32_t)k;
+      boxes.push_back(b);
+    }
+    run_boxes(*engine, boxes, srcs, {}, (uint32_t)n, out, static_cast<hipStream_t>(stream));
+  });
+}
+
+int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems, uint32_t* checksum,
+                      void* stream) {
+  return guard([&] {
+    if (!engine || (n_elems && (!src || !dst))) throw Error(MXP_ERR_ARG, "mxp_cast_f32_bf16: bad argument");
+    if (checksum) *checksum = 0;
+    if (n_elems == 0) return;
+    HIP_OK(hipSetDevice(engine->opt.device));
+    if ((reinterpret_cast<uintptr_t>(src) & 3u) || (reinterpret_cast<uintptr_t>(dst) & 1u))
+      throw Error(MXP_ERR_ARG, "mxp_cast_f32_bf16: pointers must be element aligned");
+    if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_cast_f32_bf16: dst must be 16-byte aligned");
+    const void* sb;
+    uint64_t so;
+    split_ptr(src, sb, so);
+    BoxCopy b;
+    b.src_off = so;
+    b.row_bytes = n_elems * 2;
+    b.op = kOpCastF32Bf16;
+    b.csum_slot = 0;
+    std::vector<BoxCopy> boxes{b};
+    uint32_t sum = 0;
+    run_boxes(*engine, boxes, {sb}, {dst}, 1, checksum ? &sum : nullptr,
+              static_cast<hipStream_t>(stream));
+    if (checksum) *checksum = sum;
+  });
+}
+
+int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* dst, uint64_t dst_pitch,
+                 uint64_t rows, uint64_t row_bytes, uint32_t* checksum, void* stream) {
+  return guard([&] {
+    if (!engine || (rows && row_bytes && (!src || !dst))) throw Error(MXP_ERR_ARG, "mxp_gather2d: bad argument");
+    if (checksum) *checksum = 0;
+    if (rows == 0 || row_bytes == 0) return;
+    if (rows > 1 && (src_pitch < row_bytes || dst_pitch < row_bytes))
+      throw Error(MXP_ERR_ARG, "mxp_gather2d: pitch smaller than row_bytes");
+    HIP_OK(hipSetDevice(engine->opt.device));
+    if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_gather2d: dst must be 16-byte aligned");
+    const void* sb;
+    uint64_t so;
+    split_ptr(src, sb, so);
+    BoxCopy b;
+    b.src_off = so;
+    b.src_pitch = src_pitch;
+    b.dst_pitch = dst_pitch;
+    b.rows = rows;
+    b.row_bytes = row_bytes;
+    b.op = kOpCopy;
+    b.csum_slot = 0;
+    uint32_t sum = 0;
+    run_boxes(*engine, {b}, {sb}, {dst}, 1, checksum ? &sum : nullptr, static_cast<hipStream_t>(stream));
+    if (checksum) *checksum = sum;
+  });
+}
+
+int mxp_digest_from_scalars(const uint64_t scalars[7], uint8_t out16[16]) {
+  return guard([&] {
+    if (!scalars || !out16) throw Error(MXP_ERR_ARG, "mxp_digest_from_scalars: null argument");
+    const uint64_t n = scalars[0];
+    const uint64_t body_words = n / 4, rows = body_words / kDigestRowWords;
+    std::vector<uint64_t> list{n};
+    if (rows) { list.push_back(scalars[1]); list.push_back(scalars[2]); }
+    if (body_words - rows * kDigestRowWords) { list.push_back(scalars[3]); list.push_back(scalars[4]); }
+    if (n % 4) { list.push_back(scalars[5]); list.push_back(n % 4); }
+    Blake2b h(16);
+    for (uint64_t v : list) {
+      uint8_t le[8];
+      for (int b = 0; b < 8; ++b) le[b] = (uint8_t)(v >> (8 * b));
+      h.update(le, 8);
+    }
+    h.final(out16);
+  });
+}
+
+int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n, uint8_t* out16,
+               uint64_t* scalars, void* stream_v) {
+  return guard([&] {
+    if (!engine || !out16 || n < 0 || (n && (!ptrs || !nbytes))) throw Error(MXP_ERR_ARG, "mxp_digest: bad argument");
+    if (n == 0) return;
+    mxp_engine& e = *engine;
+    HIP_OK(hipSetDevice(e.opt.device));
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    std::vector<DigestJob> jobs((size_t)n);
+    uint64_t blocks = 0;
+    for (int64_t k = 0; k < n; ++k) {
+      if (nbytes[k] && !ptrs[k]) throw Error(MXP_ERR_ARG, "mxp_digest: null pointer");
+      jobs[k].ptr = static_cast<const uint8_t*>(ptrs[k]);
+      jobs[k].nbytes = nbytes[k];
+      jobs[k].out_slot = (uint64_t)k * 5;
+      jobs[k].first_block = blocks;
+      const uint64_t rows = (nbytes[k] / 4) / kDigestRowWords;
+      blocks += rows ? (rows + kDigestRowsPerBlock - 1) / kDigestRowsPerBlock : 1;
+    }
+    if (blocks > 0x7FFFFFFFull) throw Error(MXP_ERR_ARG, "mxp_digest: batch too large for one launch");
+    const size_t o_jobs = 0;
+    const size_t o_out = align_up(jobs.size() * sizeof(DigestJob), 256);
+    const size_t total = o_out + (size_t)n * 5 * 8;
+    HIP_OK(hipStreamSynchronize(stream));
+    ensure_desc(e, total);
+    std::memset(e.desc_host, 0, total);
+    std::memcpy(e.desc_host + o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
+    HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, total, hipMemcpyHostToDevice, stream));
+    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(e.desc_dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks,
+                         reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_out), stream));
+    HIP_OK(hipMemcpyAsync(e.desc_host + o_out, e.desc_dev.p + o_out, (size_t)n * 5 * 8, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    const uint64_t* sums = reinterpret_cast<const uint64_t*>(e.desc_host + o_out);
+    for (int64_t k = 0; k < n; ++k) {
+      uint64_t sc[7] = {nbytes[k], sums[5 * k], sums[5 * k + 1], sums[5 * k + 2], sums[5 * k + 3], sums[5 * k + 4],
+                        nbytes[k] % 4};
+      if (scalars) std::memcpy(scalars + 7 * k, sc, sizeof sc);
+      Blake2b h(16);
+      const uint64_t body_words = nbytes[k] / 4, rows = body_words / kDigestRowWords;
+      std::vector<uint64_t> list{sc[0]};
+      if (rows) { list.push_back(sc[1]); list.push_back(sc[2]); }
+      if (body_words - rows * kDigestRowWords) { list.push_back(sc[3]); list.push_back(sc[4]); }
+      if (nbytes[k] % 4) { list.push_back(sc[5]); list.push_back(sc[6]); }
+      for (uint64_t v : list) {
+        uint8_t le[8];
+        for (int b = 0; b < 8; ++b) le[b] = (uint8_t)(v >> (8 * b));
+        h.update(le, 8);
+      }
+      h.final(out16 + 16 * k);
+    }
+  });
+}
+
+int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double* bytes_per_second) {
+  return guard([&] {
+    if (!engine || !bytes_per_second || bytes == 0) throw Error(MXP_ERR_ARG, "mxp_measure_h2d: bad argument");
+    mxp_engine& e = *engine;
+    HIP_OK(hipSetDevice(e.opt.device));
+    if (repeats < 1) repeats = 1;
+    void* h = nullptr;
+    void* d = nullptr;
+    HIP_OK(hipHostMalloc(&h, bytes, hipHostMallocDefault));
+    if (hipMalloc(&d, bytes) != hipSuccess) {
+      (void)hipHostFree(h);
+      throw Error(MXP_ERR_DEVICE, "mxp_measure_h2d: device allocation failed");
+    }
+    std::memset(h, 0x5a, bytes);
+    float best = 1e30f;
+    hipError_t err = hipSuccess;
+    for (int r = 0; r < repeats + 1 && err == hipSuccess; ++r) {
+      err = hipEventRecord(e.ev_a, e.streams[0]);
+      if (err == hipSuccess) err = hipMemcpyAsync(d, h, bytes, hipMemcpyHostToDevice, e.streams[0]);
+      if (err == hipSuccess) err = hipEventRecord(e.ev_b, e.streams[0]);
+      if (err == hipSuccess) err = hipEventSynchronize(e.ev_b);
+      float ms = 0;
+      if (err == hipSuccess) err = hipEventElapsedTime(&ms, e.ev_a, e.ev_b);
+      if (r > 0 && ms < best) best = ms;  // first pass warms the path
+    }
+    (void)hipFree(d);
+    (void)hipHostFree(h);
+    if (err != hipSuccess) throw Error(MXP_ERR_DEVICE, std::string("mxp_measure_h2d: ") + hipGetErrorString(err));
+    *bytes_per_second = (double)bytes / ((double)best * 1e-3);
+  });
+}
+
+int mxp_synth_host(void* dst, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed, int32_t threads) {
+  return guard([&] {
+    if (n_elems && !dst) throw Error(MXP_ERR_ARG, "mxp_synth_host: null dst");
+    if (!dtype_size(dtype)) throw Error(MXP_ERR_UNSUPPORTED, "unknown dtype code");
+    synth_host(dst, n_elems, (uint32_t)dtype, kind, seed, threads);
+  });
+}
+
+int mxp_synth_device(void* dst_dev, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed, void* stream) {
+  return guard([&] {
+    if (n_elems && !dst_dev) throw Error(MXP_ERR_ARG, "mxp_synth_device: null dst");
+    if (!dtype_size(dtype)) throw Error(MXP_ERR_UNSUPPORTED, "unknown dtype code");
+    HIP_OK(launch_synth(dst_dev, n_elems, (uint32_t)dtype, kind, seed, static_cast<hipStream_t>(stream)));
+  });
+}
+
+}  // extern "C"

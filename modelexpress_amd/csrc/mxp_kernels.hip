@@ -1,0 +1,335 @@
+// CDNA4 (gfx950) kernels for the weight-placement path.
+//
+// All of them are HBM-bound byte movers or reducers; none is a contraction, so there
+// is no MFMA here.  What matters is: 128-bit accesses that are contiguous across the
+// 64 lanes of a wavefront, thousands of workgroups per launch (256 CUs in 8 XCDs),
+// and one launch for a whole batch of tensors instead of one launch per tensor.
+//
+//  place_kernel   pitched box copy / fp32->bf16 cast with the position-weighted
+//                 checksum of every byte written fused in (reads each output byte's
+//                 source once, writes it once: 2 x output bytes of traffic for a
+//                 copy, 6 bytes per element for the cast)
+//  digest_kernel  int32-word row sums for the blake2b-hashed tensor digest
+//                 (reads each byte once)
+#include "mxp_device.h"
+
+namespace mxp {
+
+// ---------------------------------------------------------------------------
+// Checksum algebra.  The per-tensor fingerprint is
+//     sum_i  byte[i] * ((i * 2654435761 + 1) mod 2^32)   mod 2^32
+// (reference: modelexpress/tensor_utils.py:27-44).  For a group of bytes starting at
+// position i with local offsets j:
+//     sum_j b_j * ((i + j) K + 1) = K * (i * S0 + S1) + S0,   S0 = sum b_j, S1 = sum j b_j
+// so three wrapping 32-bit accumulators P = sum i*S0, R = sum S1, Q = sum S0 are kept
+// per lane and folded once at the end as K * (P + R) + Q.  S0 and S1 come from the
+// unsigned 8-bit dot-product instruction, four bytes at a time.
+// ---------------------------------------------------------------------------
+struct Csum {
+  uint32_t P = 0, Q = 0, R = 0;
+  __device__ __forceinline__ void add16(const uint4& x, uint32_t i) {
+    uint32_t s0 = __builtin_amdgcn_udot4(x.x, 0x01010101u, 0u, false);
+    s0 = __builtin_amdgcn_udot4(x.y, 0x01010101u, s0, false);
+    s0 = __builtin_amdgcn_udot4(x.z, 0x01010101u, s0, false);
+    s0 = __builtin_amdgcn_udot4(x.w, 0x01010101u, s0, false);
+    R = __builtin_amdgcn_udot4(x.x, 0x03020100u, R, false);
+    R = __builtin_amdgcn_udot4(x.y, 0x07060504u, R, false);
+    R = __builtin_amdgcn_udot4(x.z, 0x0b0a0908u, R, false);
+    R = __builtin_amdgcn_udot4(x.w, 0x0f0e0d0cu, R, false);
+    Q += s0;
+    P += i * s0;
+  }
+  // Up to four bytes packed little-endian in x (missing bytes zero).
+  __device__ __forceinline__ void add4(uint32_t x, uint32_t i) {
+    uint32_t s0 = __builtin_amdgcn_udot4(x, 0x01010101u, 0u, false);
+    R = __builtin_amdgcn_udot4(x, 0x03020100u, R, false);
+    Q += s0;
+    P += i * s0;
+  }
+  __device__ __forceinline__ uint32_t fold() const { return kKnuth * (P + R) + Q; }
+};
+
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
+  return v;
+}
+
+__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
+  return v;
+}
+
+// fp32 bits -> bf16 bits, round to nearest even; every NaN becomes `nan_bits`.
+// Reference arithmetic: torch `copy_` at modelexpress_rl/train/engines/fsdp/adapter.py:203-206
+// and refit/reshard/receiver.py:964-971.
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(uint32_t u, uint32_t nan_bits) {
+  const uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? nan_bits : r;
+}
+
+__device__ __forceinline__ uint4 cast8(const uint4& a, const uint4& b, uint32_t nan_bits) {
+  uint4 o;
+  o.x = f32_to_bf16_bits(a.x, nan_bits) | (f32_to_bf16_bits(a.y, nan_bits) << 16);
+  o.y = f32_to_bf16_bits(a.z, nan_bits) | (f32_to_bf16_bits(a.w, nan_bits) << 16);
+  o.z = f32_to_bf16_bits(b.x, nan_bits) | (f32_to_bf16_bits(b.y, nan_bits) << 16);
+  o.w = f32_to_bf16_bits(b.z, nan_bits) | (f32_to_bf16_bits(b.w, nan_bits) << 16);
+  return o;
+}
+
+// One tile of one segment.  UNIT = destination bytes handled per lane access.
+// Lanes walk the tile in flattened (row, unit) order, so neighbouring lanes touch
+// neighbouring 16-byte units of the same row: every wavefront access is a run of
+// contiguous 1 KiB pieces in both the source and the destination.
+template <int OP, int UNIT>
+__device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict__ src,
+                                         uint8_t* __restrict__ dst, uint32_t csum_base,
+                                         uint32_t n_units, uint32_t nan_bits, Csum& cs) {
+  constexpr int SRC_UNIT = (OP == kOpCastF32Bf16) ? 2 * UNIT : UNIT;
+  const uint32_t upr = s.units_per_row;
+  const uint32_t magic = s.div_magic;
+  const uint32_t sp = (uint32_t)s.src_pitch, dp = (uint32_t)s.dst_pitch;
+  // Within a tile the row offsets fit 32 bits (the planner bounds rows_per_tile * pitch).
+  auto locate = [&](uint32_t v, uint32_t& so, uint32_t& d_o) {
+    const uint32_t row = (upr == 1u) ? v : __umulhi(v, magic);
+    const uint32_t col = v - row * upr;
+    so = row * sp + col * (uint32_t)SRC_UNIT;
+    d_o = row * dp + col * (uint32_t)UNIT;
+  };
+
+  if constexpr (UNIT == 16) {
+    uint32_t v = threadIdx.x;
+    // Four independent 16-byte units in flight per lane before the first store.
+    for (; v + 3u * kPlaceThreads < n_units; v += 4u * kPlaceThreads) {
+      uint32_t so[4], d_o[4];
+      uint4 x[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) locate(v + k * kPlaceThreads, so[k], d_o[k]);
+      if constexpr (OP == kOpCastF32Bf16) {
+        uint4 a[4], b[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          a[k] = *reinterpret_cast<const uint4*>(src + so[k]);
+          b[k] = *reinterpret_cast<const uint4*>(src + so[k] + 16);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) x[k] = cast8(a[k], b[k], nan_bits);
+      } else {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) x[k] = *reinterpret_cast<const uint4*>(src + so[k]);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        if constexpr (OP != kOpChecksumOnly) *reinterpret_cast<uint4*>(dst + d_o[k]) = x[k];
+        cs.add16(x[k], csum_base + d_o[k]);
+      }
+    }
+    for (; v < n_units; v += kPlaceThreads) {
+      uint32_t so, d_o;
+      locate(v, so, d_o);
+      uint4 x;
+      if constexpr (OP == kOpCastF32Bf16) {
+        const uint4 a = *reinterpret_cast<const uint4*>(src + so);
+        const uint4 b = *reinterpret_cast<const uint4*>(src + so + 16);
+        x = cast8(a, b, nan_bits);
+      } else {
+        x = *reinterpret_cast<const uint4*>(src + so);
+      }
+      if constexpr (OP != kOpChecksumOnly) *reinterpret_cast<uint4*>(dst + d_o) = x;
+      cs.add16(x, csum_base + d_o);
+    }
+  } else {
+    for (uint32_t v = threadIdx.x; v < n_units; v += kPlaceThreads) {
+      uint32_t so, d_o;
+      locate(v, so, d_o);
+      uint32_t x;
+      if constexpr (OP == kOpCastF32Bf16) {
+        static_assert(UNIT == 2 || UNIT == 16, "cast moves one or eight elements per lane");
+        x = f32_to_bf16_bits(*reinterpret_cast<const uint32_t*>(src + so), nan_bits);
+        *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+      } else if constexpr (UNIT == 4) {
+        x = *reinterpret_cast<const uint32_t*>(src + so);
+        if constexpr (OP != kOpChecksumOnly) *reinterpret_cast<uint32_t*>(dst + d_o) = x;
+      } else {
+        x = src[so];
+        if constexpr (OP != kOpChecksumOnly) dst[d_o] = (uint8_t)x;
+      }
+      cs.add4(x, csum_base + d_o);
+    }
+  }
+}
+
+__global__ __launch_bounds__(kPlaceThreads) void place_kernel(
+    const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
+    const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
+    uint32_t* __restrict__ sums, uint32_t nan_bits) {
+  const WorkItem w = work[blockIdx.x];
+  const Seg s = segs[w.seg];
+  const uint32_t r0 = w.tile * s.rows_per_tile;
+  const uint32_t nrows = min(s.rows - r0, s.rows_per_tile);
+  const uint32_t n_units = nrows * s.units_per_row;
+  const uint8_t* src =
+      static_cast<const uint8_t*>(src_bases[s.src_buf]) + s.src_off + (uint64_t)r0 * s.src_pitch;
+  uint8_t* dst = nullptr;
+  if (s.op != kOpChecksumOnly)
+    dst = static_cast<uint8_t*>(dst_bases[s.dst_buf]) + s.dst_off + (uint64_t)r0 * s.dst_pitch;
+  // Checksum positions are taken mod 2^32, exactly as the weights are.
+  const uint32_t csum_base = (uint32_t)(s.dst_off + (uint64_t)r0 * s.dst_pitch);
+
+  Csum cs;
+  switch (s.op * 32u + s.unit) {
+    case kOpCopy * 32u + 16u: run_tile<kOpCopy, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCopy * 32u + 4u: run_tile<kOpCopy, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCopy * 32u + 1u: run_tile<kOpCopy, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF32Bf16 * 32u + 16u: run_tile<kOpCastF32Bf16, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF32Bf16 * 32u + 2u: run_tile<kOpCastF32Bf16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpChecksumOnly * 32u + 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpChecksumOnly * 32u + 4u: run_tile<kOpChecksumOnly, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpChecksumOnly * 32u + 1u: run_tile<kOpChecksumOnly, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    default: break;  // the host validates (op, unit) before upload
+  }
+
+  if (s.csum_slot != 0xFFFFFFFFu) {
+    __shared__ uint32_t part[kPlaceThreads / 64];
+    const uint32_t wsum = wave_sum_u32(cs.fold());
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = wsum;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t t = 0;
+#pragma unroll
+      for (int k = 0; k < kPlaceThreads / 64; ++k) t += part[k];
+      atomicAdd(&sums[s.csum_slot], t);
+    }
+  }
+}
+
+hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
+                        const void* const* src_bases_dev, void* const* dst_bases_dev,
+                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream) {
+  if (n_work == 0) return hipSuccess;
+  hipLaunchKernelGGL(place_kernel, dim3(n_work), dim3(kPlaceThreads), 0, stream, segs_dev,
+                     work_dev, src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits);
+  return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// tensor_digest row sums (reference: modelexpress/refit/reshard/verify.py:112-150).
+// Bytes are read as little-endian signed int32 words; whole 1024-word rows give
+// sum_r rs[r] and sum_r rs[r]*(r+1); the words after the last whole row give
+// sum_k t[k] and sum_k t[k]*(k+1); the 1..3 bytes after the last whole word are summed
+// unsigned.  All sums wrap mod 2^64.  The index weight is applied per lane before any
+// reduction (sum_r (sum_lane p)*(r+1) == sum_lane sum_r p*(r+1)), so there is a single
+// reduction per workgroup.
+// ---------------------------------------------------------------------------
+template <bool ALIGNED16>
+__device__ __forceinline__ void digest_rows(const uint8_t* __restrict__ p, uint64_t row_begin,
+                                            uint64_t row_end, unsigned long long& A,
+                                            unsigned long long& B) {
+  const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (uint64_t r = row_begin + wave; r < row_end; r += kPlaceThreads / 64) {
+    const uint8_t* row = p + r * (uint64_t)(kDigestRowWords * 4);
+    long long acc = 0;
+    if constexpr (ALIGNED16) {
+      const uint4* v = reinterpret_cast<const uint4*>(row);
+      uint4 x[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) x[k] = v[lane + 64 * k];
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        acc += (long long)(int32_t)x[k].x + (long long)(int32_t)x[k].y +
+               (long long)(int32_t)x[k].z + (long long)(int32_t)x[k].w;
+    } else {
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const uint8_t* b = row + 4u * (lane + 64u * k);
+        const uint32_t u = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) |
+                           ((uint32_t)b[3] << 24);
+        acc += (long long)(int32_t)u;
+      }
+    }
+    A += (unsigned long long)acc;
+    B += (unsigned long long)acc * (unsigned long long)(r + 1);
+  }
+}
+
+__global__ __launch_bounds__(kPlaceThreads) void digest_kernel(
+    const DigestJob* __restrict__ jobs, uint32_t n_jobs, unsigned long long* __restrict__ out) {
+  // Workgroup-uniform binary search for the job that owns this workgroup.
+  uint32_t lo = 0, hi = n_jobs;
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (jobs[mid].first_block <= blockIdx.x) lo = mid; else hi = mid;
+  }
+  const DigestJob j = jobs[lo];
+  const uint64_t blk = blockIdx.x - j.first_block;
+  const uint64_t body_words = j.nbytes >> 2;
+  const uint64_t rows = body_words / kDigestRowWords;
+  const uint64_t n_blocks = rows ? (rows + kDigestRowsPerBlock - 1) / kDigestRowsPerBlock : 1;
+  const uint64_t row_begin = blk * kDigestRowsPerBlock;
+  const uint64_t row_end = min(rows, row_begin + kDigestRowsPerBlock);
+
+  unsigned long long A = 0, B = 0, At = 0, Bt = 0, Rg = 0;
+  if (row_begin < row_end) {
+    if ((reinterpret_cast<uintptr_t>(j.ptr) & 15u) == 0)
+      digest_rows<true>(j.ptr, row_begin, row_end, A, B);
+    else
+      digest_rows<false>(j.ptr, row_begin, row_end, A, B);
+  }
+  if (blk == n_blocks - 1) {
+    const uint8_t* tail = j.ptr + rows * (uint64_t)(kDigestRowWords * 4);
+    const uint32_t tw = (uint32_t)(body_words - rows * kDigestRowWords);
+    for (uint32_t k = threadIdx.x; k < tw; k += kPlaceThreads) {
+      const uint8_t* b = tail + 4u * k;
+      const uint32_t u = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) |
+                         ((uint32_t)b[3] << 24);
+      const long long w = (long long)(int32_t)u;
+      At += (unsigned long long)w;
+      Bt += (unsigned long long)w * (unsigned long long)(k + 1);
+    }
+    if (threadIdx.x == 0) {
+      const uint32_t rag = (uint32_t)(j.nbytes & 3u);
+      for (uint32_t k = 0; k < rag; ++k) Rg += j.ptr[body_words * 4 + k];
+    }
+  }
+
+  __shared__ unsigned long long part[kPlaceThreads / 64][5];
+  unsigned long long v[5] = {A, B, At, Bt, Rg};
+#pragma unroll
+  for (int q = 0; q < 5; ++q) {
+    const unsigned long long wsum = wave_sum_u64(v[q]);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6][q] = wsum;
+  }
+  __syncthreads();
+  if (threadIdx.x < 5) {
+    unsigned long long t = 0;
+#pragma unroll
+    for (int k = 0; k < kPlaceThreads / 64; ++k) t += part[k][threadIdx.x];
+    if (t) atomicAdd(&out[j.out_slot + threadIdx.x], t);
+  }
+}
+
+hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
+                         unsigned long long* out_dev, hipStream_t stream) {
+  if (n_jobs == 0 || n_blocks == 0) return hipSuccess;
+  hipLaunchKernelGGL(digest_kernel, dim3(n_blocks), dim3(kPlaceThreads), 0, stream, jobs_dev,
+                     n_jobs, out_dev);
+  return hipGetLastError();
+}
+
+// Plain vector-store fill; used instead of a memset node so callers may capture it.
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, uint64_t n,
+                                                       uint32_t value) {
+  for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < n; i += (uint64_t)gridDim.x * 256ull)
+    p[i] = value;
+}
+
+hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  const uint64_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((uint32_t)(blocks > 4096 ? 4096 : blocks)), dim3(256), 0,
+                     stream, ptr, n, value);
+  return hipGetLastError();
+}
+
+}  // namespace mxp

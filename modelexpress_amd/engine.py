@@ -1,0 +1,313 @@
+"""Python handles over the C ABI: Checkpoint, PlacementPlan, PlacementEngine.
+
+PyTorch appears here only as the owner of device memory and streams: destination
+parameters are torch tensors whose ``data_ptr()`` is handed to the library, and all
+arithmetic happens in libmxplace.so.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import Iterable, Sequence
+
+from . import _lib as L
+
+
+@dataclass(frozen=True)
+class TensorEntry:
+    name: str
+    dtype: str
+    shape: tuple
+    file_index: int
+    file_offset: int
+    nbytes: int
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One parameter of the serving rank: what the engine allocated for it."""
+
+    name: str
+    dtype: str
+    shape: tuple
+
+    @property
+    def nbytes(self) -> int:
+        n = L.DTYPE_SIZE[self.dtype]
+        for d in self.shape:
+            n *= int(d)
+        return n
+
+
+@dataclass(frozen=True)
+class WriteEntry:
+    tensor: str
+    param: str
+    kind: str
+    cast: bool
+    src_offset: int
+    src_pitch: int
+    dst_offset: int
+    dst_pitch: int
+    rows: int
+    row_bytes: int
+    paired_runs: int
+
+
+class Checkpoint:
+    """A parsed safetensors checkpoint (directory or single file)."""
+
+    def __init__(self, model_path: str):
+        self._h = C.c_void_p()
+        L.check(L.lib().mxp_ckpt_open(str(model_path).encode(), C.byref(self._h)))
+        self.path = str(model_path)
+
+    def close(self) -> None:
+        if self._h:
+            L.lib().mxp_ckpt_close(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # noqa: BLE001 - interpreter shutdown
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __len__(self) -> int:
+        return int(L.lib().mxp_ckpt_tensor_count(self._h))
+
+    def tensors(self) -> list[TensorEntry]:
+        out = []
+        info = L.TensorInfo()
+        for i in range(len(self)):
+            L.check(L.lib().mxp_ckpt_tensor_info(self._h, i, C.byref(info)))
+            out.append(TensorEntry(info.name.decode(), L.DTYPES[info.dtype], tuple(info.shape[: info.ndim]),
+                                   info.file_index, info.file_offset, info.nbytes))
+        return out
+
+    def files(self) -> list[dict]:
+        out = []
+        info = L.FileInfo()
+        for i in range(int(L.lib().mxp_ckpt_file_count(self._h))):
+            L.check(L.lib().mxp_ckpt_file_info(self._h, i, C.byref(info)))
+            out.append({"path": info.path.decode(), "file_size": info.file_size, "data_start": info.data_start,
+                        "n_tensors": info.n_tensors})
+        return out
+
+    def find(self, name: str) -> int:
+        return int(L.lib().mxp_ckpt_find(self._h, name.encode()))
+
+
+class PlacementPlan:
+    """Destination map of one rank, built from the rank's parameter table.
+
+    ``stacked_params_mapping`` is a list of ``(fused_suffix, member_suffix)`` pairs in
+    pack order (None = built-in qkv / gate_up groups); ``expert_mapping`` rows are
+    ``(param_prefix, weight_prefix, expert_id, shard[, local_id])`` where a missing
+    ``local_id`` means the global id, -1 means "not on this rank", -2 "unknown".
+    """
+
+    def __init__(self, ckpt: Checkpoint, params: Iterable[ParamSpec], *, tp_size: int = 1, tp_rank: int = 0,
+                 stacked_params_mapping: Sequence | None = None, expert_mapping: Sequence | None = None,
+                 skip_prefixes: Sequence[str] = (), allow_cast: bool = False, allow_unmapped: bool = False,
+                 allow_uncovered: bool = False, fp8_block_check: bool = True):
+        lib = L.lib()
+        self.ckpt = ckpt
+        flags = 0
+        flags |= L.PLAN_ALLOW_CAST_F32_BF16 if allow_cast else 0
+        flags |= L.PLAN_ALLOW_UNMAPPED if allow_unmapped else 0
+        flags |= L.PLAN_ALLOW_UNCOVERED if allow_uncovered else 0
+        flags |= 0 if fp8_block_check else L.PLAN_NO_FP8_BLOCK_CHECK
+        self._h = C.c_void_p()
+        L.check(lib.mxp_plan_create(ckpt._h, tp_size, tp_rank, flags, C.byref(self._h)))
+        self.tp_size, self.tp_rank = tp_size, tp_rank
+        self.params = list(params)
+        for p in self.params:
+            shape = (C.c_int64 * max(1, len(p.shape)))(*[int(d) for d in p.shape])
+            L.check(lib.mxp_plan_add_param(self._h, p.name.encode(), L.DTYPE_CODE[p.dtype], len(p.shape), shape))
+        for fused, member in stacked_params_mapping or ():
+            L.check(lib.mxp_plan_add_stacked(self._h, str(fused).encode(), str(member).encode()))
+        for row in expert_mapping or ():
+            p_pre, w_pre, eid, shard = row[:4]
+            local = int(row[4]) if len(row) > 4 else int(eid)
+            L.check(lib.mxp_plan_add_expert(self._h, p_pre.encode(), w_pre.encode(), int(eid), shard.encode(), local))
+        for pre in skip_prefixes:
+            L.check(lib.mxp_plan_add_skip_prefix(self._h, pre.encode()))
+        L.check(lib.mxp_plan_build(self._h))
+
+    def close(self) -> None:
+        if self._h:
+            L.lib().mxp_plan_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # noqa: BLE001
+            pass
+
+    def writes(self) -> list[WriteEntry]:
+        lib = L.lib()
+        tensors = self.ckpt.tensors()
+        out = []
+        info = L.WriteInfo()
+        for i in range(int(lib.mxp_plan_write_count(self._h))):
+            L.check(lib.mxp_plan_write_info(self._h, i, C.byref(info)))
+            out.append(WriteEntry(tensors[info.tensor_index].name, self.params[info.param_index].name,
+                                  L.WRITE_KINDS[info.kind], bool(info.cast), info.src_offset, info.src_pitch,
+                                  info.dst_offset, info.dst_pitch, info.rows, info.row_bytes, info.paired_runs))
+        return out
+
+    def param_info(self) -> list[dict]:
+        lib = L.lib()
+        out = []
+        info = L.ParamInfo()
+        for i in range(int(lib.mxp_plan_param_count(self._h))):
+            L.check(lib.mxp_plan_param_info(self._h, i, C.byref(info)))
+            out.append({"name": info.name.decode(), "dtype": L.DTYPES[info.dtype],
+                        "shape": tuple(info.shape[: info.ndim]), "nbytes": info.nbytes,
+                        "bytes_written": info.bytes_written, "n_writes": info.n_writes})
+        return out
+
+    def totals(self) -> dict:
+        vals = [C.c_uint64() for _ in range(4)]
+        L.check(L.lib().mxp_plan_totals(self._h, *[C.byref(v) for v in vals]))
+        keys = ("file_bytes", "h2d_bytes", "placed_bytes", "kernel_algorithmic_bytes")
+        return {k: int(v.value) for k, v in zip(keys, vals)}
+
+
+def _ptr_array(ptrs: Sequence[int]):
+    return (C.c_void_p * max(1, len(ptrs)))(*[C.c_void_p(int(p)) for p in ptrs])
+
+
+class PlacementEngine:
+    """Device-side executor: pinned ring + streams + kernels of one GPU."""
+
+    def __init__(self, device: int = 0, *, ring_slots: int = 0, slot_bytes: int = 0, reader_threads: int = 0,
+                 streams: int = 0, tile_bytes: int = 0, nan_bits: int = 0, use_o_direct: bool = False):
+        opts = L.EngineOptions(device=device, ring_slots=ring_slots, slot_bytes=slot_bytes,
+                               reader_threads=reader_threads, streams=streams, tile_bytes=tile_bytes,
+                               nan_bits=nan_bits, use_o_direct=int(use_o_direct))
+        self._h = C.c_void_p()
+        L.check(L.lib().mxp_engine_create(C.byref(opts), C.byref(self._h)))
+        self.device = device
+
+    def close(self) -> None:
+        if self._h:
+            L.lib().mxp_engine_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # noqa: BLE001
+            pass
+
+    # ---- buffers ----
+    def allocate(self, plan: PlacementPlan, fill: int | None = None) -> list:
+        """One uint8 torch tensor per parameter of ``plan`` on this engine's device."""
+        import torch
+
+        dev = torch.device("cuda", self.device)
+        out = []
+        for p in plan.params:
+            n = max(p.nbytes, 1)
+            t = torch.empty(n, dtype=torch.uint8, device=dev) if fill is None else torch.full(
+                (n,), fill, dtype=torch.uint8, device=dev)
+            out.append(t[: p.nbytes] if p.nbytes != n else t)
+        return out
+
+    # ---- placement ----
+    def prepare(self, plan: PlacementPlan) -> None:
+        L.check(L.lib().mxp_prepare(self._h, plan._h))
+
+    def execute(self, plan: PlacementPlan, dst: Sequence) -> dict:
+        """Ingest from storage into ``dst`` (torch tensors or raw device addresses)."""
+        ptrs = _ptr_array([_addr(t) for t in dst])
+        stats = L.ExecStats()
+        rc = L.lib().mxp_execute(self._h, plan._h, ptrs, C.byref(stats))
+        if rc < 0:
+            err = L.MxpError(int(rc), L.lib().mxp_last_error().decode("utf-8", "replace"))
+            err.mutated = bool(stats.mutated)
+            raise err
+        return stats.as_dict()
+
+    def execute_resident(self, plan: PlacementPlan, staged_files: Sequence, dst: Sequence, *, stream: int = 0,
+                         timed: bool = False) -> dict | None:
+        """Placement from shard files already staged in HBM; one launch."""
+        fptrs = _ptr_array([_addr(t) for t in staged_files])
+        dptrs = _ptr_array([_addr(t) for t in dst])
+        stats = L.ExecStats() if timed else None
+        L.check(L.lib().mxp_execute_resident(self._h, plan._h, fptrs, dptrs, C.c_void_p(stream),
+                                             C.byref(stats) if timed else None))
+        return stats.as_dict() if timed else None
+
+    def checksums(self, plan: PlacementPlan) -> list[str]:
+        n = len(plan.params)
+        out = (C.c_uint32 * max(1, n))()
+        L.check(L.lib().mxp_plan_checksums(self._h, plan._h, out, n))
+        return [format(out[i], "08x") for i in range(n)]
+
+    # ---- stand-alone operators ----
+    def checksum32(self, buffers: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0) -> list[str]:
+        n = len(buffers)
+        sizes = [_nbytes(t) for t in buffers] if nbytes is None else list(nbytes)
+        out = (C.c_uint32 * max(1, n))()
+        L.check(L.lib().mxp_checksum32(self._h, _ptr_array([_addr(t) for t in buffers]),
+                                       (C.c_uint64 * max(1, n))(*sizes), n, out, C.c_void_p(stream)))
+        return [format(out[i], "08x") for i in range(n)]
+
+    def digest(self, buffers: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
+               with_scalars: bool = False):
+        n = len(buffers)
+        sizes = [_nbytes(t) for t in buffers] if nbytes is None else list(nbytes)
+        out = (C.c_uint8 * (16 * max(1, n)))()
+        sc = (C.c_uint64 * (7 * max(1, n)))()
+        L.check(L.lib().mxp_digest(self._h, _ptr_array([_addr(t) for t in buffers]),
+                                   (C.c_uint64 * max(1, n))(*sizes), n, out, sc, C.c_void_p(stream)))
+        hexes = [bytes(out[16 * i: 16 * i + 16]).hex() for i in range(n)]
+        if with_scalars:
+            return hexes, [[int(sc[7 * i + k]) for k in range(7)] for i in range(n)]
+        return hexes
+
+    def cast_f32_bf16(self, src, dst, n_elems: int, *, stream: int = 0, checksum: bool = True) -> str | None:
+        out = C.c_uint32()
+        L.check(L.lib().mxp_cast_f32_bf16(self._h, C.c_void_p(_addr(src)), C.c_void_p(_addr(dst)), n_elems,
+                                          C.byref(out) if checksum else None, C.c_void_p(stream)))
+        return format(out.value, "08x") if checksum else None
+
+    def gather2d(self, src, src_pitch: int, dst, dst_pitch: int, rows: int, row_bytes: int, *, stream: int = 0,
+                 checksum: bool = True) -> str | None:
+        out = C.c_uint32()
+        L.check(L.lib().mxp_gather2d(self._h, C.c_void_p(_addr(src)), src_pitch, C.c_void_p(_addr(dst)), dst_pitch,
+                                     rows, row_bytes, C.byref(out) if checksum else None, C.c_void_p(stream)))
+        return format(out.value, "08x") if checksum else None
+
+    def measure_h2d(self, nbytes: int = 256 << 20, repeats: int = 5) -> float:
+        out = C.c_double()
+        L.check(L.lib().mxp_measure_h2d(self._h, nbytes, repeats, C.byref(out)))
+        return float(out.value)
+
+
+def digest_from_scalars(scalars: Sequence[int]) -> str:
+    sc = (C.c_uint64 * 7)(*[int(v) & ((1 << 64) - 1) for v in scalars])
+    out = (C.c_uint8 * 16)()
+    L.check(L.lib().mxp_digest_from_scalars(sc, out))
+    return bytes(out).hex()
+
+
+def _addr(t) -> int:
+    if isinstance(t, int):
+        return t
+    return int(t.data_ptr())
+
+
+def _nbytes(t) -> int:
+    return int(t.numel() * t.element_size())

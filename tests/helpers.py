@@ -1,0 +1,79 @@
+"""Shared test helpers: run the CPU oracle over a checkpoint, interpret a product plan
+with numpy, build tiny layouts of the benchmark families."""
+
+from __future__ import annotations
+
+import numpy as np
+
+from modelexpress_amd import models
+from modelexpress_amd.engine import Checkpoint, PlacementPlan
+
+
+def oracle_place(oracle, ckpt_dir: str, rv, *, tp_size=1, tp_rank=0, allow_cast=False, nan_bits=0x7FC0,
+                 strict_params=True):
+    """The oracle's parameter buffers for one rank: ``{name: OTensor}``."""
+    weights = oracle.load_checkpoint(ckpt_dir)
+    params = {p.name: oracle.OTensor.zeros(p.shape, p.dtype) for p in rv.params}
+    skip = tuple(rv.skip_prefixes)
+    weights = [(n, t) for n, t in weights if not n.startswith(skip)] if skip else weights
+    local_of = {}
+    mapping = None
+    if rv.expert_mapping:
+        mapping = [row[:4] for row in rv.expert_mapping]
+        for row in rv.expert_mapping:
+            local_of[int(row[2])] = int(row[4]) if len(row) > 4 else int(row[2])
+
+    def expert_local(_fused_name, gid):
+        loc = local_of.get(gid, gid)
+        return None if loc == -2 else loc
+
+    m = oracle.MdlOracle(params, tp_size, tp_rank, rv.stacked_params_mapping, mapping,
+                         expert_local if mapping else None, allow_cast=allow_cast, nan_bits=nan_bits)
+    m.load_weights(weights, strict_params=strict_params)
+    return params
+
+
+def make_plan(ckpt_dir: str, rv, *, tp_size=1, tp_rank=0, **kw):
+    ck = Checkpoint(ckpt_dir)
+    plan = PlacementPlan(ck, rv.params, tp_size=tp_size, tp_rank=tp_rank,
+                         stacked_params_mapping=rv.stacked_params_mapping, expert_mapping=rv.expert_mapping,
+                         skip_prefixes=rv.skip_prefixes, **kw)
+    return ck, plan
+
+
+def apply_plan_numpy(ck: Checkpoint, plan: PlacementPlan, nan_bits=0x7FC0) -> dict:
+    """Interpret the product plan's pitched boxes on the host (checks the planner alone)."""
+    files = [np.fromfile(f["path"], dtype=np.uint8) for f in ck.files()]
+    tensors = {t.name: t for t in ck.tensors()}
+    out = {p.name: np.zeros(p.nbytes, dtype=np.uint8) for p in plan.params}
+    for w in plan.writes():
+        t = tensors[w.tensor]
+        src = files[t.file_index][t.file_offset : t.file_offset + t.nbytes]
+        dst = out[w.param]
+        mul = 2 if w.cast else 1
+        for r in range(w.rows):
+            s = src[w.src_offset + r * w.src_pitch : w.src_offset + r * w.src_pitch + w.row_bytes * mul]
+            if w.cast:
+                u = s.view("<u4").astype(np.uint64)
+                b = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+                b[(u & 0x7FFFFFFF) > 0x7F800000] = nan_bits
+                s = b.view(np.uint8)
+            dst[w.dst_offset + r * w.dst_pitch : w.dst_offset + r * w.dst_pitch + w.row_bytes] = s
+    return out
+
+
+def tiny_layouts():
+    """Small instances of the five benchmark families: ``name -> (layout, tp, ep, shards, ckpt kwargs)``."""
+    return {
+        "gpt2": (models.Gpt2(layers=2, hidden=32, ffn=64, vocab=97, positions=16), 1, 1, 1, {}),
+        "llama_tp4": (models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256), 4, 1, 3, {}),
+        "llama_f32_refit": (models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
+                            4, 1, 2, {"dtype": "F32", "edge_cases": models.NORMAL_EDGE_DENSE}),
+        "mixtral": (models.Mixtral(layers=2, hidden=32, ffn=48, q_heads=4, kv_heads=2, head_dim=8, vocab=64, experts=4),
+                    1, 1, 3, {}),
+        "mixtral_tp2": (models.Mixtral(layers=1, hidden=32, ffn=48, q_heads=4, kv_heads=2, head_dim=8, vocab=64, experts=4),
+                        2, 1, 2, {}),
+        "deepseek_ep": (models.DeepSeekV3(layers=3, dense_layers=1, hidden=512, q_lora=256, kv_lora=128, heads=4,
+                                          qk_nope=128, qk_rope=64, v_head=128, routed_experts=8, moe_ffn=512,
+                                          dense_ffn=1024, vocab=512), 2, 2, 4, {}),
+    }

@@ -1,0 +1,124 @@
+"""Stand-alone device operators against the CPU oracle, through the C ABI."""
+
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(arr: np.ndarray) -> torch.Tensor:
+    return torch.from_numpy(np.ascontiguousarray(arr).view(np.uint8).reshape(-1).copy()).cuda()
+
+
+SIZES = [0, 1, 3, 4, 15, 16, 17, 255, 4096, 4097, 65536, 65537, 8192 * 3 + 5, 1 << 20, (1 << 22) + 12345]
+
+
+def test_checksum32_matches_oracle(gpu_engine, oracle, oracle_c):
+    rng = np.random.default_rng(10)
+    bufs = [rng.integers(0, 256, n, dtype=np.uint8) for n in SIZES]
+    dev = [_dev(b) if b.size else torch.empty(0, dtype=torch.uint8, device="cuda") for b in bufs]
+    got = gpu_engine.checksum32(dev)
+    for b, g in zip(bufs, got):
+        assert g == oracle_c.checksum32(b), b.size
+    assert got[3] == oracle.safe_checksum_bigint(bufs[3].tobytes())
+    assert got[8] == oracle.safe_checksum_bytes(bufs[8])
+
+
+def test_checksum32_unaligned_views(gpu_engine, oracle_c):
+    rng = np.random.default_rng(11)
+    base = rng.integers(0, 256, 70000, dtype=np.uint8)
+    d = _dev(base)
+    for off, n in [(1, 1000), (2, 4096), (3, 65000), (4, 8192), (8, 33333), (13, 16), (16, 50000)]:
+        got = gpu_engine.checksum32([d[off: off + n]])[0]
+        assert got == oracle_c.checksum32(base[off: off + n]), (off, n)
+
+
+def test_checksum32_constant_closed_form(gpu_engine):
+    K = 2654435761
+    n = (1 << 24) + 7
+    d = torch.full((n,), 3, dtype=torch.uint8, device="cuda")
+    want = (3 * (K * (n * (n - 1) // 2) + n)) & 0xFFFFFFFF
+    assert gpu_engine.checksum32([d])[0] == format(want, "08x")
+
+
+def test_digest_matches_oracle(gpu_engine, oracle, oracle_c):
+    rng = np.random.default_rng(12)
+    sizes = [0, 1, 3, 4, 7, 4095, 4096, 4097, 4099, 65536, 65536 + 4096 * 3 + 9, 16 * 4096, 17 * 4096 + 2, 1 << 21]
+    bufs = [rng.integers(0, 256, n, dtype=np.uint8) for n in sizes]
+    dev = [_dev(b) if b.size else torch.empty(0, dtype=torch.uint8, device="cuda") for b in bufs]
+    hexes, scalars = gpu_engine.digest(dev, with_scalars=True)
+    for b, h, sc in zip(bufs, hexes, scalars):
+        assert sc == oracle_c.digest_scalars(b), b.size
+        assert h == oracle.tensor_digest_bytes(b.tobytes()), b.size
+
+
+def test_digest_reference_invariants_on_device(gpu_engine, oracle):
+    a = np.arange(8192, dtype=np.int32)
+    b = a.copy()
+    b[0:1024], b[1024:2048] = a[1024:2048], a[0:1024]
+    da, db = gpu_engine.digest([_dev(a), _dev(b)])
+    assert da != db and da == oracle.tensor_digest_bytes(a.tobytes())
+    # offset independence, including a 2-byte-aligned start (bf16 view at an odd element)
+    flat = np.arange(20000, dtype=np.uint16)
+    d = _dev(flat)
+    view = d[2 * 1409: 2 * 1409 + 2 * 9000]
+    assert gpu_engine.digest([view])[0] == oracle.tensor_digest_bytes(flat[1409: 1409 + 9000].tobytes())
+    neg = np.full(4096, -1, dtype=np.int32)
+    assert gpu_engine.digest([_dev(neg)])[0] == oracle.tensor_digest_bytes(neg.tobytes())
+
+
+def test_cast_f32_bf16_matches_oracle(gpu_engine, oracle, oracle_c):
+    rng = np.random.default_rng(13)
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=np.uint32)
+    classes = (hi[:, None] | lows[None, :]).reshape(-1)
+    rnd = rng.integers(0, 1 << 32, (1 << 20) + 3, dtype=np.uint64).astype(np.uint32)
+    for src in (classes, rnd, rnd[:1], rnd[:7], rnd[:8], rnd[:4099]):
+        s = _dev(src)
+        d = torch.zeros(src.size * 2 + 16, dtype=torch.uint8, device="cuda")
+        csum = gpu_engine.cast_f32_bf16(s, d, src.size)
+        got = d[: src.size * 2].cpu().numpy().view(np.uint16)
+        want = oracle.cast_f32_bf16_bits(src)
+        assert np.array_equal(got, want)
+        assert np.array_equal(got, oracle_c.cast_f32_bf16(src))
+        assert csum == oracle_c.checksum32(want)
+        assert int(d[src.size * 2:].sum()) == 0  # nothing written past the end
+
+
+def test_cast_nan_image_is_a_parameter(mxp, oracle):
+    from modelexpress_amd.engine import PlacementEngine
+
+    eng = PlacementEngine(0, nan_bits=0xFFFF)
+    src = np.array([0x7FC00001, 0xFFFFFFFF, 0x7F800001, 0x3F800000], dtype=np.uint32)
+    d = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    eng.cast_f32_bf16(_dev(src), d, 4)
+    assert d[:8].cpu().numpy().view(np.uint16).tolist() == [0xFFFF, 0xFFFF, 0xFFFF, 0x3F80]
+    ref = torch.from_numpy(src.view(np.float32).copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert ref[3] == 0x3F80 and all((int(v) & 0x7FFF) > 0x7F80 for v in ref[:3])
+    eng.close()
+
+
+@pytest.mark.parametrize("rows,row_bytes,src_pitch,dst_pitch,src_off", [
+    (4096, 1024, 8192, 1024, 1024 * 3),      # o_proj TP=8 column slice
+    (512, 3584, 28672, 3584, 3584 * 5),      # down_proj TP=8 column slice
+    (56, 64, 512, 64, 64 * 2),               # fp8 scale-tile column slice
+    (7, 13, 29, 17, 3),                      # byte-granular
+    (33, 20, 44, 24, 4),                     # dword-granular
+    (1, 100001, 100001, 100001, 0),          # contiguous odd size
+    (3, 70000, 140000, 70000, 16),           # rows wider than one tile row
+])
+def test_gather2d_matches_oracle(gpu_engine, oracle_c, rows, row_bytes, src_pitch, dst_pitch, src_off):
+    rng = np.random.default_rng(14)
+    src = rng.integers(0, 256, src_off + rows * src_pitch + 64, dtype=np.uint8)
+    want = np.full(rows * dst_pitch + 32, 0xEE, dtype=np.uint8)
+    for r in range(rows):
+        want[r * dst_pitch: r * dst_pitch + row_bytes] = src[src_off + r * src_pitch: src_off + r * src_pitch + row_bytes]
+    s = _dev(src)
+    d = torch.full((want.size,), 0xEE, dtype=torch.uint8, device="cuda")
+    csum = gpu_engine.gather2d(s[src_off:], src_pitch, d, dst_pitch, rows, row_bytes)
+    assert np.array_equal(d.cpu().numpy(), want)
+    acc = 0
+    for r in range(rows):
+        acc += int(oracle_c.checksum32(want[r * dst_pitch: r * dst_pitch + row_bytes], first_index=r * dst_pitch), 16)
+    assert csum == format(acc & 0xFFFFFFFF, "08x")

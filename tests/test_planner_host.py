@@ -1,0 +1,29 @@
+"""The product planner (C++, through the C ABI) against the CPU oracle, on the host:
+its pitched-box writes are interpreted with numpy and compared byte for byte with the
+oracle's parameter buffers.  No device work happens here."""
+
+import numpy as np
+import pytest
+
+from helpers import apply_plan_numpy, make_plan, oracle_place, tiny_layouts
+from modelexpress_amd import synth
+
+
+@pytest.mark.parametrize("name", list(tiny_layouts()))
+def test_plan_matches_oracle_for_every_rank(name, mxp, oracle, tmp_path):
+    layout, tp, ep, shards, ck_kw = tiny_layouts()[name]
+    cast = ck_kw.get("dtype") == "F32"
+    synth.write_checkpoint(layout.checkpoint(**ck_kw), str(tmp_path), n_shards=shards, seed=3)
+    for tp_rank in range(tp):
+        for ep_rank in range(ep):
+            if ep > 1 and ep_rank != tp_rank % ep:
+                continue
+            rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=ep_rank,
+                                  param_dtype="BF16" if cast else None)
+            want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
+            ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
+            got = apply_plan_numpy(ck, plan)
+            for p in plan.params:
+                assert got[p.name].tobytes() == want[p.name].tobytes(), (name, tp_rank, p.name)
+            info = plan.param_info()
+            assert all(i["bytes_written"] == i["nbytes"] for i in info)
