@@ -642,9 +642,10 @@ class MdlOracle:
         else:
             raise RuntimeError(f"no conversion from {src.dtype} to {dest.dtype}")
 
-    def load_weights(self, weights, strict_params: bool = True) -> dict:
-        """Classify, resolve every write, check coverage, then copy (installer.py:366-437
-        with the loaderless coverage rule of :219-251 applied to every parameter)."""
+    def resolve(self, weights, strict_params: bool = True) -> list:
+        """Classify and resolve every write, check coverage; nothing is copied
+        (installer.py:366-410 with the coverage rule of :219-251 applied to every
+        parameter).  Returns ``[(kind, dest_view, src_view)]``."""
         weights = list(weights)
         self.extend_dest_map(weights)
         writes, unmapped = [], []
@@ -672,6 +673,11 @@ class MdlOracle:
         missing = sorted(required - self.covered)
         if missing:
             raise CoverageError(f"uncovered local parameters={missing[:10]}")
+        return writes
+
+    def load_weights(self, weights, strict_params: bool = True) -> dict:
+        """Resolve everything, then copy (installer.py:419-424)."""
+        writes = self.resolve(weights, strict_params)
         counts = {"direct": 0, "fused": 0, "expert": 0}
         for kind, dest, src in writes:
             self._copy(dest, src)
