@@ -204,7 +204,7 @@ typedef struct mxp_engine_options {
   uint64_t slot_bytes;     /* bytes per slot; 0 = default 64 MiB */
   int32_t reader_threads;  /* pread workers; 0 = default 8 */
   int32_t streams;         /* HIP streams for H2D + kernels; 0 = default 4 */
-  uint32_t tile_bytes;     /* destination bytes per workgroup; 0 = default 64 KiB */
+  uint32_t tile_bytes;     /* destination bytes per workgroup; 0 = default 128 KiB */
   uint16_t nan_bits;       /* bf16 image of every NaN in the cast; 0 = default 0x7FC0 */
   uint16_t reserved0;
   int32_t use_o_direct;    /* 1 = open files with O_DIRECT (falls back if unsupported) */

@@ -10,8 +10,11 @@ from __future__ import annotations
 import ctypes as C
 from pathlib import Path
 
+import os
+
 PKG_DIR = Path(__file__).resolve().parent
-LIB_PATH = PKG_DIR / "libmxplace.so"
+# MXP_LIBRARY_PATH selects another build of the same library (same ABI), e.g. a tuning variant.
+LIB_PATH = Path(os.environ["MXP_LIBRARY_PATH"]) if os.environ.get("MXP_LIBRARY_PATH") else PKG_DIR / "libmxplace.so"
 
 MXP_MAX_DIMS = 8
 

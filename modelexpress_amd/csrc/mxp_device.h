@@ -56,7 +56,9 @@ struct alignas(16) DigestJob {
 };
 
 constexpr uint32_t kKnuth = 2654435761u;
-constexpr int kPlaceThreads = 256;
+constexpr int kPlaceThreads = 1024;  // lanes per placement workgroup (16 wavefronts)
+constexpr int kPlaceBatch = 8;       // 16-byte units each lane keeps in flight
+constexpr int kDigestThreads = 256;
 constexpr uint32_t kDigestRowWords = 1024;   // 4 KiB rows
 constexpr uint32_t kDigestRowsPerBlock = 16; // 64 KiB per workgroup
 

@@ -368,7 +368,7 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     if (o.slot_bytes == 0) o.slot_bytes = 64ull << 20;
     if (o.reader_threads <= 0) o.reader_threads = 8;
     if (o.streams <= 0) o.streams = 4;
-    if (o.tile_bytes == 0) o.tile_bytes = 64 * 1024;
+    if (o.tile_bytes == 0) o.tile_bytes = kPlaceThreads * kPlaceBatch * 16;
     if (o.nan_bits == 0) o.nan_bits = 0x7FC0;
     if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
     if (o.tile_bytes < 1024 || o.tile_bytes > (1u << 20)) throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 1 MiB]");

@@ -78,6 +78,19 @@ __device__ __forceinline__ uint4 cast8(const uint4& a, const uint4& b, uint32_t 
   return o;
 }
 
+// 128-bit non-temporal accesses: every byte is touched exactly once, so nothing is worth
+// keeping in L2 / Infinity Cache (measured: +3..4% over plain accesses on this copy).
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld16(const uint8_t* p) {
+  const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void st16(uint8_t* p, const uint4& v) {
+  u32x4 t;
+  t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w;
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+}
+
 // One tile of one segment.  UNIT = destination bytes handled per lane access.
 // Lanes walk the tile in flattened (row, unit) order, so neighbouring lanes touch
 // neighbouring 16-byte units of the same row: every wavefront access is a run of
@@ -99,45 +112,51 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
   };
 
   if constexpr (UNIT == 16) {
-    uint32_t v = threadIdx.x;
-    // Four independent 16-byte units in flight per lane before the first store.
-    for (; v + 3u * kPlaceThreads < n_units; v += 4u * kPlaceThreads) {
-      uint32_t so[4], d_o[4];
-      uint4 x[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) locate(v + k * kPlaceThreads, so[k], d_o[k]);
+    // One batch = kPlaceBatch units per lane: every load of the batch is issued before its
+    // first store, so a workgroup presents the memory system with a burst of reads over
+    // one contiguous region followed by a burst of writes over another.  With the default
+    // tile (kPlaceThreads * kPlaceBatch * 16 B = 128 KiB) a workgroup runs exactly one
+    // batch; that shape measured fastest (5.98 TB/s against 5.16 TB/s for 256 lanes x 4).
+    constexpr int U = kPlaceBatch;
+    for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += (uint32_t)U * kPlaceThreads) {
+      uint32_t d_o[U];
+      uint4 x[U];
+      bool ok[U];
       if constexpr (OP == kOpCastF32Bf16) {
-        uint4 a[4], b[4];
+        uint4 a[U], b[U];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          a[k] = *reinterpret_cast<const uint4*>(src + so[k]);
-          b[k] = *reinterpret_cast<const uint4*>(src + so[k] + 16);
+        for (int k = 0; k < U; ++k) {
+          const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
+          ok[k] = v < n_units;
+          if (ok[k]) {
+            uint32_t so;
+            locate(v, so, d_o[k]);
+            a[k] = ld16(src + so);
+            b[k] = ld16(src + so + 16);
+          }
         }
 #pragma unroll
-        for (int k = 0; k < 4; ++k) x[k] = cast8(a[k], b[k], nan_bits);
+        for (int k = 0; k < U; ++k)
+          if (ok[k]) x[k] = cast8(a[k], b[k], nan_bits);
       } else {
 #pragma unroll
-        for (int k = 0; k < 4; ++k) x[k] = *reinterpret_cast<const uint4*>(src + so[k]);
+        for (int k = 0; k < U; ++k) {
+          const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
+          ok[k] = v < n_units;
+          if (ok[k]) {
+            uint32_t so;
+            locate(v, so, d_o[k]);
+            x[k] = ld16(src + so);
+          }
+        }
       }
 #pragma unroll
-      for (int k = 0; k < 4; ++k) {
-        if constexpr (OP != kOpChecksumOnly) *reinterpret_cast<uint4*>(dst + d_o[k]) = x[k];
-        cs.add16(x[k], csum_base + d_o[k]);
+      for (int k = 0; k < U; ++k) {
+        if (ok[k]) {
+          if constexpr (OP != kOpChecksumOnly) st16(dst + d_o[k], x[k]);
+          cs.add16(x[k], csum_base + d_o[k]);
+        }
       }
-    }
-    for (; v < n_units; v += kPlaceThreads) {
-      uint32_t so, d_o;
-      locate(v, so, d_o);
-      uint4 x;
-      if constexpr (OP == kOpCastF32Bf16) {
-        const uint4 a = *reinterpret_cast<const uint4*>(src + so);
-        const uint4 b = *reinterpret_cast<const uint4*>(src + so + 16);
-        x = cast8(a, b, nan_bits);
-      } else {
-        x = *reinterpret_cast<const uint4*>(src + so);
-      }
-      if constexpr (OP != kOpChecksumOnly) *reinterpret_cast<uint4*>(dst + d_o) = x;
-      cs.add16(x, csum_base + d_o);
     }
   } else {
     for (uint32_t v = threadIdx.x; v < n_units; v += kPlaceThreads) {
@@ -227,7 +246,7 @@ __device__ __forceinline__ void digest_rows(const uint8_t* __restrict__ p, uint6
                                             uint64_t row_end, unsigned long long& A,
                                             unsigned long long& B) {
   const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (uint64_t r = row_begin + wave; r < row_end; r += kPlaceThreads / 64) {
+  for (uint64_t r = row_begin + wave; r < row_end; r += kDigestThreads / 64) {
     const uint8_t* row = p + r * (uint64_t)(kDigestRowWords * 4);
     long long acc = 0;
     if constexpr (ALIGNED16) {
@@ -253,7 +272,7 @@ __device__ __forceinline__ void digest_rows(const uint8_t* __restrict__ p, uint6
   }
 }
 
-__global__ __launch_bounds__(kPlaceThreads) void digest_kernel(
+__global__ __launch_bounds__(kDigestThreads) void digest_kernel(
     const DigestJob* __restrict__ jobs, uint32_t n_jobs, unsigned long long* __restrict__ out) {
   // Workgroup-uniform binary search for the job that owns this workgroup.
   uint32_t lo = 0, hi = n_jobs;
@@ -279,7 +298,7 @@ __global__ __launch_bounds__(kPlaceThreads) void digest_kernel(
   if (blk == n_blocks - 1) {
     const uint8_t* tail = j.ptr + rows * (uint64_t)(kDigestRowWords * 4);
     const uint32_t tw = (uint32_t)(body_words - rows * kDigestRowWords);
-    for (uint32_t k = threadIdx.x; k < tw; k += kPlaceThreads) {
+    for (uint32_t k = threadIdx.x; k < tw; k += kDigestThreads) {
       const uint8_t* b = tail + 4u * k;
       const uint32_t u = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) |
                          ((uint32_t)b[3] << 24);
@@ -293,7 +312,7 @@ __global__ __launch_bounds__(kPlaceThreads) void digest_kernel(
     }
   }
 
-  __shared__ unsigned long long part[kPlaceThreads / 64][5];
+  __shared__ unsigned long long part[kDigestThreads / 64][5];
   unsigned long long v[5] = {A, B, At, Bt, Rg};
 #pragma unroll
   for (int q = 0; q < 5; ++q) {
@@ -304,7 +323,7 @@ __global__ __launch_bounds__(kPlaceThreads) void digest_kernel(
   if (threadIdx.x < 5) {
     unsigned long long t = 0;
 #pragma unroll
-    for (int k = 0; k < kPlaceThreads / 64; ++k) t += part[k][threadIdx.x];
+    for (int k = 0; k < kDigestThreads / 64; ++k) t += part[k][threadIdx.x];
     if (t) atomicAdd(&out[j.out_slot + threadIdx.x], t);
   }
 }
@@ -312,7 +331,7 @@ __global__ __launch_bounds__(kPlaceThreads) void digest_kernel(
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
                          unsigned long long* out_dev, hipStream_t stream) {
   if (n_jobs == 0 || n_blocks == 0) return hipSuccess;
-  hipLaunchKernelGGL(digest_kernel, dim3(n_blocks), dim3(kPlaceThreads), 0, stream, jobs_dev,
+  hipLaunchKernelGGL(digest_kernel, dim3(n_blocks), dim3(kDigestThreads), 0, stream, jobs_dev,
                      n_jobs, out_dev);
   return hipGetLastError();
 }

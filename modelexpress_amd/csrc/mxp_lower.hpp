@@ -23,7 +23,7 @@ struct BoxCopy {
 };
 
 struct LowerOptions {
-  uint32_t tile_bytes = 64 * 1024;  // destination bytes one workgroup handles
+  uint32_t tile_bytes = 128 * 1024;  // destination bytes one workgroup handles (one batch)
   uint32_t flat_row_bytes = 8192;   // virtual row width used to tile contiguous runs
   uint32_t max_row_bytes = 32768;   // wider pitched rows are split by columns
 };
