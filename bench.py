@@ -38,7 +38,7 @@ HBM_PEAK_GBPS = 8000.0
 # counter scaled by its reading for a plain 1 GiB device copy).  Counters cannot be read
 # from inside this process, so the figure is carried here and reported only when the
 # workload is the profiled one.
-PROFILED_TRAFFIC_BYTES = {("llama", 32, 8): 4_095_900_000}
+PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_095_900_000}
 
 
 def _log(msg: str) -> None:
@@ -62,11 +62,18 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--rank", type=int, default=3, help="tensor-parallel rank whose slice is placed")
-    ap.add_argument("--layers", type=int, default=32, help="reduce only for a quick functional check")
+    ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
+                    help="BASELINE.json configuration (1-based); 2 = Llama-3-8B, the one the metric is quoted on")
+    ap.add_argument("--rank", type=int, default=3, help="tensor-parallel (and expert-parallel) rank whose share is placed")
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the configuration's own)")
+    ap.add_argument("--max-file-gb", type=float, default=40.0,
+                    help="write real checkpoint files (ingest and CPU legs) only below this size")
     ap.add_argument("--tile-kib", type=int, default=0, help="destination KiB per workgroup (0 = library default)")
     ap.add_argument("--no-e2e", action="store_true", help="skip the file-ingest leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--slot-mib", type=int, default=16, help="pinned ring slot size for the ingest leg")
+    ap.add_argument("--ring-slots", type=int, default=32)
+    ap.add_argument("--readers", type=int, default=0, help="reader threads for the ingest leg (0 = host cores, at most 16)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB device copy (a kernel of known traffic, for scaling profiler counters)")
     ap.add_argument("--seed", type=int, default=20240229)
@@ -85,14 +92,41 @@ def main() -> int:
     from modelexpress_amd.engine import Checkpoint, PlacementEngine, PlacementPlan
 
     _lib.lib()  # fail loudly if the HIP library is missing
-    tp = 8
-    layout = models.Llama(layers=args.layers)
-    tensors = layout.checkpoint()
+    layout, tp, ep, n_shards, ck_dtype, ck_kind = models.baseline_config(args.config)
+    if args.layers:
+        layout.dims["layers"] = args.layers
+        if args.config == 5:
+            n_shards = max(1, round(163 * args.layers / 61))
+    elif args.config == 5:
+        # The whole 681 GB model cannot be staged on one GPU: 3 dense + 8 MoE layers are run
+        # at their real shapes (per-layer work is identical across the 58 MoE layers).
+        layout.dims["layers"] = 11
+        n_shards = 30
+    n_layers = layout.dims["layers"]
+    cast = ck_dtype == "F32"
+    ck_kwargs = {}
+    if ck_dtype and args.config in (2, 3):
+        ck_kwargs = {"dtype": ck_dtype, "edge_cases": ck_kind}
+    tensors = layout.checkpoint(**ck_kwargs)
     total_bytes = sum(t.nbytes for t in tensors)
-    rv = layout.rank_view(tp_size=tp, tp_rank=args.rank)
+    rank = args.rank % tp
+    ep_rank = rank % ep
+    rv = layout.rank_view(tp_size=tp, tp_rank=rank, ep_size=ep, ep_rank=ep_rank, param_dtype="BF16" if cast else None)
     host_threads = min(16, os.cpu_count() or 1)
+    workloads = {
+        1: "configs[0]: GPT-2-small-shaped fp16 checkpoint, one safetensors file; every tensor placed unsliced (TP=1) "
+           "with its checksum",
+        2: "configs[1]: Llama-3-8B-shaped bf16 checkpoint, 4 safetensors shards resident in HBM; one TP=8 rank slice "
+           "(q/k/v/gate/up rows, o/down columns, vocab-split embeddings), fused QKV and gate_up, 195 buffers with checksums",
+        3: "configs[2]: RL refit of the resident Llama-3-8B TP=8 rank slice from an fp32 checkpoint staged in HBM: "
+           "slice + fp32->bf16 round-to-nearest-even cast (denormals, +-inf, NaN at 1e-6 density) + checksums",
+        4: "configs[3]: Mixtral-8x7B-shaped bf16 checkpoint, 19 shards resident in HBM; experts stacked into "
+           "w13 [8,28672,4096] / w2 [8,4096,14336], fused QKV, TP=1",
+        5: "configs[4]: DeepSeek-V3-shaped fp8-e4m3 weights with fp32 128x128 scale tiles; one TP=8 / EP=8 rank share "
+           "(MLA projections sliced, 32 of 256 routed experts stacked, scale tiles block-aligned)",
+    }
 
-    want_files = not (args.no_e2e and args.no_cpu)
+    want_files = not (args.no_e2e and args.no_cpu) and total_bytes <= args.max_file_gb * 1e9
     workdir = _pick_workdir(total_bytes) if want_files else None
     files_real = workdir is not None
     if workdir is None:
@@ -100,16 +134,15 @@ def main() -> int:
     try:
         t0 = time.perf_counter()
         if files_real:
-            synth.write_checkpoint(tensors, workdir, n_shards=4, seed=args.seed, threads=host_threads)
+            synth.write_checkpoint(tensors, workdir, n_shards=n_shards, seed=args.seed, threads=host_threads)
             _log(f"wrote {total_bytes / 1e9:.2f} GB checkpoint to {workdir} in {time.perf_counter() - t0:.1f}s")
         else:
-            synth.write_headers_only(tensors, workdir, n_shards=4)
+            synth.write_headers_only(tensors, workdir, n_shards=n_shards)
             _log("no room for checkpoint files: resident leg only")
         ck = Checkpoint(workdir)
-        plan = PlacementPlan(ck, rv.params, tp_size=tp, tp_rank=args.rank,
-                             stacked_params_mapping=rv.stacked_params_mapping)
-        eng = PlacementEngine(0, ring_slots=8, slot_bytes=64 << 20, reader_threads=host_threads, streams=4,
-                              tile_bytes=args.tile_kib * 1024)
+        plan = PlacementPlan(ck, rv.params, tp_size=tp, tp_rank=rank, stacked_params_mapping=rv.stacked_params_mapping,
+                             expert_mapping=rv.expert_mapping, allow_cast=cast)
+        eng = PlacementEngine(0, tile_bytes=args.tile_kib * 1024)
         totals = plan.totals()
         placed = totals["placed_bytes"]
         algo = totals["kernel_algorithmic_bytes"]
@@ -149,7 +182,7 @@ def main() -> int:
         achieved = algo / (k_avg * 1e-3) / 1e9
         roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
-                    "traffic": PROFILED_TRAFFIC_BYTES.get(("llama", args.layers, tp)),
+                    "traffic": PROFILED_TRAFFIC_BYTES.get((layout.family, n_layers, tp, cast)),
                     "kernel": "place_kernel", "kernel_ms_avg": round(k_avg, 4), "kernel_ms_min": round(min(k_ms), 4),
                     "algorithmic_bytes": algo, "workgroups": info["n_workgroups"], "segments": info["n_segments"]}
 
@@ -157,11 +190,10 @@ def main() -> int:
             "metric": "placed-weight GB/s into HBM end-to-end + kernel HBM GB/s vs peak, Llama-3-8B",
             "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "u8", "data": "synthetic",
-            "config": {"workload": "configs[1]: Llama-3-8B-shaped bf16 checkpoint, 4 safetensors shards resident in HBM; "
-                                   "one TP=8 rank slice (q/k/v/gate/up rows, o/down columns, vocab-split embeddings), "
-                                   "fused QKV and gate_up, 195 buffers with checksums",
-                       "layers": args.layers, "tp_size": tp, "tp_rank": args.rank, "checkpoint_bytes": total_bytes,
+            "dtype": "f32->bf16" if cast else "u8", "data": "synthetic",
+            "config": {"workload": workloads[args.config], "family": layout.family,
+                       "layers": n_layers, "tp_size": tp, "tp_rank": rank, "ep_size": ep, "ep_rank": ep_rank,
+                       "checkpoint_bytes": total_bytes,
                        "placed_bytes": placed, "buffers": len(plan.params), "timed": "device placement, one launch per step"},
             "roofline": roofline,
         }
@@ -170,35 +202,46 @@ def main() -> int:
         agree = True
         if files_real and not args.no_e2e:
             h2d_peak = eng.measure_h2d(256 << 20, 5) / 1e9
-            best = None
-            for i in range(3):
-                dst2 = dst if i else eng.allocate(plan, fill=0)
-                st = eng.execute(plan, dst2)
-                if i and (best is None or st["wall_seconds"] < best["wall_seconds"]):
-                    best = st
-            ingest_sums = eng.checksums(plan)
-            agree = agree and ingest_sums == resident_sums
-            w = best["wall_seconds"]
-            out["e2e_ingest"] = {
-                "placed_gbps": round(best["placed_bytes"] / w / 1e9, 2), "h2d_gbps": round(best["h2d_bytes"] / w / 1e9, 2),
-                "h2d_peak_gbps": round(h2d_peak, 2), "frac_of_h2d_peak": round(best["h2d_bytes"] / w / 1e9 / h2d_peak, 4),
-                "wall_s": round(w, 4), "file_bytes": best["file_bytes"], "h2d_bytes": best["h2d_bytes"],
-                "reader_threads": host_threads, "ring": "8 x 64 MiB pinned", "source": f"page cache ({workdir})",
-                "checksums_match_resident": ingest_sums == resident_sums}
-            _log(f"e2e ingest: {out['e2e_ingest']}")
+            for key, pack in (("e2e_ingest", True), ("e2e_ingest_band", False)):
+                e2 = PlacementEngine(0, ring_slots=args.ring_slots, slot_bytes=args.slot_mib << 20,
+                                     reader_threads=args.readers or host_threads, streams=4,
+                                     tile_bytes=args.tile_kib * 1024, pack_strided_on_host=pack)
+                best = None
+                for i in range(4):
+                    st = e2.execute(plan, dst)
+                    if i and (best is None or st["wall_seconds"] < best["wall_seconds"]):
+                        best = st
+                ingest_sums = e2.checksums(plan)
+                e2.close()
+                agree = agree and ingest_sums == resident_sums
+                w = best["wall_seconds"]
+                out[key] = {
+                    "placed_gbps": round(best["placed_bytes"] / w / 1e9, 2), "h2d_gbps": round(best["h2d_bytes"] / w / 1e9, 2),
+                    "h2d_peak_gbps": round(h2d_peak, 2), "frac_of_h2d_peak": round(best["h2d_bytes"] / w / 1e9 / h2d_peak, 4),
+                    "wall_s": round(w, 4), "file_bytes": best["file_bytes"], "h2d_bytes": best["h2d_bytes"],
+                    "strided_slices": "rows packed into the pinned slot by the readers" if pack else
+                                      "whole row bands staged, gathered on the device",
+                    "reader_threads": args.readers or host_threads,
+                    "ring": f"{args.ring_slots} x {args.slot_mib} MiB pinned", "source": f"page cache ({workdir})",
+                    "checksums_match_resident": ingest_sums == resident_sums}
+                _log(f"{key}: {out[key]}")
 
         # ---- CPU baseline: the oracle placing the same rank from the same files ----
         if files_real and not args.no_cpu:
             from oracle import cpu_path
 
-            res = cpu_path.run(workdir, [(p.name, p.dtype, p.shape) for p in rv.params], tp_size=tp, tp_rank=args.rank,
-                               stacked=rv.stacked_params_mapping, threads=host_threads, repeats=3)
+            local_of = {int(r[2]): int(r[4]) for r in (rv.expert_mapping or [])}
+            res = cpu_path.run(workdir, [(p.name, p.dtype, p.shape) for p in rv.params], tp_size=tp, tp_rank=rank,
+                               stacked=rv.stacked_params_mapping,
+                               expert_mapping=[r[:4] for r in rv.expert_mapping] if rv.expert_mapping else None,
+                               expert_local=(lambda _f, g: local_of.get(g, g)) if rv.expert_mapping else None,
+                               allow_cast=cast, threads=host_threads, repeats=3)
             cpu_sums = [res["checksums"][p.name] for p in rv.params]
             agree = agree and cpu_sums == resident_sums
             out["cpu_baseline"] = {
                 "value": round(res["placed_bytes"] / res["place_s"] / 1e9, 3), "unit": "GB/s", "cores": res["threads"],
                 "kind": "port",
-                "sample": f"the full TP rank slice ({res['placed_bytes']} placed bytes, {res['n_writes']} writes) from the "
+                "sample": f"the full rank share ({res['placed_bytes']} placed bytes, {res['n_writes']} writes) from the "
                           f"same files, best of 3; parse {res['parse_s']:.3f}s + plan {res['plan_s']:.3f}s not included",
                 "place_s": round(res["place_s"], 4), "host_cpus": os.cpu_count(),
                 "checksums_match_gpu": cpu_sums == resident_sums}

@@ -200,13 +200,16 @@ typedef struct mxp_engine mxp_engine;
 
 typedef struct mxp_engine_options {
   int32_t device;          /* HIP device ordinal */
-  int32_t ring_slots;      /* pinned host slots (each with a device bounce slot); 0 = default 8 */
-  uint64_t slot_bytes;     /* bytes per slot; 0 = default 64 MiB */
+  int32_t ring_slots;      /* pinned host slots (each with a device bounce slot); 0 = default 32 */
+  uint64_t slot_bytes;     /* bytes per slot; 0 = default 16 MiB */
   int32_t reader_threads;  /* pread workers; 0 = default 8 */
   int32_t streams;         /* HIP streams for H2D + kernels; 0 = default 4 */
   uint32_t tile_bytes;     /* destination bytes per workgroup; 0 = default 128 KiB */
   uint16_t nan_bits;       /* bf16 image of every NaN in the cast; 0 = default 0x7FC0 */
-  uint16_t reserved0;
+  uint16_t pack_strided_on_host; /* strided slices: 1 = readers pack the needed rows into the
+                                    slot (only placed bytes cross PCIe), 2 = stage whole row
+                                    bands and gather on the device, 0 = default (1, or 2
+                                    with use_o_direct) */
   int32_t use_o_direct;    /* 1 = open files with O_DIRECT (falls back if unsupported) */
 } mxp_engine_options;
 

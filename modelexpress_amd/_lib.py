@@ -77,7 +77,7 @@ class ParamInfo(C.Structure):
 class EngineOptions(C.Structure):
     _fields_ = [("device", C.c_int32), ("ring_slots", C.c_int32), ("slot_bytes", C.c_uint64),
                 ("reader_threads", C.c_int32), ("streams", C.c_int32), ("tile_bytes", C.c_uint32),
-                ("nan_bits", C.c_uint16), ("reserved0", C.c_uint16), ("use_o_direct", C.c_int32)]
+                ("nan_bits", C.c_uint16), ("pack_strided_on_host", C.c_uint16), ("use_o_direct", C.c_int32)]
 
 
 class ExecStats(C.Structure):

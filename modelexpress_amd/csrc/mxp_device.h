@@ -32,7 +32,7 @@ struct alignas(16) Seg {
   uint32_t src_buf;    // index into the source base-pointer table
   uint32_t dst_buf;    // index into the destination base-pointer table
   uint32_t op;         // SegOp
-  uint32_t unit;       // bytes per lane access on the destination side: 16, 4, 2 or 1
+  uint32_t unit;       // bytes per lane access on the destination side: 16, 8 (cast), 4, 2 or 1
   uint32_t rows_per_tile;
   uint32_t csum_slot;  // index into the checksum accumulator array, ~0u = none
   uint32_t units_per_row;  // row_bytes / unit

@@ -76,6 +76,7 @@ using namespace mxp;
 struct mxp_plan::Lowered {
   uint64_t slot_bytes = 0;
   uint32_t tile_bytes = 0;
+  bool host_pack = false;
   // resident tables: source buffer index = shard file index
   DevBuf<Seg> res_segs;
   DevBuf<WorkItem> res_work;
@@ -128,12 +129,15 @@ void free_lowered(mxp_plan::Lowered* l) { delete l; }
 // (file, offset) order, and lowers both the ingest and the resident descriptor tables.
 void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   if (!pl.built) throw Error(MXP_ERR_STATE, "plan has not been built");
-  if (pl.lowered && pl.lowered->slot_bytes == eng.opt.slot_bytes && pl.lowered->tile_bytes == eng.opt.tile_bytes)
+  const bool host_pack = eng.opt.pack_strided_on_host == 1;
+  if (pl.lowered && pl.lowered->slot_bytes == eng.opt.slot_bytes && pl.lowered->tile_bytes == eng.opt.tile_bytes &&
+      pl.lowered->host_pack == host_pack)
     return;
   if (pl.lowered) { free_lowered(pl.lowered); pl.lowered = nullptr; }
   auto L = std::make_unique<mxp_plan::Lowered>();
   L->slot_bytes = eng.opt.slot_bytes;
   L->tile_bytes = eng.opt.tile_bytes;
+  L->host_pack = host_pack;
   LowerOptions lo;
   lo.tile_bytes = eng.opt.tile_bytes;
   const mxp_ckpt& ck = *pl.ckpt;
@@ -168,8 +172,9 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   // ---- ingest: pieces in file order ----
   struct Piece {
     int file;
-    uint64_t file_off, nbytes;  // byte range to read
+    uint64_t file_off, nbytes;  // byte range to read (one row of it when rows > 1)
     BoxCopy box;                // src_off relative to the start of the range
+    uint64_t rows = 1, file_pitch = 0;  // rows > 1: strided in the file, packed in the slot
   };
   std::vector<Piece> pieces;
   const uint64_t slot = eng.opt.slot_bytes;
@@ -196,6 +201,22 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
         p.box.row_bytes = n;
         p.box.src_pitch = n * sm;
         p.box.dst_pitch = n;
+        pieces.push_back(p);
+      }
+    } else if (host_pack) {
+      // strided source, packed by the readers: only the needed bytes cross PCIe and the
+      // slot holds the rows back to back, so the device sees a plain copy
+      if (row_src > slot) throw Error(MXP_ERR_UNSUPPORTED, "a source row of '" + t.name + "' does not fit a staging slot");
+      const uint64_t max_rows = slot / row_src;
+      for (uint64_t r = 0; r < w.rows; r += max_rows) {
+        const uint64_t nr = std::min(max_rows, w.rows - r);
+        Piece p{t.file_index, t0 + r * w.src_pitch, row_src, b, nr, w.src_pitch};
+        p.box.src_off = 0;
+        p.box.dst_off = w.dst_offset + r * w.dst_pitch;
+        p.box.rows = nr;
+        p.box.row_bytes = w.row_bytes;
+        p.box.src_pitch = row_src;
+        p.box.dst_pitch = w.dst_pitch;
         pieces.push_back(p);
       }
     } else {
@@ -233,7 +254,8 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
     };
     for (auto& p : pieces) {
       uint64_t at = align_up(cur.used_bytes, 256);
-      if (!cur.ranges.empty() && at + p.nbytes > slot) {
+      const uint64_t in_slot = p.nbytes * p.rows;
+      if (!cur.ranges.empty() && at + in_slot > slot) {
         close();
         at = 0;
       }
@@ -241,9 +263,9 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
         cur.seg_begin = (uint32_t)segs.size();
         cur.work_begin = (uint32_t)work.size();
       }
-      cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at});
-      cur.used_bytes = at + p.nbytes;
-      L->file_bytes += p.nbytes;
+      cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at, p.rows, p.file_pitch});
+      cur.used_bytes = at + in_slot;
+      L->file_bytes += in_slot;
       p.box.src_off = at;
       const size_t w0 = work.size();
       lower_box(p.box, lo, segs, work);
@@ -364,12 +386,16 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     auto e = std::make_unique<mxp_engine>();
     if (opts) e->opt = *opts;
     auto& o = e->opt;
-    if (o.ring_slots <= 0) o.ring_slots = 8;
-    if (o.slot_bytes == 0) o.slot_bytes = 64ull << 20;
+    if (o.ring_slots <= 0) o.ring_slots = 32;
+    if (o.slot_bytes == 0) o.slot_bytes = 16ull << 20;
     if (o.reader_threads <= 0) o.reader_threads = 8;
     if (o.streams <= 0) o.streams = 4;
     if (o.tile_bytes == 0) o.tile_bytes = kPlaceThreads * kPlaceBatch * 16;
     if (o.nan_bits == 0) o.nan_bits = 0x7FC0;
+    // Packing strided rows on the host issues one read per row: right for the page cache,
+    // wrong for direct I/O, where whole row bands are staged and gathered on the device.
+    if (o.pack_strided_on_host == 0) o.pack_strided_on_host = o.use_o_direct ? 2 : 1;
+    if (o.pack_strided_on_host > 2) throw Error(MXP_ERR_ARG, "pack_strided_on_host must be 0, 1 or 2");
     if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
     if (o.tile_bytes < 1024 || o.tile_bytes > (1u << 20)) throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 1 MiB]");
     if (o.ring_slots > 256 || o.reader_threads > 256 || o.streams > 64) throw Error(MXP_ERR_ARG, "ring, thread or stream count too large");
@@ -480,7 +506,9 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
         if (turn > 0) HIP_OK(hipEventSynchronize(sl.done));
         const double t0 = now_s();
         for (const auto& r : ch.ranges)
-          pread_full(fds[r.file], sl.host + r.slot_off, r.nbytes, r.file_off, ck.files[r.file].path);
+          for (uint64_t row = 0; row < r.rows; ++row)
+            pread_full(fds[r.file], sl.host + r.slot_off + row * r.nbytes, r.nbytes, r.file_off + row * r.file_pitch,
+                       ck.files[r.file].path);
         read_s[tid] += now_s() - t0;
         hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
         HIP_OK(hipMemcpyAsync(sl.dev, sl.host, ch.used_bytes, hipMemcpyHostToDevice, st));

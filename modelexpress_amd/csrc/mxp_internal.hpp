@@ -76,7 +76,8 @@ struct ExpertRec { std::string param_prefix, weight_prefix; int expert_id; std::
 
 // One slot-sized unit of ingest work: byte ranges packed into a staging slot and the
 // device segments that consume them.
-struct FileRange { int file; uint64_t file_off, nbytes, slot_off; };
+// `rows` pieces of `nbytes`, `file_pitch` apart in the file, packed back to back in the slot.
+struct FileRange { int file; uint64_t file_off, nbytes, slot_off; uint64_t rows = 1, file_pitch = 0; };
 struct Chunk {
   std::vector<FileRange> ranges;
   uint64_t used_bytes = 0;   // bytes of the slot that cross PCIe

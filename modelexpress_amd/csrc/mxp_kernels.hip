@@ -39,6 +39,14 @@ struct Csum {
     Q += s0;
     P += i * s0;
   }
+  __device__ __forceinline__ void add8(uint32_t lo, uint32_t hi, uint32_t i) {
+    uint32_t s0 = __builtin_amdgcn_udot4(lo, 0x01010101u, 0u, false);
+    s0 = __builtin_amdgcn_udot4(hi, 0x01010101u, s0, false);
+    R = __builtin_amdgcn_udot4(lo, 0x03020100u, R, false);
+    R = __builtin_amdgcn_udot4(hi, 0x07060504u, R, false);
+    Q += s0;
+    P += i * s0;
+  }
   // Up to four bytes packed little-endian in x (missing bytes zero).
   __device__ __forceinline__ void add4(uint32_t x, uint32_t i) {
     uint32_t s0 = __builtin_amdgcn_udot4(x, 0x01010101u, 0u, false);
@@ -69,12 +77,10 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(uint32_t u, uint32_t nan_bi
   return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? nan_bits : r;
 }
 
-__device__ __forceinline__ uint4 cast8(const uint4& a, const uint4& b, uint32_t nan_bits) {
-  uint4 o;
+__device__ __forceinline__ uint2 cast4(const uint4& a, uint32_t nan_bits) {
+  uint2 o;
   o.x = f32_to_bf16_bits(a.x, nan_bits) | (f32_to_bf16_bits(a.y, nan_bits) << 16);
   o.y = f32_to_bf16_bits(a.z, nan_bits) | (f32_to_bf16_bits(a.w, nan_bits) << 16);
-  o.z = f32_to_bf16_bits(b.x, nan_bits) | (f32_to_bf16_bits(b.y, nan_bits) << 16);
-  o.w = f32_to_bf16_bits(b.z, nan_bits) | (f32_to_bf16_bits(b.w, nan_bits) << 16);
   return o;
 }
 
@@ -89,6 +95,12 @@ __device__ __forceinline__ void st16(uint8_t* p, const uint4& v) {
   u32x4 t;
   t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w;
   __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+}
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void st8(uint8_t* p, const uint2& v) {
+  u32x2 t;
+  t.x = v.x; t.y = v.y;
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x2*>(p));
 }
 
 // One tile of one segment.  UNIT = destination bytes handled per lane access.
@@ -111,7 +123,35 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
     d_o = row * dp + col * (uint32_t)UNIT;
   };
 
-  if constexpr (UNIT == 16) {
+  if constexpr (OP == kOpCastF32Bf16 && UNIT == 8) {
+    // Cast: a unit is four elements, one 16-byte load and one 8-byte store per lane, so a
+    // wavefront load covers 1 KiB of contiguous source and a store 512 B of contiguous
+    // destination.  Sixteen loads per lane are in flight before the first store.
+    constexpr int U = 2 * kPlaceBatch;
+    for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += (uint32_t)U * kPlaceThreads) {
+      uint32_t d_o[U];
+      uint4 a[U];
+      bool ok[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
+        ok[k] = v < n_units;
+        if (ok[k]) {
+          uint32_t so;
+          locate(v, so, d_o[k]);
+          a[k] = ld16(src + so);
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        if (ok[k]) {
+          const uint2 x = cast4(a[k], nan_bits);
+          st8(dst + d_o[k], x);
+          cs.add8(x.x, x.y, csum_base + d_o[k]);
+        }
+      }
+    }
+  } else if constexpr (UNIT == 16) {
     // One batch = kPlaceBatch units per lane: every load of the batch is issued before its
     // first store, so a workgroup presents the memory system with a burst of reads over
     // one contiguous region followed by a burst of writes over another.  With the default
@@ -122,32 +162,14 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
       uint32_t d_o[U];
       uint4 x[U];
       bool ok[U];
-      if constexpr (OP == kOpCastF32Bf16) {
-        uint4 a[U], b[U];
 #pragma unroll
-        for (int k = 0; k < U; ++k) {
-          const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
-          ok[k] = v < n_units;
-          if (ok[k]) {
-            uint32_t so;
-            locate(v, so, d_o[k]);
-            a[k] = ld16(src + so);
-            b[k] = ld16(src + so + 16);
-          }
-        }
-#pragma unroll
-        for (int k = 0; k < U; ++k)
-          if (ok[k]) x[k] = cast8(a[k], b[k], nan_bits);
-      } else {
-#pragma unroll
-        for (int k = 0; k < U; ++k) {
-          const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
-          ok[k] = v < n_units;
-          if (ok[k]) {
-            uint32_t so;
-            locate(v, so, d_o[k]);
-            x[k] = ld16(src + so);
-          }
+      for (int k = 0; k < U; ++k) {
+        const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
+        ok[k] = v < n_units;
+        if (ok[k]) {
+          uint32_t so;
+          locate(v, so, d_o[k]);
+          x[k] = ld16(src + so);
         }
       }
 #pragma unroll
@@ -164,7 +186,7 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
       locate(v, so, d_o);
       uint32_t x;
       if constexpr (OP == kOpCastF32Bf16) {
-        static_assert(UNIT == 2 || UNIT == 16, "cast moves one or eight elements per lane");
+        static_assert(UNIT == 2, "the element-wise cast path moves one element per lane");
         x = f32_to_bf16_bits(*reinterpret_cast<const uint32_t*>(src + so), nan_bits);
         *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
       } else if constexpr (UNIT == 4) {
@@ -201,7 +223,7 @@ __global__ __launch_bounds__(kPlaceThreads) void place_kernel(
     case kOpCopy * 32u + 16u: run_tile<kOpCopy, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCopy * 32u + 4u: run_tile<kOpCopy, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCopy * 32u + 1u: run_tile<kOpCopy, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
-    case kOpCastF32Bf16 * 32u + 16u: run_tile<kOpCastF32Bf16, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF32Bf16 * 32u + 8u: run_tile<kOpCastF32Bf16, 8>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF32Bf16 * 32u + 2u: run_tile<kOpCastF32Bf16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 4u: run_tile<kOpChecksumOnly, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;

@@ -45,7 +45,7 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
   };
   uint32_t unit;
   if (b.op == kOpCastF32Bf16) {
-    if (all_mult(16, 16)) unit = 16;
+    if (all_mult(8, 16)) unit = 8;
     else if (all_mult(2, 4)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
   } else {

@@ -191,10 +191,12 @@ class PlacementEngine:
     """Device-side executor: pinned ring + streams + kernels of one GPU."""
 
     def __init__(self, device: int = 0, *, ring_slots: int = 0, slot_bytes: int = 0, reader_threads: int = 0,
-                 streams: int = 0, tile_bytes: int = 0, nan_bits: int = 0, use_o_direct: bool = False):
+                 streams: int = 0, tile_bytes: int = 0, nan_bits: int = 0, use_o_direct: bool = False,
+                 pack_strided_on_host: bool | None = None):
+        pack = 0 if pack_strided_on_host is None else (1 if pack_strided_on_host else 2)
         opts = L.EngineOptions(device=device, ring_slots=ring_slots, slot_bytes=slot_bytes,
                                reader_threads=reader_threads, streams=streams, tile_bytes=tile_bytes,
-                               nan_bits=nan_bits, use_o_direct=int(use_o_direct))
+                               nan_bits=nan_bits, pack_strided_on_host=pack, use_o_direct=int(use_o_direct))
         self._h = C.c_void_p()
         L.check(L.lib().mxp_engine_create(C.byref(opts), C.byref(self._h)))
         self.device = device

@@ -54,3 +54,18 @@ def gpu_engine(mxp):
     eng = PlacementEngine(0, ring_slots=4, slot_bytes=1 << 20, reader_threads=4, streams=2)
     yield eng
     eng.close()
+
+
+@pytest.fixture(scope="session")
+def gpu_engine_band(mxp):
+    """Engine that stages whole row bands for strided slices (device gather) and uses slots
+    small enough that tensors are split across several chunks."""
+    import torch
+
+    if not torch.cuda.is_available():
+        pytest.fail("a gpu-marked test ran without a GPU; the HIP path has no fallback")
+    from modelexpress_amd.engine import PlacementEngine
+
+    eng = PlacementEngine(0, ring_slots=3, slot_bytes=1 << 16, reader_threads=3, streams=2, pack_strided_on_host=False)
+    yield eng
+    eng.close()

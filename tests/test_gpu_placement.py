@@ -16,7 +16,7 @@ def _stage_files(ck):
 
 
 @pytest.mark.parametrize("name", list(tiny_layouts()))
-def test_families_match_oracle(name, gpu_engine, oracle, tmp_path):
+def test_families_match_oracle(name, gpu_engine, gpu_engine_band, oracle, tmp_path):
     layout, tp, ep, shards, ck_kw = tiny_layouts()[name]
     cast = ck_kw.get("dtype") == "F32"
     synth.write_checkpoint(layout.checkpoint(**ck_kw), str(tmp_path), n_shards=shards, seed=7)
@@ -26,14 +26,17 @@ def test_families_match_oracle(name, gpu_engine, oracle, tmp_path):
                               param_dtype="BF16" if cast else None)
         want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
         ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
-        for mode in ("ingest", "resident"):
-            dst = gpu_engine.allocate(plan, fill=0xAB)
-            if mode == "ingest":
-                stats = gpu_engine.execute(plan, dst)
-                assert stats["placed_bytes"] == sum(p.nbytes for p in plan.params)
+        for mode in ("ingest", "ingest_band", "resident"):
+            eng = gpu_engine_band if mode == "ingest_band" else gpu_engine
+            dst = eng.allocate(plan, fill=0xAB)
+            if mode == "resident":
+                eng.execute_resident(plan, _stage_files(ck), dst)
             else:
-                gpu_engine.execute_resident(plan, _stage_files(ck), dst)
-            sums = gpu_engine.checksums(plan)
+                stats = eng.execute(plan, dst)
+                assert stats["placed_bytes"] == sum(p.nbytes for p in plan.params)
+                if mode == "ingest":  # packed on the host: nothing but placed bytes (times the cast factor) is read
+                    assert stats["file_bytes"] == sum(p.nbytes for p in plan.params) * (2 if cast else 1)
+            sums = eng.checksums(plan)
             for p, d, s in zip(plan.params, dst, sums):
                 assert d.cpu().numpy().tobytes() == want[p.name].tobytes(), (name, mode, tp_rank, p.name)
                 assert s == oracle.safe_checksum(want[p.name]), (name, mode, tp_rank, p.name)
