@@ -277,6 +277,12 @@ int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n
 int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* dst,
                  uint64_t dst_pitch, uint64_t rows, uint64_t row_bytes, uint32_t* checksum,
                  void* stream);
+/* n independent contiguous device copies in one launch, with the checksum of each
+ * destination in out_checksums[k] when not NULL: the device form of the batched
+ * torch._foreach_copy_ install (refit/reshard/receiver.py:939-955).  Destinations must
+ * be 16-byte aligned and must not overlap each other. */
+int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dsts, const uint64_t* nbytes,
+                   int64_t n, uint32_t* out_checksums, void* stream);
 /* Measured pinned host -> device bandwidth of this box in bytes per second
  * (hipMemcpyAsync of `bytes` from a pinned buffer, best of `repeats`). */
 int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double* bytes_per_second);

@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
@@ -731,6 +732,45 @@ int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* 
     uint32_t sum = 0;
     run_boxes(*engine, {b}, {sb}, {dst}, 1, checksum ? &sum : nullptr, static_cast<hipStream_t>(stream));
     if (checksum) *checksum = sum;
+  });
+}
+
+int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dsts, const uint64_t* nbytes, int64_t n,
+                   uint32_t* out_checksums, void* stream) {
+  return guard([&] {
+    if (!engine || n < 0 || (n && (!srcs || !dsts || !nbytes))) throw Error(MXP_ERR_ARG, "mxp_copy_batch: bad argument");
+    if (n == 0) return;
+    HIP_OK(hipSetDevice(engine->opt.device));
+    std::vector<BoxCopy> boxes;
+    std::vector<const void*> sv;
+    std::vector<void*> dv;
+    std::vector<std::pair<uintptr_t, uintptr_t>> spans;
+    for (int64_t k = 0; k < n; ++k) {
+      if (nbytes[k] && (!srcs[k] || !dsts[k])) throw Error(MXP_ERR_ARG, "mxp_copy_batch: null pointer");
+      if (reinterpret_cast<uintptr_t>(dsts[k]) & 15u) throw Error(MXP_ERR_ARG, "mxp_copy_batch: dst must be 16-byte aligned");
+      const void* sb;
+      uint64_t so;
+      split_ptr(srcs[k], sb, so);
+      sv.push_back(sb);
+      dv.push_back(dsts[k]);
+      BoxCopy b;
+      b.src_buf = (uint32_t)k;
+      b.dst_buf = (uint32_t)k;
+      b.src_off = so;
+      b.row_bytes = nbytes[k];
+      b.op = kOpCopy;
+      b.csum_slot = (uint32_t)k;
+      boxes.push_back(b);
+      if (nbytes[k]) spans.emplace_back(reinterpret_cast<uintptr_t>(dsts[k]), reinterpret_cast<uintptr_t>(dsts[k]) + nbytes[k]);
+    }
+    // One launch gives no ordering between copies: overlapping destinations are refused
+    // (the reference serialises them in plan order instead, receiver.py:289-321).
+    std::sort(spans.begin(), spans.end());
+    for (size_t i = 1; i < spans.size(); ++i)
+      if (spans[i].first < spans[i - 1].second) throw Error(MXP_ERR_ARG, "mxp_copy_batch: destinations overlap");
+    std::vector<uint32_t> sums((size_t)n, 0);
+    run_boxes(*engine, boxes, sv, dv, (uint32_t)n, out_checksums ? sums.data() : nullptr, static_cast<hipStream_t>(stream));
+    if (out_checksums) std::memcpy(out_checksums, sums.data(), (size_t)n * 4);
   });
 }
 

@@ -292,6 +292,17 @@ class PlacementEngine:
                                      rows, row_bytes, C.byref(out) if checksum else None, C.c_void_p(stream)))
         return format(out.value, "08x") if checksum else None
 
+    def copy_batch(self, srcs: Sequence, dsts: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
+                   checksums: bool = True) -> list[str] | None:
+        """n contiguous device copies in one launch (optionally with destination checksums)."""
+        n = len(srcs)
+        sizes = [_nbytes(t) for t in dsts] if nbytes is None else list(nbytes)
+        out = (C.c_uint32 * max(1, n))()
+        L.check(L.lib().mxp_copy_batch(self._h, _ptr_array([_addr(t) for t in srcs]),
+                                       _ptr_array([_addr(t) for t in dsts]), (C.c_uint64 * max(1, n))(*sizes), n,
+                                       out if checksums else None, C.c_void_p(stream)))
+        return [format(out[i], "08x") for i in range(n)] if checksums else None
+
     def measure_h2d(self, nbytes: int = 256 << 20, repeats: int = 5) -> float:
         out = C.c_double()
         L.check(L.lib().mxp_measure_h2d(self._h, nbytes, repeats, C.byref(out)))

@@ -1,0 +1,133 @@
+"""Refit of resident parameters from a new checkpoint version (plan -> stage -> apply).
+
+Mirrors the shape of the reference's generator-engine refit boundary
+(modelexpress_rl/inference/adapter.py:59-93: ``create_transfer_plan`` /
+``validate_transfer_plan`` / ``stage_weight`` -- transfer and verify with the live weights
+untouched -- / ``apply_weight`` / ``release_staged_weight`` / ``close``) for a source that
+is a safetensors checkpoint on local storage instead of a set of RDMA publishers:
+
+* plan: the placement plan of the resident layout against the new checkpoint; an fp32
+  checkpoint into bf16 parameters plans the round-to-nearest-even cast
+  (refit/reshard/transfer_plan.py:49-61: dtype mismatch -> staged, then converted);
+* stage: ingest + slice + cast into staging buffers, then recompute the per-parameter
+  ``tensor_digest`` on the device and compare it with the digests the publisher stamped
+  (modelexpress_rl/inference/nixl_staged_transfer.py:529-549): a mismatch, or a digest that
+  is required but missing, raises and leaves the live weights as they were;
+* apply: one batched device copy of staging into the live parameters, with the
+  checksums of what was installed.
+
+``in_place=True`` skips the staging copy (stage writes the live parameters directly):
+that waives the "untouched until verified" guarantee and is therefore explicit.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any
+
+import torch
+
+from .adapter import PlacementLayout
+from .engine import Checkpoint, PlacementEngine, PlacementPlan
+
+
+@dataclass(frozen=True)
+class RefitInputs:
+    """One version to install: where it is and what it must digest to."""
+
+    version_id: str
+    checkpoint_path: str
+    layout_signature: str = ""
+    expected_digests: dict = field(default_factory=dict)  # parameter name -> 32 hex chars
+    require_digests: bool = False
+
+    @property
+    def physical_fingerprint(self) -> tuple:
+        """The assumptions whose drift invalidates a cached plan (adapter.py:40-56)."""
+        return (self.layout_signature, self.checkpoint_path)
+
+
+@dataclass
+class RefitPlan:
+    inputs: RefitInputs
+    ckpt: Checkpoint
+    plan: PlacementPlan
+    fingerprint: tuple
+
+
+@dataclass
+class StagedWeights:
+    plan: RefitPlan
+    buffers: list  # staging tensors, or the live parameters when in_place
+    checksums: list
+    digests: list
+    stats: dict
+    in_place: bool
+
+
+class HipRefitAdapter:
+    """Refit executor for one rank's resident parameters."""
+
+    supported_payload_formats = frozenset({"safetensors"})
+
+    def __init__(self, layout: PlacementLayout, *, device: int = 0, engine: PlacementEngine | None = None,
+                 in_place: bool = False):
+        self.layout = layout
+        self.device = device
+        self.in_place = in_place
+        self._own_engine = engine is None
+        self.engine = engine or PlacementEngine(device)
+
+    def create_transfer_plan(self, inputs: RefitInputs) -> RefitPlan:
+        ck = Checkpoint(inputs.checkpoint_path)
+        lay = self.layout
+        plan = PlacementPlan(ck, lay.params, tp_size=lay.tp_size, tp_rank=lay.tp_rank,
+                             stacked_params_mapping=lay.stacked_params_mapping, expert_mapping=lay.expert_mapping,
+                             skip_prefixes=lay.skip_prefixes, allow_cast=True)
+        return RefitPlan(inputs, ck, plan, inputs.physical_fingerprint)
+
+    def validate_transfer_plan(self, plan: Any, inputs: RefitInputs) -> bool:
+        return isinstance(plan, RefitPlan) and plan.fingerprint == inputs.physical_fingerprint
+
+    def stage_weight(self, plan: RefitPlan) -> StagedWeights:
+        eng = self.engine
+        buffers = list(self.layout.destinations) if self.in_place else eng.allocate(plan.plan)
+        stats = eng.execute(plan.plan, buffers)
+        sums = eng.checksums(plan.plan)
+        sizes = [p.nbytes for p in plan.plan.params]
+        digests = eng.digest(buffers, sizes)
+        staged = StagedWeights(plan, buffers, sums, digests, stats, self.in_place)
+        self._verify(staged)
+        return staged
+
+    def _verify(self, staged: StagedWeights) -> None:
+        inputs = staged.plan.inputs
+        names = [p.name for p in staged.plan.plan.params]
+        for name, got in zip(names, staged.digests):
+            want = inputs.expected_digests.get(name)
+            if want is None:
+                if inputs.require_digests:
+                    raise RuntimeError(f"refit {inputs.version_id}: no published digest for {name}; refusing to install")
+                continue
+            if want != got:
+                raise RuntimeError(f"refit {inputs.version_id}: digest mismatch for {name}: "
+                                   f"published {want}, staged {got}")
+
+    def apply_weight(self, staged: StagedWeights) -> dict:
+        names = [p.name for p in staged.plan.plan.params]
+        if staged.in_place:
+            return dict(zip(names, staged.checksums))
+        sizes = [p.nbytes for p in staged.plan.plan.params]
+        sums = self.engine.copy_batch(staged.buffers, list(self.layout.destinations), sizes)
+        torch.cuda.synchronize(self.device)
+        if sums != staged.checksums:
+            raise RuntimeError(f"refit {staged.plan.inputs.version_id}: installed bytes differ from the staged ones")
+        return dict(zip(names, sums))
+
+    def release_staged_weight(self, staged: StagedWeights) -> None:
+        if not staged.in_place:
+            staged.buffers.clear()
+
+    def close(self) -> None:
+        if self._own_engine:
+            self.engine.close()

@@ -1,0 +1,83 @@
+"""Full-size checks (BASELINE configuration 2: Llama-3-8B, one TP=8 rank slice, 16 GB
+staged in HBM) through properties that do not need the oracle to process 16 GB:
+
+* the checkpoint is generated on the device by the seeded generator, which produces the
+  same bytes as the host generator, so any single tensor can be regenerated on the host
+  and pushed through the CPU oracle's slice rule;
+* the checksum accumulated inside the placement kernel must equal the stand-alone
+  checksum of the finished buffer (a second, independent device pass) for all 195
+  buffers, and the oracle's checksum for the regenerated ones;
+* placing twice gives identical bytes (no dependence on what the buffers held).
+"""
+
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+from modelexpress_amd import _lib as L
+from modelexpress_amd import models, synth
+from modelexpress_amd.engine import Checkpoint, PlacementEngine, PlacementPlan
+
+pytestmark = pytest.mark.gpu
+
+SEED = 77
+TP, RANK = 8, 5
+
+
+def _host_tensor(spec, seed) -> np.ndarray:
+    n = spec.nbytes // L.DTYPE_SIZE[spec.dtype]
+    buf = np.empty(spec.nbytes, dtype=np.uint8)
+    L.check(L.lib().mxp_synth_host(C.c_void_p(buf.ctypes.data), n, L.DTYPE_CODE[spec.dtype], spec.kind,
+                                   synth.tensor_seed(seed, spec.name), 8))
+    return buf.reshape(tuple(spec.shape) + (L.DTYPE_SIZE[spec.dtype],))
+
+
+def test_llama3_8b_rank_slice_full_size(oracle, oracle_c, tmp_path, mxp):
+    layout = models.Llama()
+    tensors = layout.checkpoint()
+    by_name = {t.name: t for t in tensors}
+    synth.write_headers_only(tensors, str(tmp_path), n_shards=4)
+    ck = Checkpoint(str(tmp_path))
+    assert len(ck) == 291 and sum(t.nbytes for t in ck.tensors()) == 16_060_522_496
+    rv = layout.rank_view(tp_size=TP, tp_rank=RANK)
+    plan = PlacementPlan(ck, rv.params, tp_size=TP, tp_rank=RANK, stacked_params_mapping=rv.stacked_params_mapping)
+    assert len(plan.params) == 195 and plan.totals()["placed_bytes"] == 2_008_031_232
+    eng = PlacementEngine(0)
+    staged = synth.stage_on_device(ck, tensors, seed=SEED)
+    dst = eng.allocate(plan, fill=0x5A)
+    eng.execute_resident(plan, staged, dst)
+    fused = eng.checksums(plan)
+    alone = eng.checksum32(dst)
+    assert fused == alone  # 195 buffers, two independent device passes
+
+    # regenerate single tensors on the host and apply the oracle's slice rule
+    OT = oracle.OTensor
+    m = oracle.MdlOracle({}, tp_size=TP, tp_rank=RANK)
+    idx = {p.name: i for i, p in enumerate(plan.params)}
+    layer = "model.layers.17."
+    q, k, v = (OT(_host_tensor(by_name[layer + f"self_attn.{x}_proj.weight"], SEED), "BF16") for x in "qkv")
+    qkv_shape = plan.params[idx[layer + "self_attn.qkv_proj.weight"]].shape
+    parts = [m.tp_local_tensor(t, (t.shape[0] // TP, t.shape[1])) for t in (q, k, v)]
+    want_qkv = np.concatenate([np.ascontiguousarray(p.data) for p in parts])
+    assert want_qkv.shape[:2] == tuple(qkv_shape)
+    checks = {layer + "self_attn.qkv_proj.weight": want_qkv}
+    o = OT(_host_tensor(by_name[layer + "self_attn.o_proj.weight"], SEED), "BF16")
+    checks[layer + "self_attn.o_proj.weight"] = np.ascontiguousarray(m.tp_local_tensor(o, (4096, 512)).data)
+    d = OT(_host_tensor(by_name[layer + "mlp.down_proj.weight"], SEED), "BF16")
+    checks[layer + "mlp.down_proj.weight"] = np.ascontiguousarray(m.tp_local_tensor(d, (4096, 1792)).data)
+    n = OT(_host_tensor(by_name["model.norm.weight"], SEED), "BF16")
+    checks["model.norm.weight"] = np.ascontiguousarray(n.data)
+    for name, want in checks.items():
+        got = dst[idx[name]].cpu().numpy()
+        assert got.tobytes() == want.tobytes(), name
+        assert fused[idx[name]] == oracle_c.checksum32(want), name
+    assert fused[idx["model.norm.weight"]] == oracle.safe_checksum_bytes(checks["model.norm.weight"])
+
+    # idempotence: a second placement over the finished buffers changes nothing
+    before = [t.clone() for t in dst[:8]]
+    eng.execute_resident(plan, staged, dst)
+    assert eng.checksums(plan) == fused
+    assert all(torch.equal(a, b) for a, b in zip(before, dst[:8]))
+    eng.close()

@@ -1,0 +1,210 @@
+"""The strategy chain, the iterator-shaped path and the refit flow on a real GPU."""
+
+import os
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+from torch import nn
+
+from helpers import oracle_place
+from modelexpress_amd import models, synth
+from modelexpress_amd.adapter import EngineAdapter, StrategyFailed
+from modelexpress_amd.load_strategy import (HipPlacementStrategy, LoadContext, LoadResult, LoadStrategyChain,
+                                            iter_checkpoint_tensors, layout_from_module)
+from modelexpress_amd.refit import HipRefitAdapter, RefitInputs
+
+pytestmark = pytest.mark.gpu
+
+LAYOUT = models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256)
+TP, RANK = 4, 1
+
+
+class ToyModel(nn.Module):
+    """A module whose parameters are exactly one rank's table (what an engine allocates)."""
+
+    stacked_params_mapping = [("qkv_proj", "q_proj"), ("qkv_proj", "k_proj"), ("qkv_proj", "v_proj"),
+                              ("gate_up_proj", "gate_proj"), ("gate_up_proj", "up_proj")]
+
+    def __init__(self, rv, device="cuda"):
+        super().__init__()
+        self._names = []
+        for p in rv.params:
+            key = p.name.replace(".", "__")
+            self.register_parameter(key, nn.Parameter(torch.zeros(p.shape, dtype=torch.bfloat16, device=device),
+                                                      requires_grad=False))
+            self._names.append((key, p.name))
+
+    def named_parameters(self, *a, **k):
+        for key, name in self._names:
+            yield name, getattr(self, key)
+
+
+class ToyAdapter(EngineAdapter):
+    def __init__(self, rv):
+        self.rv = rv
+        self.reinit_calls = 0
+        self.native_calls = 0
+
+    def get_device_id(self):
+        return 0
+
+    def placement_layout(self, result):
+        return layout_from_module(result.model, tp_size=TP, tp_rank=RANK)
+
+    def reinit_for_retry(self, result):
+        self.reinit_calls += 1
+        fresh = ToyModel(self.rv)
+        return LoadResult(value=fresh, model=fresh)
+
+    def load_via_native(self, result):
+        self.native_calls += 1
+        return result
+
+
+def _ctx(adapter, path):
+    return LoadContext(model_config=SimpleNamespace(model=path), adapter=adapter)
+
+
+def test_chain_places_into_param_data(oracle, tmp_path, monkeypatch, mxp):
+    synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=2, seed=21)
+    rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
+    want = oracle_place(oracle, str(tmp_path), rv, tp_size=TP, tp_rank=RANK)
+    monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
+    model = ToyModel(rv)
+    ptrs = {n: p.data_ptr() for n, p in model.named_parameters()}
+    ad = ToyAdapter(rv)
+    ctx = _ctx(ad, str(tmp_path))
+    out = LoadStrategyChain.run(model, ctx)
+    assert out is model and ad.reinit_calls == 0 and ad.native_calls == 0
+    for name, p in model.named_parameters():
+        assert p.data_ptr() == ptrs[name]  # written in place, never replaced
+        assert p.data.view(torch.uint8).cpu().numpy().tobytes() == want[name].tobytes(), name
+    assert set(ctx.tensors) == set(want)
+
+
+def test_truncated_shard_is_a_mutated_failure_and_the_chain_recovers(tmp_path, monkeypatch, mxp):
+    info = synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=2, seed=22)
+    rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
+    monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
+    monkeypatch.setenv("MXP_SLOT_MIB", "1")
+    model = ToyModel(rv)
+    ad = ToyAdapter(rv)
+    st = HipPlacementStrategy()
+
+    # Plan against intact files, then cut the last shard: the failure happens mid-ingest.
+    class LateTruncation(HipPlacementStrategy):
+        def load(self, result, ctx):
+            orig = self.__class__.__mro__[1].load
+
+            def cut(*_a, **_k):
+                pass
+
+            import modelexpress_amd.engine as E
+
+            real_execute = E.PlacementEngine.execute
+
+            def execute(eng, plan, dst):
+                size = os.path.getsize(info["files"][-1])
+                with open(info["files"][-1], "r+b") as f:
+                    f.truncate(size // 2)
+                return real_execute(eng, plan, dst)
+
+            monkeypatch.setattr(E.PlacementEngine, "execute", execute)
+            try:
+                return orig(self, result, ctx)
+            finally:
+                monkeypatch.setattr(E.PlacementEngine, "execute", real_execute)
+
+    with pytest.raises(StrategyFailed) as e:
+        LateTruncation().load(LoadResult(value=model, model=model), _ctx(ad, str(tmp_path)))
+    assert "MXP_ERR_IO" in str(e.value)
+    # through the chain: rollback, re-initialise if bytes moved, then the native loader
+    synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=2, seed=22)
+    model2 = ToyModel(rv)
+    out = LoadStrategyChain.run(model2, _ctx(ad, str(tmp_path)), [LateTruncation(), *LoadStrategyChain.default_strategies()[2:]])
+    assert ad.native_calls == 1
+    assert (out is not model2) == (ad.reinit_calls == 1)
+    assert st.name == "hip_placement"
+
+
+def test_bad_checkpoint_is_a_clean_miss(tmp_path, monkeypatch, mxp):
+    (tmp_path / "model.safetensors").write_bytes(b"\x05\x00\x00\x00\x00\x00\x00\x00{nope")
+    rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
+    monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
+    model = ToyModel(rv)
+    with pytest.raises(StrategyFailed) as e:
+        HipPlacementStrategy().load(LoadResult(value=model, model=model), _ctx(ToyAdapter(rv), str(tmp_path)))
+    assert e.value.mutated is False
+    assert all(int(p.data.view(torch.uint8).sum()) == 0 for _n, p in model.named_parameters())
+
+
+def test_iter_checkpoint_tensors_matches_oracle(oracle, tmp_path, mxp):
+    synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=3, seed=23)
+    want = dict(oracle.load_checkpoint(str(tmp_path)))
+    seen = []
+    for name, t in iter_checkpoint_tensors(str(tmp_path)):
+        assert t.is_cuda and t.dtype == torch.bfloat16 and tuple(t.shape) == want[name].shape
+        assert t.contiguous().view(torch.uint8).cpu().numpy().tobytes() == want[name].tobytes(), name
+        seen.append(name)
+    assert seen == [n for n, _ in oracle.load_checkpoint(str(tmp_path))]
+
+
+def test_copy_batch_and_overlap_rule(gpu_engine, oracle_c, mxp):
+    rng = np.random.default_rng(30)
+    sizes = [0, 16, 100, 4096, 65536 + 48, 1 << 20]
+    srcs = [torch.from_numpy(rng.integers(0, 256, max(n, 1), dtype=np.uint8)).cuda()[:n] for n in sizes]
+    dsts = [torch.zeros(max(n, 16), dtype=torch.uint8, device="cuda") for n in sizes]
+    sums = gpu_engine.copy_batch(srcs, dsts, sizes)
+    for s, d, n, c in zip(srcs, dsts, sizes, sums):
+        assert torch.equal(d[:n], s)
+        assert c == oracle_c.checksum32(s.cpu().numpy())
+    big = torch.zeros(4096, dtype=torch.uint8, device="cuda")
+    with pytest.raises(mxp.MxpError, match="overlap"):  # receiver.py:289-321: only disjoint copies are batched
+        gpu_engine.copy_batch([srcs[3], srcs[3]], [big, big[16:]], [4096 - 16, 4096 - 16])
+
+
+def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
+    # config 3 in miniature: resident bf16 rank slice, new fp32 checkpoint with edge cases
+    base, new = tmp_path / "v0", tmp_path / "v1"
+    synth.write_checkpoint(LAYOUT.checkpoint(), str(base), n_shards=2, seed=24)
+    synth.write_checkpoint(LAYOUT.checkpoint(dtype="F32", edge_cases=models.NORMAL_EDGE_DENSE), str(new), n_shards=3, seed=25)
+    rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
+    model = ToyModel(rv)
+    layout = layout_from_module(model, tp_size=TP, tp_rank=RANK)
+    os.environ["MX_MODEL_URI"] = str(base)
+    try:
+        LoadStrategyChain.run(model, _ctx(ToyAdapter(rv), str(base)))
+    finally:
+        del os.environ["MX_MODEL_URI"]
+    v0 = {n: p.data.view(torch.uint8).cpu().numpy().tobytes() for n, p in model.named_parameters()}
+    want = oracle_place(oracle, str(new), rv, tp_size=TP, tp_rank=RANK, allow_cast=True)
+    digests = {n: oracle.tensor_digest(t) for n, t in want.items()}
+
+    ad = HipRefitAdapter(layout)
+    # a wrong published digest: nothing is installed
+    bad = dict(digests)
+    first = next(iter(bad))
+    bad[first] = "0" * 32
+    plan = ad.create_transfer_plan(RefitInputs("v1", str(new), "sig", bad, require_digests=True))
+    with pytest.raises(RuntimeError, match="digest mismatch"):  # nixl_staged_transfer.py:529-549
+        ad.stage_weight(plan)
+    assert {n: p.data.view(torch.uint8).cpu().numpy().tobytes() for n, p in model.named_parameters()} == v0
+    # a missing digest when they are required
+    plan = ad.create_transfer_plan(RefitInputs("v1", str(new), "sig", {}, require_digests=True))
+    with pytest.raises(RuntimeError, match="no published digest"):
+        ad.stage_weight(plan)
+    # the good path
+    inputs = RefitInputs("v1", str(new), "sig", digests, require_digests=True)
+    plan = ad.create_transfer_plan(inputs)
+    assert ad.validate_transfer_plan(plan, inputs)
+    assert not ad.validate_transfer_plan(plan, RefitInputs("v2", str(new), "other-layout", digests))
+    staged = ad.stage_weight(plan)
+    assert {n: p.data.view(torch.uint8).cpu().numpy().tobytes() for n, p in model.named_parameters()} == v0
+    sums = ad.apply_weight(staged)
+    for n, p in model.named_parameters():
+        assert p.data.view(torch.uint8).cpu().numpy().tobytes() == want[n].tobytes(), n
+        assert sums[n] == oracle.safe_checksum(want[n])
+    ad.release_staged_weight(staged)
+    ad.close()

@@ -1,0 +1,184 @@
+"""Chain and strategy semantics on the host, restating the assertions of the reference's
+tests/test_model_streamer_strategy.py (cited per test) against this package's classes."""
+
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from modelexpress_amd import envs
+from modelexpress_amd.adapter import EngineAdapter, StrategyFailed, UnsupportedCapability, gated_capability
+from modelexpress_amd.accelerators import HipAcceleratorBackend, accelerator_backend_for
+from modelexpress_amd.load_strategy import (DefaultStrategy, HipPlacementStrategy, HipStreamerStrategy, LoadContext,
+                                            LoadResult, LoadStrategy, LoadStrategyChain, _resolve_model_uri)
+
+
+class _Backend(HipAcceleratorBackend):
+    def supports_hip_placement(self) -> bool:
+        return True
+
+
+def _ctx(adapter=None, **cfg):
+    return LoadContext(model_config=SimpleNamespace(**cfg), adapter=adapter, accelerator_backend=_Backend())
+
+
+class _IterAdapter(EngineAdapter):
+    def __init__(self, fail_apply=False, fail_build=False):
+        self.fail_apply, self.fail_build = fail_apply, fail_build
+        self.applied, self.reinit_calls, self.after_calls = [], 0, 0
+
+    def apply_weight_iter(self, result, weights_iter):
+        for name, t in weights_iter:
+            self.applied.append(name)
+            if self.fail_apply:
+                raise RuntimeError("boom mid-stream")
+        return result
+
+    def build_model_streamer_weight_iter(self, model_uri, model=None):
+        if self.fail_build:
+            raise FileNotFoundError(model_uri)
+        yield "a", torch.zeros(1)
+        yield "b", torch.zeros(1)
+
+    def after_weight_iter_load(self, result):
+        self.after_calls += 1
+        return result
+
+    def reinit_for_retry(self, result):
+        self.reinit_calls += 1
+        return LoadResult(value="fresh-model", model=None)
+
+    def load_via_native(self, result):
+        result.metadata["native"] = True
+        return result
+
+
+def test_gated_capability_identity_rule():
+    # adapter.py:37-51, base.py:53-60: eligible only when the concrete class overrides
+    assert HipStreamerStrategy().is_available(_ctx(EngineAdapter())) is False
+    assert getattr(EngineAdapter.apply_weight_iter, "__gated_capability__", False)
+    with pytest.raises(UnsupportedCapability):
+        EngineAdapter().placement_layout(None)
+    assert HipStreamerStrategy().is_available(_ctx(None)) is False
+
+
+def test_streamer_requires_uri(monkeypatch):
+    # test_model_streamer_strategy.py:145-226
+    monkeypatch.delenv("MX_MODEL_URI", raising=False)
+    assert HipStreamerStrategy().is_available(_ctx(_IterAdapter())) is False
+    monkeypatch.setenv("MX_MODEL_URI", "/models/x")
+    assert HipStreamerStrategy().is_available(_ctx(_IterAdapter())) is True
+    assert envs.MX_MODEL_URI == "/models/x"  # live read
+
+
+def test_uri_resolution_order(monkeypatch):
+    # model_streamer_strategy.py:27-35: env -> model_weights -> model -> model_path
+    monkeypatch.setenv("MX_MODEL_URI", "/env")
+    assert _resolve_model_uri(_ctx(model_weights="/w", model="/m", model_path="/p")) == "/env"
+    monkeypatch.delenv("MX_MODEL_URI")
+    assert _resolve_model_uri(_ctx(model_weights="/w", model="/m", model_path="/p")) == "/w"
+    assert _resolve_model_uri(_ctx(model_weights=None, model="/m", model_path="/p")) == "/m"
+    assert _resolve_model_uri(_ctx(model_path="/p")) == "/p"
+    assert _resolve_model_uri(_ctx()) == ""
+
+
+def test_streamer_mutated_flags(monkeypatch):
+    # test_model_streamer_strategy.py:228-283
+    monkeypatch.setenv("MX_MODEL_URI", "/models/x")
+    ok = _IterAdapter()
+    out = HipStreamerStrategy().load(LoadResult(value="m"), _ctx(ok))
+    assert ok.applied == ["a", "b"] and ok.after_calls == 1 and out.value == "m"
+    with pytest.raises(StrategyFailed) as e:
+        HipStreamerStrategy().load(LoadResult(value="m"), _ctx(_IterAdapter(fail_apply=True)))
+    assert e.value.mutated is True
+    # the iterator is lazy: a build failure surfaces inside apply and counts as mutated,
+    # exactly as in the reference where _stream_weights is a generator
+    with pytest.raises(StrategyFailed) as e:
+        HipStreamerStrategy().load(LoadResult(value="m"), _ctx(_IterAdapter(fail_build=True)))
+    assert e.value.mutated is True
+    monkeypatch.delenv("MX_MODEL_URI")
+    with pytest.raises(StrategyFailed) as e:
+        HipStreamerStrategy().load(LoadResult(value="m"), _ctx(_IterAdapter()))
+    assert e.value.mutated is False
+
+
+class _Scripted(LoadStrategy):
+    def __init__(self, name, behaviour, available=True):
+        self.name, self.behaviour, self.available = name, behaviour, available
+        self.rolled_back = 0
+
+    def is_available(self, ctx):
+        return self.available
+
+    def load(self, result, ctx):
+        if self.behaviour == "ok":
+            return result
+        if self.behaviour == "miss":
+            raise StrategyFailed("clean miss", mutated=False)
+        if self.behaviour == "dirty":
+            raise StrategyFailed("dirty", mutated=True)
+        raise ValueError("unexpected")
+
+    def rollback(self, ctx):
+        self.rolled_back += 1
+
+
+def test_chain_order_skip_rollback_and_reinit():
+    # test_model_streamer_strategy.py:405-502, load_strategy/__init__.py:79-117
+    ad = _IterAdapter()
+    s = [_Scripted("unavailable", "ok", available=False), _Scripted("miss", "miss"), _Scripted("boom", "raise"),
+         _Scripted("dirty", "dirty"), _Scripted("winner", "ok"), _Scripted("never", "ok")]
+    out = LoadStrategyChain.run("model", _ctx(ad), s)
+    assert out == "fresh-model"  # re-initialised after the dirty failure, then loaded by "winner"
+    assert [x.rolled_back for x in s] == [0, 1, 1, 1, 0, 0]
+    assert ad.reinit_calls == 1
+
+
+def test_chain_exhaustion_and_reinit_errors():
+    with pytest.raises(RuntimeError, match="No loading strategy succeeded"):
+        LoadStrategyChain.run("model", _ctx(_IterAdapter()), [_Scripted("miss", "miss")])
+    with pytest.raises(RuntimeError, match="no adapter can reinitialize"):
+        LoadStrategyChain.run("model", _ctx(None), [_Scripted("dirty", "dirty")])
+    with pytest.raises(RuntimeError, match="does not support retry"):
+        LoadStrategyChain.run("model", _ctx(EngineAdapter()), [_Scripted("dirty", "dirty")])
+
+
+def test_default_chain_falls_through_to_native(monkeypatch):
+    monkeypatch.delenv("MX_MODEL_URI", raising=False)
+    ad = _IterAdapter()
+    assert [s.name for s in LoadStrategyChain.default_strategies()] == ["hip_placement", "model_streamer", "default"]
+    assert LoadStrategyChain.run("model", _ctx(ad)) == "model"
+    assert DefaultStrategy().is_available(_ctx(EngineAdapter())) is False
+
+
+class _PlaceAdapter(_IterAdapter):
+    def placement_layout(self, result):
+        raise RuntimeError("layout unavailable")
+
+
+def test_hip_placement_availability_and_clean_miss(monkeypatch, tmp_path):
+    monkeypatch.delenv("MX_MODEL_URI", raising=False)
+    st = HipPlacementStrategy()
+    assert st.is_available(_ctx(_IterAdapter())) is False  # capability not overridden
+    assert st.is_available(_ctx(_PlaceAdapter())) is False  # no URI
+    monkeypatch.setenv("MX_MODEL_URI", "s3://bucket/model")
+    assert st.is_available(_ctx(_PlaceAdapter())) is False  # object stores are not this strategy's
+    monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
+    assert st.is_available(_ctx(_PlaceAdapter())) is True
+    ctx = _ctx(_PlaceAdapter())
+    ctx.accelerator_backend = HipAcceleratorBackend()
+    if not torch.cuda.is_available():
+        assert st.is_available(ctx) is False  # no device
+    with pytest.raises(StrategyFailed) as e:  # planning failures never count as mutated
+        st.load(LoadResult(value="m"), _ctx(_PlaceAdapter()))
+    assert e.value.mutated is False
+
+
+def test_accelerator_backend_selection():
+    # accelerators/__init__.py:41-61, base.py:16-72
+    b = accelerator_backend_for("cuda:0")
+    assert b.name == "rocm" and b.torch_device_type == "cuda" and b.nixl_mem_type == "VRAM"
+    assert not (b.supports_gds() or b.supports_vmm() or b.supports_pool_reg() or b.supports_rdma_p2p())
+    assert b.torch_device(1) == torch.device("cuda", 1)
+    with pytest.raises(ValueError, match="Unsupported accelerator backend"):
+        accelerator_backend_for("xpu:0")
