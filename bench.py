@@ -198,6 +198,24 @@ def main() -> int:
             "roofline": roofline,
         }
 
+        # ---- the read-only operators over the finished buffers (1 x bytes each) ----
+        sizes = [p.nbytes for p in plan.params]
+        if placed <= 8e9:
+            ops = {}
+            for op_name, fn in (("checksum32", lambda: eng.checksum32(dst, sizes)), ("tensor_digest", lambda: eng.digest(dst, sizes))):
+                fn()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                reps = 10
+                for _ in range(reps):
+                    res = fn()
+                dt = (time.perf_counter() - t0) / reps
+                ops[op_name] = {"buffers": len(dst), "bytes": placed, "ms_per_call_wall": round(dt * 1e3, 4),
+                                "gbps_wall": round(placed / dt / 1e9, 1),
+                                "note": "one batched launch; wall time includes descriptor upload, result copy and sync"}
+            ops["checksum32"]["matches_fused"] = eng.checksum32(dst, sizes) == resident_sums
+            out["ops"] = ops
+
         # ---- end-to-end ingest from files through the pinned ring ----
         agree = True
         if files_real and not args.no_e2e:

@@ -277,6 +277,26 @@ int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n
 int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* dst,
                  uint64_t dst_pitch, uint64_t rows, uint64_t row_bytes, uint32_t* checksum,
                  void* stream);
+/* One pitched box between two device addresses. */
+typedef struct mxp_box {
+  const void* src;
+  void* dst;           /* 16-byte aligned unless rows == 1 and the box is byte-granular */
+  uint64_t src_pitch;  /* bytes between rows in the source (ignored when rows == 1) */
+  uint64_t dst_pitch;
+  uint64_t rows;
+  uint64_t row_bytes;  /* destination bytes per row */
+  uint64_t csum_index; /* checksum position of the first destination byte */
+  uint32_t csum_group; /* which output checksum this box adds to, 0 .. n_groups-1 */
+  uint32_t cast;       /* 1: source is fp32, destination bf16 */
+} mxp_box;
+/* n boxes in one launch: the batched form of the staged re-slice of
+ * refit/reshard/receiver.py:919-960 (as_strided + copy_ per view) and of shard_region
+ * (refit/reshard/verify.py:158-183).  out_checksums[g], when not NULL, receives the sum of
+ * the position-weighted checksums of every box in group g (a whole buffer's checksum when
+ * its boxes tile it and csum_index is the offset inside the buffer).  Boxes must not
+ * overlap in the destination. */
+int mxp_place_boxes(mxp_engine* engine, const mxp_box* boxes, int64_t n, uint32_t n_groups,
+                    uint32_t* out_checksums, void* stream);
 /* n independent contiguous device copies in one launch, with the checksum of each
  * destination in out_checksums[k] when not NULL: the device form of the batched
  * torch._foreach_copy_ install (refit/reshard/receiver.py:939-955).  Destinations must

@@ -74,6 +74,12 @@ class ParamInfo(C.Structure):
                 ("n_writes", C.c_int32), ("reserved", C.c_int32)]
 
 
+class Box(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("src_pitch", C.c_uint64), ("dst_pitch", C.c_uint64),
+                ("rows", C.c_uint64), ("row_bytes", C.c_uint64), ("csum_index", C.c_uint64),
+                ("csum_group", C.c_uint32), ("cast", C.c_uint32)]
+
+
 class EngineOptions(C.Structure):
     _fields_ = [("device", C.c_int32), ("ring_slots", C.c_int32), ("slot_bytes", C.c_uint64),
                 ("reader_threads", C.c_int32), ("streams", C.c_int32), ("tile_bytes", C.c_uint32),
@@ -131,6 +137,7 @@ SIGNATURES = {
     "mxp_digest": (C.c_int, [_P, _PP, _U64P, C.c_int64, C.POINTER(C.c_uint8), _U64P, _P]),
     "mxp_cast_f32_bf16": (C.c_int, [_P, _P, _P, C.c_uint64, _U32P, _P]),
     "mxp_gather2d": (C.c_int, [_P, _P, C.c_uint64, _P, C.c_uint64, C.c_uint64, C.c_uint64, _U32P, _P]),
+    "mxp_place_boxes": (C.c_int, [_P, C.POINTER(Box), C.c_int64, C.c_uint32, _U32P, _P]),
     "mxp_copy_batch": (C.c_int, [_P, _PP, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_digest_from_scalars": (C.c_int, [_U64P, C.POINTER(C.c_uint8)]),

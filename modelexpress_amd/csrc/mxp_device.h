@@ -37,7 +37,8 @@ struct alignas(16) Seg {
   uint32_t csum_slot;  // index into the checksum accumulator array, ~0u = none
   uint32_t units_per_row;  // row_bytes / unit
   uint32_t div_magic;  // floor(2^32 / units_per_row) + 1, exact for n*d < 2^32
-  uint32_t pad0, pad1;
+  uint32_t csum_bias;  // added (mod 2^32) to the destination offset to get the checksum position
+  uint32_t pad1;
 };
 static_assert(sizeof(Seg) == 80, "Seg layout is part of the host<->device contract");
 

@@ -735,6 +735,55 @@ int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* 
   });
 }
 
+int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n_groups, uint32_t* out_checksums,
+                    void* stream) {
+  return guard([&] {
+    if (!engine || n < 0 || (n && !in) || (out_checksums && n_groups == 0))
+      throw Error(MXP_ERR_ARG, "mxp_place_boxes: bad argument");
+    if (n == 0) {
+      for (uint32_t g = 0; out_checksums && g < n_groups; ++g) out_checksums[g] = 0;
+      return;
+    }
+    HIP_OK(hipSetDevice(engine->opt.device));
+    std::vector<BoxCopy> boxes;
+    std::vector<const void*> sv;
+    std::vector<void*> dv;
+    for (int64_t k = 0; k < n; ++k) {
+      const mxp_box& x = in[k];
+      if (x.rows == 0 || x.row_bytes == 0) continue;
+      if (!x.src || !x.dst) throw Error(MXP_ERR_ARG, "mxp_place_boxes: null pointer");
+      if (x.csum_group >= (n_groups ? n_groups : 1)) throw Error(MXP_ERR_ARG, "mxp_place_boxes: csum_group out of range");
+      const uint64_t sm = x.cast ? 2 : 1;
+      if (x.rows > 1 && (x.src_pitch < x.row_bytes * sm || x.dst_pitch < x.row_bytes))
+        throw Error(MXP_ERR_ARG, "mxp_place_boxes: pitch smaller than the row");
+      const void* sb;
+      const void* db;
+      uint64_t so, d_o;
+      split_ptr(x.src, sb, so);
+      split_ptr(x.dst, db, d_o);
+      BoxCopy b;
+      b.src_buf = (uint32_t)sv.size();
+      b.dst_buf = (uint32_t)dv.size();
+      sv.push_back(sb);
+      dv.push_back(const_cast<void*>(db));
+      b.src_off = so;
+      b.dst_off = d_o;
+      b.src_pitch = x.src_pitch;
+      b.dst_pitch = x.dst_pitch;
+      b.rows = x.rows;
+      b.row_bytes = x.row_bytes;
+      b.op = x.cast ? kOpCastF32Bf16 : kOpCopy;
+      b.csum_slot = out_checksums ? x.csum_group : 0xFFFFFFFFu;
+      b.csum_bias = x.csum_index - d_o;  // positions are relative to the caller's buffer, not the aligned base
+      boxes.push_back(b);
+    }
+    std::vector<uint32_t> sums(n_groups ? n_groups : 1, 0);
+    run_boxes(*engine, boxes, sv, dv, n_groups ? n_groups : 1, out_checksums ? sums.data() : nullptr,
+              static_cast<hipStream_t>(stream));
+    if (out_checksums) std::memcpy(out_checksums, sums.data(), (size_t)n_groups * 4);
+  });
+}
+
 int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dsts, const uint64_t* nbytes, int64_t n,
                    uint32_t* out_checksums, void* stream) {
   return guard([&] {

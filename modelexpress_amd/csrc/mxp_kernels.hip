@@ -216,7 +216,7 @@ __global__ __launch_bounds__(kPlaceThreads) void place_kernel(
   if (s.op != kOpChecksumOnly)
     dst = static_cast<uint8_t*>(dst_bases[s.dst_buf]) + s.dst_off + (uint64_t)r0 * s.dst_pitch;
   // Checksum positions are taken mod 2^32, exactly as the weights are.
-  const uint32_t csum_base = (uint32_t)(s.dst_off + (uint64_t)r0 * s.dst_pitch);
+  const uint32_t csum_base = (uint32_t)(s.dst_off + (uint64_t)r0 * s.dst_pitch) + s.csum_bias;
 
   Csum cs;
   switch (s.op * 32u + s.unit) {

@@ -20,6 +20,7 @@ struct BoxCopy {
   uint64_t rows = 1, row_bytes = 0;
   uint32_t op = kOpCopy;
   uint32_t csum_slot = 0xFFFFFFFFu;
+  uint64_t csum_bias = 0;  // checksum position = destination offset + bias (mod 2^32)
 };
 
 struct LowerOptions {
@@ -66,6 +67,7 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
   s.op = b.op;
   s.unit = unit;
   s.csum_slot = b.csum_slot;
+  s.csum_bias = (uint32_t)b.csum_bias;
   s.units_per_row = s.row_bytes / unit;
   s.div_magic = s.units_per_row > 1 ? (uint32_t)((1ull << 32) / s.units_per_row) + 1u : 0u;
   uint64_t rpt = std::max<uint64_t>(1, o.tile_bytes / b.row_bytes);

@@ -292,6 +292,66 @@ class PlacementEngine:
                                      rows, row_bytes, C.byref(out) if checksum else None, C.c_void_p(stream)))
         return format(out.value, "08x") if checksum else None
 
+    def place_boxes(self, boxes: Sequence[dict], n_groups: int = 1, *, stream: int = 0,
+                    checksums: bool = True) -> list[str] | None:
+        """n pitched boxes in one launch.  Each box is a dict with ``src``, ``dst`` (tensors or
+        device addresses), ``rows``, ``row_bytes`` and optionally ``src_pitch``, ``dst_pitch``,
+        ``csum_index``, ``csum_group``, ``cast``."""
+        arr = (L.Box * max(1, len(boxes)))()
+        for i, b in enumerate(boxes):
+            arr[i] = L.Box(src=_addr(b["src"]), dst=_addr(b["dst"]), src_pitch=b.get("src_pitch", 0),
+                           dst_pitch=b.get("dst_pitch", 0), rows=b["rows"], row_bytes=b["row_bytes"],
+                           csum_index=b.get("csum_index", 0), csum_group=b.get("csum_group", 0),
+                           cast=int(b.get("cast", 0)))
+        out = (C.c_uint32 * max(1, n_groups))()
+        L.check(L.lib().mxp_place_boxes(self._h, arr, len(boxes), n_groups, out if checksums else None,
+                                        C.c_void_p(stream)))
+        return [format(out[i], "08x") for i in range(n_groups)] if checksums else None
+
+    def shard_region(self, full, global_shape: Sequence[int], shard_offset: Sequence[int], shape: Sequence[int],
+                     itemsize: int, out=None, *, stream: int = 0):
+        """The sub-box of an assembled full tensor that one publisher owns, as a contiguous
+        device buffer with its checksum (refit/reshard/verify.py:158-183).  ``full`` holds
+        the row-major bytes of the whole tensor."""
+        import torch
+
+        if not len(global_shape) == len(shard_offset) == len(shape):
+            raise ValueError(f"rank mismatch: global_shape {tuple(global_shape)}, shard_offset "
+                             f"{tuple(shard_offset)} and shape {tuple(shape)} must have equal rank")
+        n = itemsize
+        for d in shape:
+            n *= int(d)
+        if out is None:
+            out = torch.empty(max(n, 1), dtype=torch.uint8, device=torch.device("cuda", self.device))[:n]
+        # merge trailing dims that are taken whole, keep the next one as the row index
+        dims = [(int(g), int(o), int(s)) for g, o, s in zip(global_shape, shard_offset, shape)]
+        run_src = run_dst = itemsize
+        while dims and dims[-1][1] == 0 and dims[-1][2] == dims[-1][0]:
+            g, _o, s = dims.pop()
+            run_src *= g
+            run_dst *= s
+        base = _addr(full)
+        boxes = []
+        if not dims:
+            boxes.append({"src": base, "dst": out, "rows": 1, "row_bytes": run_dst, "csum_index": 0})
+        else:
+            g, o, s = dims.pop()  # innermost sliced dim: a contiguous piece of s * run bytes per outer index
+            piece = s * run_dst
+            src_stride = g * run_src
+            strides, acc = [], src_stride
+            for gg, _oo, _ss in reversed(dims):
+                strides.append(acc)
+                acc *= gg
+            strides.reverse()
+            import itertools
+
+            for k, idx in enumerate(itertools.product(*[range(ss) for _g, _o, ss in dims])):
+                off = o * run_src + sum((i + oo) * st for i, (_gg, oo, _ss), st in zip(idx, dims, strides))
+                boxes.append({"src": base + off, "dst": _addr(out) + k * piece, "rows": 1, "row_bytes": piece,
+                              "csum_index": k * piece})
+        sums = self.place_boxes(boxes, 1, stream=stream)
+        return out, sums[0]
+
     def copy_batch(self, srcs: Sequence, dsts: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
                    checksums: bool = True) -> list[str] | None:
         """n contiguous device copies in one launch (optionally with destination checksums)."""

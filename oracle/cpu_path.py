@@ -71,10 +71,24 @@ def run(ckpt_dir: str, rank_params: list, *, tp_size=1, tp_rank=0, stacked=None,
         d0 = dest.data.ctypes.data
         s0 = src.data.ctypes.data
         for d_off, s_off, rows, row_bytes, dp, sp in _boxes(dest.data, src.data, cast):
-            recs.append(cbind.OrcWrite(src=s0 + s_off, dst=d0 + d_off, src_pitch=sp, dst_pitch=dp, rows=rows,
-                                       row_bytes=row_bytes, dst_index=d0 + d_off - base_addr[pname],
-                                       param=index[pname], cast=int(cast)))
             placed += rows * row_bytes
+            # Pieces of at most ~4 MiB, so one large tensor does not serialise the thread pool.
+            if rows == 1:
+                step = 4 << 20
+                for lo in range(0, row_bytes, step):
+                    n = min(step, row_bytes - lo)
+                    recs.append(cbind.OrcWrite(src=s0 + s_off + lo * (2 if cast else 1), dst=d0 + d_off + lo, src_pitch=0,
+                                               dst_pitch=0, rows=1, row_bytes=n,
+                                               dst_index=d0 + d_off + lo - base_addr[pname], param=index[pname],
+                                               cast=int(cast)))
+            else:
+                step = max(1, (4 << 20) // row_bytes)
+                for lo in range(0, rows, step):
+                    n = min(step, rows - lo)
+                    recs.append(cbind.OrcWrite(src=s0 + s_off + lo * sp, dst=d0 + d_off + lo * dp, src_pitch=sp,
+                                               dst_pitch=dp, rows=n, row_bytes=row_bytes,
+                                               dst_index=d0 + d_off + lo * dp - base_addr[pname], param=index[pname],
+                                               cast=int(cast)))
     t_plan = time.perf_counter() - t0
     best = None
     sums = None

@@ -122,3 +122,52 @@ def test_gather2d_matches_oracle(gpu_engine, oracle_c, rows, row_bytes, src_pitc
     for r in range(rows):
         acc += int(oracle_c.checksum32(want[r * dst_pitch: r * dst_pitch + row_bytes], first_index=r * dst_pitch), 16)
     assert csum == format(acc & 0xFFFFFFFF, "08x")
+
+
+def test_place_boxes_mixed_batch(gpu_engine, oracle, oracle_c):
+    rng = np.random.default_rng(15)
+    src_a = rng.integers(0, 256, 64 * 512, dtype=np.uint8)           # (64, 512) bytes, take cols 128..255
+    src_f = rng.integers(0, 1 << 32, 4096, dtype=np.uint64).astype(np.uint32)  # fp32 bits, cast 1000 elements
+    src_c = rng.integers(0, 256, 5000, dtype=np.uint8)
+    da, df, dc = _dev(src_a), _dev(src_f), _dev(src_c)
+    out = torch.zeros(64 * 128 + 2048 + 5008, dtype=torch.uint8, device="cuda")
+    o_a, o_f, o_c = 0, 64 * 128, 64 * 128 + 2048
+    boxes = [
+        {"src": da[128:], "dst": out[o_a:], "src_pitch": 512, "dst_pitch": 128, "rows": 64, "row_bytes": 128,
+         "csum_index": 0, "csum_group": 0},
+        {"src": df[4 * 8:], "dst": out[o_f:], "rows": 1, "row_bytes": 2000, "cast": 1, "csum_index": 0, "csum_group": 1},
+        {"src": dc[3:], "dst": out[o_c:], "rows": 1, "row_bytes": 4990, "csum_index": 10, "csum_group": 2},
+    ]
+    sums = gpu_engine.place_boxes(boxes, 3)
+    got = out.cpu().numpy()
+    want_a = np.ascontiguousarray(src_a.reshape(64, 512)[:, 128:256])
+    want_f = oracle.cast_f32_bf16_bits(src_f[8:1008]).view(np.uint8)
+    want_c = src_c[3:4993]
+    assert got[o_a:o_a + want_a.size].tobytes() == want_a.tobytes()
+    assert got[o_f:o_f + 2000].tobytes() == want_f.tobytes()
+    assert got[o_c:o_c + 4990].tobytes() == want_c.tobytes()
+    assert sums[0] == oracle_c.checksum32(want_a)
+    assert sums[1] == oracle_c.checksum32(want_f)
+    assert sums[2] == oracle_c.checksum32(want_c, first_index=10)
+
+
+def test_shard_region_matches_oracle(gpu_engine, oracle):
+    # refit/reshard/verify.py:158-183 and tests/test_reshard_refit_verify.py:135-171
+    OT = oracle.OTensor
+    full = np.arange(24, dtype=np.float32).reshape(4, 6)
+    d = _dev(full)
+    buf, csum = gpu_engine.shard_region(d, (4, 6), (1, 2), (2, 3), 4)
+    want = oracle.shard_region(OT.from_array(full.reshape(-1), "F32"), (4, 6), (1, 2), (2, 3))
+    assert buf.cpu().numpy().tobytes() == want.tobytes() == np.ascontiguousarray(full[1:3, 2:5]).tobytes()
+    assert csum == oracle.safe_checksum(want)
+    assert gpu_engine.digest([buf])[0] == oracle.tensor_digest(want)
+    with pytest.raises(ValueError, match="rank mismatch"):
+        gpu_engine.shard_region(d, (4, 6), (1,), (2, 3), 4)
+    rng = np.random.default_rng(16)
+    big = rng.integers(0, 1 << 16, (6, 40, 96), dtype=np.uint16)
+    db = _dev(big)
+    for off, shp in [((1, 8, 0), (4, 16, 96)), ((0, 0, 32), (6, 40, 48)), ((2, 3, 5), (3, 30, 7)), ((0, 0, 0), (6, 40, 96))]:
+        buf, csum = gpu_engine.shard_region(db, big.shape, off, shp, 2)
+        want = oracle.shard_region(OT.from_array(big.reshape(-1), "BF16"), big.shape, off, shp)
+        assert buf.cpu().numpy().tobytes() == want.tobytes(), (off, shp)
+        assert csum == oracle.safe_checksum(want)
