@@ -74,6 +74,9 @@ def main() -> int:
     ap.add_argument("--slot-mib", type=int, default=16, help="pinned ring slot size for the ingest leg")
     ap.add_argument("--ring-slots", type=int, default=32)
     ap.add_argument("--readers", type=int, default=0, help="reader threads for the ingest leg (0 = host cores, at most 16)")
+    ap.add_argument("--cold", action="store_true",
+                    help="also run the ingest leg with O_DIRECT from a file system that supports it (MXP_BENCH_DIR), "
+                         "bypassing the page cache")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB device copy (a kernel of known traffic, for scaling profiler counters)")
     ap.add_argument("--seed", type=int, default=20240229)
@@ -243,6 +246,20 @@ def main() -> int:
                     "ring": f"{args.ring_slots} x {args.slot_mib} MiB pinned", "source": f"page cache ({workdir})",
                     "checksums_match_resident": ingest_sums == resident_sums}
                 _log(f"{key}: {out[key]}")
+
+        if files_real and args.cold:
+            e2 = PlacementEngine(0, ring_slots=args.ring_slots, slot_bytes=args.slot_mib << 20,
+                                 reader_threads=args.readers or host_threads, streams=4, use_o_direct=True)
+            st = e2.execute(plan, dst)
+            cold_sums = e2.checksums(plan)
+            e2.close()
+            agree = agree and cold_sums == resident_sums
+            out["e2e_ingest_direct_io"] = {
+                "placed_gbps": round(st["placed_bytes"] / st["wall_seconds"] / 1e9, 3),
+                "file_gbps": round(st["file_bytes"] / st["wall_seconds"] / 1e9, 3), "wall_s": round(st["wall_seconds"], 3),
+                "file_bytes": st["file_bytes"], "source": f"O_DIRECT reads from {workdir} (first pass, storage-bound)",
+                "checksums_match_resident": cold_sums == resident_sums}
+            _log(f"e2e_ingest_direct_io: {out['e2e_ingest_direct_io']}")
 
         # ---- CPU baseline: the oracle placing the same rank from the same files ----
         if files_real and not args.no_cpu:

@@ -14,6 +14,7 @@
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <mutex>
@@ -78,6 +79,7 @@ struct mxp_plan::Lowered {
   uint64_t slot_bytes = 0;
   uint32_t tile_bytes = 0;
   bool host_pack = false;
+  bool direct_io = false;
   // resident tables: source buffer index = shard file index
   DevBuf<Seg> res_segs;
   DevBuf<WorkItem> res_work;
@@ -132,13 +134,17 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   if (!pl.built) throw Error(MXP_ERR_STATE, "plan has not been built");
   const bool host_pack = eng.opt.pack_strided_on_host == 1;
   if (pl.lowered && pl.lowered->slot_bytes == eng.opt.slot_bytes && pl.lowered->tile_bytes == eng.opt.tile_bytes &&
-      pl.lowered->host_pack == host_pack)
+      pl.lowered->host_pack == host_pack && pl.lowered->direct_io == (eng.opt.use_o_direct != 0))
     return;
   if (pl.lowered) { free_lowered(pl.lowered); pl.lowered = nullptr; }
   auto L = std::make_unique<mxp_plan::Lowered>();
   L->slot_bytes = eng.opt.slot_bytes;
   L->tile_bytes = eng.opt.tile_bytes;
   L->host_pack = host_pack;
+  L->direct_io = eng.opt.use_o_direct != 0;
+  // Direct I/O reads whole 4 KiB blocks at 4 KiB offsets into 4 KiB aligned memory: every
+  // range is widened to block boundaries and the box starts that many bytes into the slot.
+  const uint64_t blk = L->direct_io ? 4096 : 1;
   LowerOptions lo;
   lo.tile_bytes = eng.opt.tile_bytes;
   const mxp_ckpt& ck = *pl.ckpt;
@@ -178,7 +184,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
     uint64_t rows = 1, file_pitch = 0;  // rows > 1: strided in the file, packed in the slot
   };
   std::vector<Piece> pieces;
-  const uint64_t slot = eng.opt.slot_bytes;
+  const uint64_t slot = L->direct_io ? eng.opt.slot_bytes - 2 * blk : eng.opt.slot_bytes;
   for (const auto& w : pl.writes) {
     const TensorRec& t = ck.tensors[w.tensor];
     const uint64_t sm = w.cast ? 2 : 1;
@@ -254,9 +260,17 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       cur = Chunk();
     };
     for (auto& p : pieces) {
-      uint64_t at = align_up(cur.used_bytes, 256);
+      uint64_t at = align_up(cur.used_bytes, L->direct_io ? blk : 256);
+      uint64_t lead = 0, need = 0;
+      if (L->direct_io) {
+        const uint64_t a0 = p.file_off / blk * blk, a1 = align_up(p.file_off + p.nbytes, blk);
+        lead = p.file_off - a0;
+        need = lead + p.nbytes;
+        p.file_off = a0;
+        p.nbytes = a1 - a0;
+      }
       const uint64_t in_slot = p.nbytes * p.rows;
-      if (!cur.ranges.empty() && at + in_slot > slot) {
+      if (!cur.ranges.empty() && at + in_slot > eng.opt.slot_bytes) {
         close();
         at = 0;
       }
@@ -264,10 +278,10 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
         cur.seg_begin = (uint32_t)segs.size();
         cur.work_begin = (uint32_t)work.size();
       }
-      cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at, p.rows, p.file_pitch});
+      cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at, p.rows, p.file_pitch, need});
       cur.used_bytes = at + in_slot;
       L->file_bytes += in_slot;
-      p.box.src_off = at;
+      p.box.src_off = at + lead;
       const size_t w0 = work.size();
       lower_box(p.box, lo, segs, work);
       // work items index segments relative to the chunk's first segment
@@ -304,14 +318,21 @@ void upload_dst(mxp_plan::Lowered& L, const mxp_plan& pl, void* const* dst_ptrs)
   L.dst_host.assign(dst_ptrs, dst_ptrs + n);
 }
 
-void pread_full(int fd, uint8_t* dst, uint64_t n, uint64_t off, const std::string& path) {
+// Reads n bytes at off.  `need` (0 = n) is how many of them must exist: a range rounded up
+// for direct I/O may run past the end of the file.
+void pread_full(int fd, uint8_t* dst, uint64_t n, uint64_t off, const std::string& path, uint64_t need = 0) {
+  const uint64_t total = n;
+  if (need == 0) need = n;
   while (n) {
     const ssize_t r = ::pread(fd, dst, (size_t)std::min<uint64_t>(n, 1ull << 30), (off_t)off);
     if (r < 0) {
       if (errno == EINTR) continue;
       throw Error(MXP_ERR_IO, "read failed on " + path + ": " + std::strerror(errno));
     }
-    if (r == 0) throw Error(MXP_ERR_IO, "unexpected end of file in " + path + " at offset " + std::to_string(off));
+    if (r == 0) {
+      if (total - n >= need) return;
+      throw Error(MXP_ERR_IO, "unexpected end of file in " + path + " at offset " + std::to_string(off));
+    }
     dst += r;
     off += (uint64_t)r;
     n -= (uint64_t)r;
@@ -397,6 +418,8 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     // wrong for direct I/O, where whole row bands are staged and gathered on the device.
     if (o.pack_strided_on_host == 0) o.pack_strided_on_host = o.use_o_direct ? 2 : 1;
     if (o.pack_strided_on_host > 2) throw Error(MXP_ERR_ARG, "pack_strided_on_host must be 0, 1 or 2");
+    if (o.use_o_direct && o.pack_strided_on_host == 1)
+      throw Error(MXP_ERR_ARG, "direct I/O reads whole blocks; it cannot be combined with per-row host packing");
     if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
     if (o.tile_bytes < 1024 || o.tile_bytes > (1u << 20)) throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 1 MiB]");
     if (o.ring_slots > 256 || o.reader_threads > 256 || o.streams > 64) throw Error(MXP_ERR_ARG, "ring, thread or stream count too large");
@@ -489,8 +512,15 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
   const size_t n_slots = e.slots.size();
 
   auto worker = [&](int tid) {
+    // The kernel refuses direct I/O into HIP pinned memory (EFAULT: the mapping cannot be
+    // pinned again by the block layer), so direct reads land in an ordinary block-aligned
+    // buffer and are copied into the slot.
+    void* direct_buf = nullptr;
+    struct Free { void*& p; ~Free() { std::free(p); } } free_direct{direct_buf};
     try {
       HIP_OK(hipSetDevice(e.opt.device));
+      if (L.direct_io && ::posix_memalign(&direct_buf, 4096, e.opt.slot_bytes) != 0)
+        throw Error(MXP_ERR_STATE, "out of host memory for the direct I/O buffer");
       for (;;) {
         const size_t c = next.fetch_add(1);
         if (c >= n_chunks || abort.load()) break;
@@ -507,9 +537,16 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
         if (turn > 0) HIP_OK(hipEventSynchronize(sl.done));
         const double t0 = now_s();
         for (const auto& r : ch.ranges)
-          for (uint64_t row = 0; row < r.rows; ++row)
-            pread_full(fds[r.file], sl.host + r.slot_off + row * r.nbytes, r.nbytes, r.file_off + row * r.file_pitch,
-                       ck.files[r.file].path);
+          for (uint64_t row = 0; row < r.rows; ++row) {
+            uint8_t* into = sl.host + r.slot_off + row * r.nbytes;
+            if (direct_buf) {
+              pread_full(fds[r.file], static_cast<uint8_t*>(direct_buf), r.nbytes, r.file_off + row * r.file_pitch,
+                         ck.files[r.file].path, r.need);
+              std::memcpy(into, direct_buf, r.need ? r.need : r.nbytes);
+            } else {
+              pread_full(fds[r.file], into, r.nbytes, r.file_off + row * r.file_pitch, ck.files[r.file].path, r.need);
+            }
+          }
         read_s[tid] += now_s() - t0;
         hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
         HIP_OK(hipMemcpyAsync(sl.dev, sl.host, ch.used_bytes, hipMemcpyHostToDevice, st));

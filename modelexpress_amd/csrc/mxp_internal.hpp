@@ -77,7 +77,12 @@ struct ExpertRec { std::string param_prefix, weight_prefix; int expert_id; std::
 // One slot-sized unit of ingest work: byte ranges packed into a staging slot and the
 // device segments that consume them.
 // `rows` pieces of `nbytes`, `file_pitch` apart in the file, packed back to back in the slot.
-struct FileRange { int file; uint64_t file_off, nbytes, slot_off; uint64_t rows = 1, file_pitch = 0; };
+struct FileRange {
+  int file;
+  uint64_t file_off, nbytes, slot_off;
+  uint64_t rows = 1, file_pitch = 0;
+  uint64_t need = 0;  // bytes that must exist (a direct-I/O range is rounded up past them); 0 = all
+};
 struct Chunk {
   std::vector<FileRange> ranges;
   uint64_t used_bytes = 0;   // bytes of the slot that cross PCIe
