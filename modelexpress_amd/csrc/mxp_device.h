@@ -59,14 +59,14 @@ struct alignas(16) DigestJob {
 constexpr uint32_t kKnuth = 2654435761u;
 constexpr int kPlaceThreads = 1024;  // lanes per placement workgroup (16 wavefronts)
 constexpr int kPlaceBatch = 8;       // 16-byte units each lane keeps in flight
-constexpr int kDigestThreads = 256;
+constexpr int kDigestThreads = 1024;
 constexpr uint32_t kDigestRowWords = 1024;   // 4 KiB rows
-constexpr uint32_t kDigestRowsPerBlock = 16; // 64 KiB per workgroup
+constexpr uint32_t kDigestRowsPerBlock = 32; // 128 KiB per workgroup, two rows per wavefront
 
 // ---- launch wrappers (mxp_kernels.hip) -------------------------------------
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
-                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream);
+                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only = false);
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
                          unsigned long long* out_dev, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);

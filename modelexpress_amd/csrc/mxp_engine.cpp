@@ -375,10 +375,12 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
   if (!dsts.empty()) std::memcpy(e.desc_host + o_dst, dsts.data(), dsts.size() * sizeof(void*));
   HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, total, hipMemcpyHostToDevice, stream));
   uint8_t* d = e.desc_dev.p;
+  bool checksum_only = !boxes.empty();
+  for (const auto& b : boxes) checksum_only = checksum_only && b.op == kOpChecksumOnly;
   HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + o_segs), reinterpret_cast<const WorkItem*>(d + o_work),
                       (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + o_src),
                       reinterpret_cast<void* const*>(d + o_dst), reinterpret_cast<uint32_t*>(d + o_sum),
-                      e.opt.nan_bits, stream));
+                      e.opt.nan_bits, stream, checksum_only));
   if (sums_out && n_sums) {
     HIP_OK(hipMemcpyAsync(e.desc_host + o_sum, d + o_sum, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));

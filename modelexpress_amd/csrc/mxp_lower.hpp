@@ -24,7 +24,7 @@ struct BoxCopy {
 };
 
 struct LowerOptions {
-  uint32_t tile_bytes = 128 * 1024;  // destination bytes one workgroup handles (one batch)
+  uint32_t tile_bytes = 128 * 1024;  // SOURCE bytes one workgroup handles (one batch of loads)
   uint32_t flat_row_bytes = 8192;   // virtual row width used to tile contiguous runs
   uint32_t max_row_bytes = 32768;   // wider pitched rows are split by columns
 };
@@ -70,7 +70,7 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
   s.csum_bias = (uint32_t)b.csum_bias;
   s.units_per_row = s.row_bytes / unit;
   s.div_magic = s.units_per_row > 1 ? (uint32_t)((1ull << 32) / s.units_per_row) + 1u : 0u;
-  uint64_t rpt = std::max<uint64_t>(1, o.tile_bytes / b.row_bytes);
+  uint64_t rpt = std::max<uint64_t>(1, o.tile_bytes / (b.row_bytes * sm));
   rpt = std::min<uint64_t>(rpt, b.rows);
   // In-tile byte offsets are 32-bit on the device, and the reciprocal division is exact
   // only while (units in tile) * (units per row) < 2^32.
