@@ -280,6 +280,17 @@ def main() -> int:
                           f"same files, best of 3; parse {res['parse_s']:.3f}s + plan {res['plan_s']:.3f}s not included",
                 "place_s": round(res["place_s"], 4), "host_cpus": os.cpu_count(),
                 "checksums_match_gpu": cpu_sums == resident_sums}
+            if layout.family == "llama" and not cast:
+                # The literal torch-CPU formulation of the reference on one layer's seven matrices.
+                lp = f"model.layers.{n_layers // 2}."
+                sample = [(lp + "self_attn.q_proj.weight", 0), (lp + "self_attn.k_proj.weight", 0),
+                          (lp + "self_attn.v_proj.weight", 0), (lp + "self_attn.o_proj.weight", 1),
+                          (lp + "mlp.gate_proj.weight", 0), (lp + "mlp.up_proj.weight", 0), (lp + "mlp.down_proj.weight", 1)]
+                fr = cpu_path.run_faithful_sample(workdir, sample, tp, rank, host_threads)
+                out["cpu_baseline"]["faithful_torch_ops"] = {
+                    "value": round(fr["placed_bytes"] / fr["seconds"] / 1e9, 3), "unit": "GB/s", "cores": host_threads,
+                    "sample": f"one layer's q/k/v/o/gate/up/down slices ({fr['placed_bytes']} bytes): narrow().contiguous(), "
+                              "copy_, and safe_checksum as the reference writes it (int64 arange per byte)"}
         else:
             out["cpu_baseline"] = {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "skipped"}
         out["checksums_agree"] = agree

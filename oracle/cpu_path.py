@@ -99,3 +99,34 @@ def run(ckpt_dir: str, rank_params: list, *, tp_size=1, tp_rank=0, stacked=None,
         best = dt if best is None else min(best, dt)
     return {"parse_s": t_parse, "plan_s": t_plan, "place_s": best, "placed_bytes": placed, "n_writes": len(recs),
             "params": params, "checksums": dict(zip([n for n, _d, _s in rank_params], sums)), "threads": threads}
+
+
+def run_faithful_sample(ckpt_dir: str, names: list, tp_size: int, tp_rank: int, threads: int) -> dict:
+    """The reference's own op sequence on torch CPU tensors, for a handful of tensors:
+    ``narrow(axis, r*n, n).contiguous()`` (installer.py:317), ``dest.copy_(src)``
+    (installer.py:419-424) and ``safe_checksum`` exactly as written -- int64 ``arange`` of one
+    entry per byte, int64 products, masked sum (tensor_utils.py:36-42) -- applied to the
+    flattened tensor (the 1-D case, the only one in which the reference returns a value).
+    Returns bytes processed and seconds; used only to report how the literal formulation
+    compares with the one-pass C form."""
+    import torch
+
+    torch.set_num_threads(threads)
+    weights = dict(O.load_checkpoint(ckpt_dir, mmap=True))
+    placed = 0
+    t0 = time.perf_counter()
+    sums = {}
+    for name, axis in names:
+        src = weights[name]
+        t = torch.from_numpy(np.ascontiguousarray(src.data).reshape(src.shape + (src.data.shape[-1],)))
+        local = t.shape[axis] // tp_size
+        shard = t.narrow(axis, tp_rank * local, local).contiguous()
+        dest = torch.empty_like(shard)
+        dest.copy_(shard)
+        flat = dest.reshape(-1)
+        idx = torch.arange(flat.numel(), dtype=torch.int64)
+        w = (idx * 2654435761 + 1) & 0xFFFFFFFF
+        mixed = (flat.to(torch.int64) * w) & 0xFFFFFFFF
+        sums[name] = format(mixed.sum().item() & 0xFFFFFFFF, "08x")
+        placed += flat.numel()
+    return {"seconds": time.perf_counter() - t0, "placed_bytes": placed, "checksums": sums}

@@ -1,0 +1,49 @@
+"""Committed golden vectors (tests/golden/vectors.json, made by tests/golden/make_vectors.py
+without the oracle or the product) against the oracle on the host and the HIP path on the GPU."""
+
+import json
+from pathlib import Path
+
+import numpy as np
+import pytest
+
+from golden.make_vectors import lcg_bytes
+
+VEC = json.loads((Path(__file__).parent / "golden" / "vectors.json").read_text())
+
+
+def test_oracle_matches_golden_vectors(oracle, oracle_c):
+    for v in VEC["checksum"]:
+        raw = lcg_bytes(v["seed"], v["n"])
+        if v["hex"] is not None:
+            assert raw.hex() == v["hex"]
+        assert oracle.safe_checksum_bytes(raw) == v["checksum"]
+        assert oracle_c.checksum32(np.frombuffer(raw, dtype=np.uint8)) == v["checksum"]
+    for v in VEC["digest"]:
+        raw = lcg_bytes(v["seed"], v["n"])
+        sc = [x & ((1 << 64) - 1) for x in oracle.tensor_digest_scalars(raw)]
+        assert [str(x) for x in sc] == v["scalars"]
+        assert oracle.tensor_digest_bytes(raw) == v["digest"]
+    bits = np.array(VEC["cast"]["f32_bits"], dtype=np.uint32)
+    want = np.array(VEC["cast"]["bf16_bits"], dtype=np.uint16)
+    assert np.array_equal(oracle.cast_f32_bf16_bits(bits), want)
+    assert np.array_equal(oracle_c.cast_f32_bf16(bits), want)
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_golden_vectors(gpu_engine):
+    import torch
+
+    def dev(raw):
+        return torch.from_numpy(np.frombuffer(raw, dtype=np.uint8).copy()).cuda() if raw else \
+            torch.empty(0, dtype=torch.uint8, device="cuda")
+
+    bufs = [dev(lcg_bytes(v["seed"], v["n"])) for v in VEC["checksum"]]
+    assert gpu_engine.checksum32(bufs) == [v["checksum"] for v in VEC["checksum"]]
+    assert gpu_engine.digest(bufs) == [v["digest"] for v in VEC["digest"]]
+    bits = np.array(VEC["cast"]["f32_bits"], dtype=np.uint32)
+    want = np.array(VEC["cast"]["bf16_bits"], dtype=np.uint16)
+    src = torch.from_numpy(bits.view(np.uint8).copy()).cuda()
+    dst = torch.zeros(bits.size * 2, dtype=torch.uint8, device="cuda")
+    gpu_engine.cast_f32_bf16(src, dst, bits.size)
+    assert np.array_equal(dst.cpu().numpy().view(np.uint16), want)
