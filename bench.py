@@ -217,6 +217,25 @@ def main() -> int:
                                 "gbps_wall": round(placed / dt / 1e9, 1),
                                 "note": "one batched launch; wall time includes descriptor upload, result copy and sync"}
             ops["checksum32"]["matches_fused"] = eng.checksum32(dst, sizes) == resident_sums
+            # LDS-tiled transpose (permuted copies): a square bf16 matrix and the MLA W_UK_T shape
+            for label, shape, perm in (("transpose_bf16_16384x16384", (16384, 16384), (1, 0)),
+                                       ("mla_w_uk_t_bf16_128x128x512", (128, 128, 512), (1, 2, 0))):
+                nbytes = 2
+                for v in shape:
+                    nbytes *= v
+                a = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 256)
+                b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+                eng.permute_copy(a, b, shape, perm, 2, checksum=False)
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ev0.record()
+                for _ in range(10):
+                    eng.permute_copy(a, b, shape, perm, 2, checksum=False)
+                ev1.record()
+                torch.cuda.synchronize()
+                ms = ev0.elapsed_time(ev1) / 10
+                ops[label] = {"bytes": nbytes, "ms": round(ms, 4), "gbps_algorithmic": round(2 * nbytes / ms / 1e6, 1),
+                              "frac_of_hbm_peak": round(2 * nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                del a, b
             out["ops"] = ops
 
         # ---- end-to-end ingest from files through the pinned ring ----

@@ -143,6 +143,19 @@ int mxp_plan_add_expert(mxp_plan* plan, const char* param_prefix, const char* we
                         int32_t expert_id, const char* shard, int32_t local_expert_id);
 /* Skip checkpoint tensors whose name starts with `prefix` (e.g. other pipeline stages). */
 int mxp_plan_add_skip_prefix(mxp_plan* plan, const char* prefix);
+/* A virtual checkpoint tensor: a full shape assembled from boxes ("shards") of real
+ * checkpoint tensors, the published-tensor model of the reference's reshard path
+ * (PublishedTensor.full_shape + shards[].shard_offset/shape; plan_pull intersects the
+ * needed box with every shard box, refit/reshard/slice_plan.py:248-256,297-339).  The
+ * virtual tensor is then placed like a checkpoint tensor of that name; the real tensors it
+ * is made of are consumed.  This is how trainer-native layouts enter: Megatron's
+ * by-KV-group interleaved linear_qkv becomes virtual q/k/v tensors made of row bands
+ * (modelexpress_rl/train/engines/megatron/aliases.py:206-263,291-350), a fused gate/up
+ * tensor two halves (aliases.py:116-168).  Shards must not overlap; the part of the virtual
+ * tensor a rank needs must be covered (else MXP_ERR_COVERAGE from mxp_plan_build). */
+int64_t mxp_plan_add_virtual(mxp_plan* plan, const char* name, int32_t ndim, const int64_t* full_shape);
+int mxp_plan_add_virtual_shard(mxp_plan* plan, int64_t virtual_index, const char* source_tensor,
+                               const int64_t* source_offset, const int64_t* shard_offset, const int64_t* shape);
 int mxp_plan_build(mxp_plan* plan);
 
 #define MXP_WRITE_DIRECT 0
@@ -297,6 +310,18 @@ typedef struct mxp_box {
  * overlap in the destination. */
 int mxp_place_boxes(mxp_engine* engine, const mxp_box* boxes, int64_t n, uint32_t n_groups,
                     uint32_t* out_checksums, void* stream);
+/* dst = src.permute(perm).contiguous() for an ndim-dimensional tensor (ndim <= 8) of
+ * elem_size-byte elements (1, 2, 4 or 8).  `shape` is the source's shape, `src_strides`
+ * its strides in elements (NULL = contiguous row-major; a narrowed view passes the parent's
+ * strides), `perm[d]` the source dimension that becomes destination dimension d.
+ * Replaces W_UV = w_uv.transpose(0,1) and W_UK_T = w_uk.permute(1,2,0)
+ * (engines/vllm/refit/receiver.py:252-261) and the permuted views of
+ * refit/reshard/slice_plan.py:166-220.  Permutations that keep the innermost dimension run
+ * as a batched row gather; the others as an LDS-tiled transpose.  *checksum, when not
+ * NULL, receives the checksum of the destination bytes. */
+int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
+                     const int64_t* src_strides, const int32_t* perm, int32_t elem_size, uint32_t* checksum,
+                     void* stream);
 /* n independent contiguous device copies in one launch, with the checksum of each
  * destination in out_checksums[k] when not NULL: the device form of the batched
  * torch._foreach_copy_ install (refit/reshard/receiver.py:939-955).  Destinations must

@@ -121,6 +121,9 @@ SIGNATURES = {
     "mxp_plan_add_stacked": (C.c_int, [_P, C.c_char_p, C.c_char_p]),
     "mxp_plan_add_expert": (C.c_int, [_P, C.c_char_p, C.c_char_p, C.c_int32, C.c_char_p, C.c_int32]),
     "mxp_plan_add_skip_prefix": (C.c_int, [_P, C.c_char_p]),
+    "mxp_plan_add_virtual": (C.c_int64, [_P, C.c_char_p, C.c_int32, C.POINTER(C.c_int64)]),
+    "mxp_plan_add_virtual_shard": (C.c_int, [_P, C.c_int64, C.c_char_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64),
+                                             C.POINTER(C.c_int64)]),
     "mxp_plan_build": (C.c_int, [_P]),
     "mxp_plan_param_count": (C.c_int64, [_P]),
     "mxp_plan_write_count": (C.c_int64, [_P]),
@@ -138,6 +141,8 @@ SIGNATURES = {
     "mxp_cast_f32_bf16": (C.c_int, [_P, _P, _P, C.c_uint64, _U32P, _P]),
     "mxp_gather2d": (C.c_int, [_P, _P, C.c_uint64, _P, C.c_uint64, C.c_uint64, C.c_uint64, _U32P, _P]),
     "mxp_place_boxes": (C.c_int, [_P, C.POINTER(Box), C.c_int64, C.c_uint32, _U32P, _P]),
+    "mxp_permute_copy": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64),
+                                   C.POINTER(C.c_int32), C.c_int32, _U32P, _P]),
     "mxp_copy_batch": (C.c_int, [_P, _PP, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_digest_from_scalars": (C.c_int, [_U64P, C.POINTER(C.c_uint8)]),

@@ -21,6 +21,7 @@ LIB_PATH = PKG_DIR / "libmxplace.so"
 SOURCES = (
     "mxp_kernels.hip",
     "mxp_synth.hip",
+    "mxp_permute.hip",
     "mxp_ckpt.cpp",
     "mxp_plan.cpp",
     "mxp_engine.cpp",

@@ -71,6 +71,23 @@ hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_
                          unsigned long long* out_dev, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);
 
+// Batched 2-D transpose (mxp_permute.hip).  "i" = the destination's innermost dimension,
+// "j" = the source's innermost dimension; strides are in elements.
+constexpr int kMaxBatchDims = 6;
+struct TransposeDesc {
+  uint64_t ni, nj;   // extents
+  uint64_t si;       // source stride of i (source stride of j is 1)
+  uint64_t dj;       // destination stride of j (destination stride of i is 1)
+  uint32_t tiles_i, tiles_j;
+  uint64_t batch_size[kMaxBatchDims];     // unused entries are 1
+  uint64_t batch_sstride[kMaxBatchDims];
+  uint64_t batch_dstride[kMaxBatchDims];
+  uint32_t vec_src, vec_dst;  // 16-byte accesses are aligned on that side
+  uint32_t csum_bias, pad;
+};
+hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
+                            uint32_t* sum_out, hipStream_t stream);
+
 // Synthetic-checkpoint generator (mxp_synth.hip), same arithmetic on host and device.
 enum SynthKind : uint32_t {
   kSynthNormal = 0,   // ~N(0, 0.02): centred sum of four 16-bit uniforms times a constant

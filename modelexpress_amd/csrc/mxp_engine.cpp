@@ -823,6 +823,147 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n
   });
 }
 
+int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
+                     const int64_t* src_strides, const int32_t* perm, int32_t elem_size, uint32_t* checksum,
+                     void* stream_v) {
+  return guard([&] {
+    if (!engine || ndim < 0 || ndim > MXP_MAX_DIMS || (ndim && (!shape || !perm)))
+      throw Error(MXP_ERR_ARG, "mxp_permute_copy: bad argument");
+    if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8)
+      throw Error(MXP_ERR_ARG, "mxp_permute_copy: elem_size must be 1, 2, 4 or 8");
+    if (checksum) *checksum = 0;
+    mxp_engine& e = *engine;
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    const uint64_t es = (uint64_t)elem_size;
+    // Dimensions in destination order.
+    std::vector<uint64_t> size, ss;
+    {
+      std::vector<int64_t> rm((size_t)ndim, 1);
+      for (int d = ndim - 2; d >= 0; --d) rm[d] = rm[d + 1] * shape[d + 1];
+      std::vector<bool> seen((size_t)ndim, false);
+      for (int d = 0; d < ndim; ++d) {
+        if (perm[d] < 0 || perm[d] >= ndim || seen[perm[d]]) throw Error(MXP_ERR_ARG, "mxp_permute_copy: perm is not a permutation");
+        seen[perm[d]] = true;
+        if (shape[perm[d]] < 0) throw Error(MXP_ERR_ARG, "mxp_permute_copy: negative extent");
+        const int64_t st = src_strides ? src_strides[perm[d]] : rm[perm[d]];
+        if (st < 0) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: negative strides are not supported");
+        size.push_back((uint64_t)shape[perm[d]]);
+        ss.push_back((uint64_t)st);
+      }
+    }
+    uint64_t total = 1;
+    for (auto n : size) total *= n;
+    if (total == 0) return;
+    if (!src || !dst) throw Error(MXP_ERR_ARG, "mxp_permute_copy: null pointer");
+    if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_permute_copy: dst must be 16-byte aligned");
+    if (reinterpret_cast<uintptr_t>(src) % es) throw Error(MXP_ERR_ARG, "mxp_permute_copy: src is not element aligned");
+    HIP_OK(hipSetDevice(e.opt.device));
+    // Drop unit dims; merge neighbours that are contiguous in the source too (the
+    // destination is contiguous, so it always merges).
+    {
+      std::vector<uint64_t> n2, s2;
+      for (size_t d = 0; d < size.size(); ++d)
+        if (size[d] != 1) { n2.push_back(size[d]); s2.push_back(ss[d]); }
+      size.clear();
+      ss.clear();
+      for (size_t d = 0; d < n2.size(); ++d) {
+        if (!size.empty() && ss.back() == s2[d] * n2[d]) {
+          size.back() *= n2[d];
+          ss.back() = s2[d];
+        } else {
+          size.push_back(n2[d]);
+          ss.push_back(s2[d]);
+        }
+      }
+      if (size.empty()) { size.push_back(1); ss.push_back(1); }
+    }
+    const size_t nd = size.size();
+    std::vector<uint64_t> ds(nd, 1);
+    for (int d = (int)nd - 2; d >= 0; --d) ds[d] = ds[d + 1] * size[d + 1];
+
+    if (ss[nd - 1] == 1 || total == 1) {
+      // The innermost dimension is kept: rows of size[last] elements, gathered.
+      const uint64_t row_bytes = size[nd - 1] * es;
+      const void* sb;
+      uint64_t so;
+      split_ptr(src, sb, so);
+      std::vector<BoxCopy> boxes;
+      BoxCopy b;
+      b.row_bytes = row_bytes;
+      b.op = kOpCopy;
+      b.csum_slot = checksum ? 0u : 0xFFFFFFFFu;
+      if (nd == 1) {
+        b.src_off = so;
+        boxes.push_back(b);
+      } else {
+        b.rows = size[nd - 2];
+        b.src_pitch = ss[nd - 2] * es;
+        b.dst_pitch = row_bytes;
+        uint64_t outer = 1;
+        for (size_t d = 0; d + 2 < nd; ++d) outer *= size[d];
+        if (outer > (1u << 20)) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: too many row bands");
+        std::vector<uint64_t> idx(nd, 0);
+        for (uint64_t o = 0; o < outer; ++o) {
+          uint64_t s_el = 0, d_el = 0;
+          for (size_t d = 0; d + 2 < nd; ++d) { s_el += idx[d] * ss[d]; d_el += idx[d] * ds[d]; }
+          BoxCopy x = b;
+          x.src_off = so + s_el * es;
+          x.dst_off = d_el * es;
+          boxes.push_back(x);
+          for (int d = (int)nd - 3; d >= 0; --d) { if (++idx[d] < size[d]) break; idx[d] = 0; }
+        }
+      }
+      uint32_t sum = 0;
+      run_boxes(e, boxes, {sb}, {dst}, 1, checksum ? &sum : nullptr, stream);
+      if (checksum) *checksum = sum;
+      return;
+    }
+
+    // True transpose: i = destination innermost, j = the source's unit-stride dimension.
+    int c = -1;
+    for (size_t d = 0; d + 1 < nd; ++d)
+      if (ss[d] == 1) c = (int)d;
+    if (c < 0) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: the source has no unit-stride dimension");
+    if (nd - 2 > (size_t)kMaxBatchDims) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: too many batch dimensions");
+    TransposeDesc td{};
+    td.ni = size[nd - 1];
+    td.si = ss[nd - 1];
+    td.nj = size[c];
+    td.dj = ds[c];
+    const uint64_t tile_i = 512, tile_j = es == 1 ? 128 : es == 2 ? 64 : es == 4 ? 32 : 16;  // TileOf<ES>
+    td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
+    td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
+    bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * es) % 16 == 0;
+    bool vd = (td.dj * es) % 16 == 0;
+    int k = kMaxBatchDims - 1;
+    for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
+    for (int d = (int)nd - 2; d >= 0; --d) {
+      if (d == c) continue;
+      td.batch_size[k] = size[d];
+      td.batch_sstride[k] = ss[d];
+      td.batch_dstride[k] = ds[d];
+      vs = vs && (ss[d] * es) % 16 == 0;
+      vd = vd && (ds[d] * es) % 16 == 0;
+      --k;
+    }
+    td.vec_src = vs;
+    td.vec_dst = vd;
+    uint32_t* sum_dev = nullptr;
+    if (checksum) {
+      HIP_OK(hipStreamSynchronize(stream));
+      ensure_desc(e, 256);
+      sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
+      HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
+    }
+    HIP_OK(launch_transpose(src, dst, td, elem_size, sum_dev, stream));
+    if (checksum) {
+      HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
+      HIP_OK(hipStreamSynchronize(stream));
+      std::memcpy(checksum, e.desc_host, 4);
+    }
+  });
+}
+
 int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dsts, const uint64_t* nbytes, int64_t n,
                    uint32_t* out_checksums, void* stream) {
   return guard([&] {

@@ -71,6 +71,21 @@ struct WriteRec {
   uint64_t paired_runs = 0;
 };
 
+// A virtual checkpoint tensor assembled from boxes of real tensors: the published-tensor /
+// shard model of the reference's reshard path (a full shape plus shards at offsets).
+struct VirtualShard {
+  int64_t tensor = -1;                 // real source tensor
+  std::vector<int64_t> src_offset;     // box origin inside the source tensor
+  std::vector<int64_t> shard_offset;   // box origin inside the virtual tensor
+  std::vector<int64_t> shape;
+};
+struct VirtualRec {
+  std::string name;
+  std::vector<int64_t> shape;
+  int dtype = -1;
+  std::vector<VirtualShard> shards;
+};
+
 struct StackedRec { std::string fused, member; int order; };
 struct ExpertRec { std::string param_prefix, weight_prefix; int expert_id; std::string shard; int local_id; };
 
@@ -107,6 +122,7 @@ struct mxp_plan {
   std::vector<mxp::StackedRec> stacked;
   std::vector<mxp::ExpertRec> experts;
   std::vector<std::string> skip_prefixes;
+  std::vector<mxp::VirtualRec> virtuals;
   std::vector<mxp::WriteRec> writes;
   std::vector<std::string> skipped;  // tensors deliberately not placed
   bool built = false;

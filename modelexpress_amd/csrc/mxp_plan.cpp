@@ -350,6 +350,45 @@ struct Planner {
     }
   }
 
+  // A write whose source is a virtual tensor: intersect the needed box with every shard
+  // (refit/reshard/slice_plan.py:248-256,297-339) and emit one strided copy per overlap.
+  void emit_virtual(const VirtualRec& v, int kind, const View& local, const View& dest) {
+    const size_t nd = v.shape.size();
+    const Shape vs = row_major(v.shape);
+    Shape lo(nd), ext(nd);
+    int64_t want = 1, got = 0;
+    for (size_t d = 0; d < nd; ++d) {
+      lo[d] = v.shape[d] ? (local.base / vs[d]) % v.shape[d] : 0;
+      ext[d] = local.shape[d];
+      want *= ext[d];
+    }
+    for (const auto& sh : v.shards) {
+      const TensorRec& t = ck.tensors[sh.tensor];
+      const Shape ts = row_major(t.shape);
+      View sv, dv = dest;
+      sv.shape.resize(nd);
+      sv.stride = ts;
+      bool empty = false;
+      int64_t vol = 1;
+      for (size_t d = 0; d < nd; ++d) {
+        const int64_t a = std::max(lo[d], sh.shard_offset[d]);
+        const int64_t b = std::min(lo[d] + ext[d], sh.shard_offset[d] + sh.shape[d]);
+        if (a >= b) { empty = true; break; }
+        sv.base += (sh.src_offset[d] + a - sh.shard_offset[d]) * ts[d];
+        sv.shape[d] = b - a;
+        dv.base += (a - lo[d]) * dest.stride[d];
+        dv.shape[d] = b - a;
+        vol *= b - a;
+      }
+      if (empty) continue;
+      got += vol;
+      emit_writes(sh.tensor, kind, sv, dv);
+    }
+    if (got != want)
+      throw Error(MXP_ERR_COVERAGE, "virtual tensor '" + v.name + "': its shards cover " + std::to_string(got) +
+                                        " of the " + std::to_string(want) + " elements this rank needs");
+  }
+
   // The fp8 block rule made explicit: when a weight has a companion scale of shape
   // [ceil(N/128), ceil(K/128)], a slice of the weight must start and end on 128
   // boundaries so the same shape rule applied to the scale selects exactly its tiles.
@@ -391,20 +430,36 @@ struct Planner {
       for (const auto& c : counts) if (c.second == 2) premerge_suffixes.push_back(c.first);
     }
 
-    std::vector<int64_t> todo;
-    for (int64_t i = 0; i < (int64_t)ck.tensors.size(); ++i) {
-      bool skip = false;
+    // Items to place: every real tensor that no virtual tensor consumes, then the virtual ones.
+    struct Item { const std::string* name; const Shape* shape; int64_t real, virt; };
+    std::vector<Item> todo;
+    std::set<int64_t> consumed;
+    for (const auto& v : pl.virtuals) {
+      if (v.shards.empty()) throw Error(MXP_ERR_ARG, "virtual tensor '" + v.name + "' has no shards");
+      if (ck.by_name.count(v.name)) throw Error(MXP_ERR_ARG, "virtual tensor '" + v.name + "' shadows a checkpoint tensor");
+      for (const auto& sh : v.shards) consumed.insert(sh.tensor);
+    }
+    auto skipped_by_prefix = [&](const std::string& n) {
       for (const auto& pre : pl.skip_prefixes)
-        if (ck.tensors[i].name.compare(0, pre.size(), pre) == 0) skip = true;
-      if (skip) pl.skipped.push_back(ck.tensors[i].name); else todo.push_back(i);
+        if (n.compare(0, pre.size(), pre) == 0) return true;
+      return false;
+    };
+    for (int64_t i = 0; i < (int64_t)ck.tensors.size(); ++i) {
+      if (consumed.count(i)) continue;
+      if (skipped_by_prefix(ck.tensors[i].name)) pl.skipped.push_back(ck.tensors[i].name);
+      else todo.push_back(Item{&ck.tensors[i].name, &ck.tensors[i].shape, i, -1});
+    }
+    for (int64_t i = 0; i < (int64_t)pl.virtuals.size(); ++i) {
+      if (skipped_by_prefix(pl.virtuals[i].name)) pl.skipped.push_back(pl.virtuals[i].name);
+      else todo.push_back(Item{&pl.virtuals[i].name, &pl.virtuals[i].shape, -1, i});
     }
 
     // ---- classification (installer.py:470-564) ----
     std::vector<std::pair<int64_t, std::vector<Member>>> groups;
     std::unordered_map<int64_t, size_t> group_index;
-    std::set<int64_t> skipped_experts;
-    for (int64_t ti : todo) {
-      const TensorRec& t = ck.tensors[ti];
+    std::set<const std::string*> skipped_experts;
+    for (const Item& it : todo) {
+      struct { const std::string& name; const Shape& shape; } t{*it.name, *it.shape};
       int64_t pm_param;
       if (premerged_destination(t.name, t.shape, premerge_suffixes, pm_param)) {
         premerged[t.name] = {pm_param, 2};
@@ -421,7 +476,7 @@ struct Planner {
         View dest;
         const int r = resolve_expert(t.name, t.shape, dest);
         if (r == 1) { expert[t.name] = dest; covered.insert(dest.param); continue; }
-        if (r == 2) { skipped_experts.insert(ti); continue; }
+        if (r == 2) { skipped_experts.insert(it.name); continue; }
       }
       for (const auto& g : groups_def) {
         if (contains(t.name, g.member + ".") || ends_with(t.name, g.member + ".weight")) {
@@ -445,9 +500,17 @@ struct Planner {
 
     // ---- resolution (installer.py:341-410): every write before any copy ----
     std::vector<std::string> unmapped;
-    for (int64_t ti : todo) {
-      const TensorRec& t = ck.tensors[ti];
-      if (skipped_experts.count(ti)) { pl.skipped.push_back(t.name); continue; }
+    auto emit = [&](const Item& it, int kind, const View& sv, const View& dv) {
+      if (it.real >= 0) {
+        check_fp8_blocks(ck.tensors[it.real], sv);
+        emit_writes(it.real, kind, sv, dv);
+      } else {
+        emit_virtual(pl.virtuals[it.virt], kind, sv, dv);
+      }
+    };
+    for (const Item& it : todo) {
+      struct { const std::string& name; const Shape& shape; } t{*it.name, *it.shape};
+      if (skipped_experts.count(it.name)) { pl.skipped.push_back(t.name); continue; }
       const View src = full_view(t.shape);
       auto pm = premerged.find(t.name);
       if (pm != premerged.end()) {
@@ -464,8 +527,7 @@ struct Planner {
         for (int part = 0; part < parts; ++part) {
           const View sv = narrow(src, 0, part * part_src + (int64_t)rank * part_dst, part_dst);
           const View dv = narrow(dfull, 0, part * part_dst, part_dst);
-          check_fp8_blocks(t, sv);
-          emit_writes(ti, MXP_WRITE_PREMERGED, sv, dv);
+          emit(it, MXP_WRITE_PREMERGED, sv, dv);
         }
         continue;
       }
@@ -486,8 +548,7 @@ struct Planner {
         unmapped.push_back(t.name);
         continue;
       }
-      check_fp8_blocks(t, local);
-      emit_writes(ti, kind, local, dest);
+      emit(it, kind, local, dest);
     }
 
     // ---- coverage (installer.py:219-251), extended to every parameter ----
@@ -637,6 +698,56 @@ int mxp_plan_add_skip_prefix(mxp_plan* plan, const char* prefix) {
     if (!plan || !prefix) throw Error(MXP_ERR_ARG, "mxp_plan_add_skip_prefix: null argument");
     if (plan->built) throw Error(MXP_ERR_STATE, "plan is already built");
     plan->skip_prefixes.push_back(prefix);
+  });
+}
+
+int64_t mxp_plan_add_virtual(mxp_plan* plan, const char* name, int32_t ndim, const int64_t* full_shape) {
+  int64_t idx = -1;
+  const int rc = guard([&] {
+    if (!plan || !name || ndim < 0 || ndim > MXP_MAX_DIMS || (ndim && !full_shape))
+      throw Error(MXP_ERR_ARG, "mxp_plan_add_virtual: bad argument");
+    if (plan->built) throw Error(MXP_ERR_STATE, "plan is already built");
+    for (const auto& v : plan->virtuals)
+      if (v.name == name) throw Error(MXP_ERR_ARG, std::string("duplicate virtual tensor ") + name);
+    VirtualRec v;
+    v.name = name;
+    for (int d = 0; d < ndim; ++d) {
+      if (full_shape[d] < 0) throw Error(MXP_ERR_ARG, "negative dimension");
+      v.shape.push_back(full_shape[d]);
+    }
+    idx = (int64_t)plan->virtuals.size();
+    plan->virtuals.push_back(std::move(v));
+  });
+  return rc == MXP_OK ? idx : rc;
+}
+
+int mxp_plan_add_virtual_shard(mxp_plan* plan, int64_t virtual_index, const char* source_tensor,
+                               const int64_t* source_offset, const int64_t* shard_offset, const int64_t* shape) {
+  return guard([&] {
+    if (!plan || !source_tensor || virtual_index < 0 || virtual_index >= (int64_t)plan->virtuals.size())
+      throw Error(MXP_ERR_ARG, "mxp_plan_add_virtual_shard: bad argument");
+    if (plan->built) throw Error(MXP_ERR_STATE, "plan is already built");
+    VirtualRec& v = plan->virtuals[virtual_index];
+    auto it = plan->ckpt->by_name.find(source_tensor);
+    if (it == plan->ckpt->by_name.end())
+      throw Error(MXP_ERR_ARG, std::string("virtual shard source '") + source_tensor + "' is not in the checkpoint");
+    const TensorRec& t = plan->ckpt->tensors[it->second];
+    const size_t nd = v.shape.size();
+    if (t.shape.size() != nd) throw Error(MXP_ERR_ARG, "virtual shard: rank mismatch with '" + t.name + "'");
+    if (nd && (!source_offset || !shard_offset || !shape)) throw Error(MXP_ERR_ARG, "virtual shard: null box");
+    if (v.dtype >= 0 && v.dtype != t.dtype) throw Error(MXP_ERR_ARG, "virtual tensor '" + v.name + "' mixes dtypes");
+    VirtualShard sh;
+    sh.tensor = it->second;
+    for (size_t d = 0; d < nd; ++d) {
+      if (shape[d] < 0 || source_offset[d] < 0 || shard_offset[d] < 0 || source_offset[d] + shape[d] > t.shape[d] ||
+          shard_offset[d] + shape[d] > v.shape[d])
+        throw Error(MXP_ERR_ARG, "virtual shard of '" + v.name + "' leaves its source or the virtual tensor");
+      sh.src_offset.push_back(source_offset[d]);
+      sh.shard_offset.push_back(shard_offset[d]);
+      sh.shape.push_back(shape[d]);
+    }
+    v.dtype = t.dtype;
+    v.shards.push_back(std::move(sh));
   });
 }
 

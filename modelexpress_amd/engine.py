@@ -41,6 +41,16 @@ class ParamSpec:
 
 
 @dataclass(frozen=True)
+class VirtualTensor:
+    """A checkpoint tensor assembled from boxes of real tensors.  ``shards`` rows are
+    ``(source_tensor_name, source_offset, shard_offset, shape)`` with per-dimension tuples."""
+
+    name: str
+    shape: tuple
+    shards: tuple
+
+
+@dataclass(frozen=True)
 class WriteEntry:
     tensor: str
     param: str
@@ -116,7 +126,8 @@ class PlacementPlan:
 
     def __init__(self, ckpt: Checkpoint, params: Iterable[ParamSpec], *, tp_size: int = 1, tp_rank: int = 0,
                  stacked_params_mapping: Sequence | None = None, expert_mapping: Sequence | None = None,
-                 skip_prefixes: Sequence[str] = (), allow_cast: bool = False, allow_unmapped: bool = False,
+                 skip_prefixes: Sequence[str] = (), virtual_tensors: Sequence[VirtualTensor] = (),
+                 allow_cast: bool = False, allow_unmapped: bool = False,
                  allow_uncovered: bool = False, fp8_block_check: bool = True):
         lib = L.lib()
         self.ckpt = ckpt
@@ -140,6 +151,13 @@ class PlacementPlan:
             L.check(lib.mxp_plan_add_expert(self._h, p_pre.encode(), w_pre.encode(), int(eid), shard.encode(), local))
         for pre in skip_prefixes:
             L.check(lib.mxp_plan_add_skip_prefix(self._h, pre.encode()))
+        for v in virtual_tensors:
+            nd = len(v.shape)
+            arr = lambda t: (C.c_int64 * max(1, nd))(*[int(x) for x in t])  # noqa: E731
+            vi = L.check(lib.mxp_plan_add_virtual(self._h, v.name.encode(), nd, arr(v.shape)))
+            for source, src_off, shard_off, shape in v.shards:
+                L.check(lib.mxp_plan_add_virtual_shard(self._h, vi, source.encode(), arr(src_off), arr(shard_off),
+                                                       arr(shape)))
         L.check(lib.mxp_plan_build(self._h))
 
     def close(self) -> None:
@@ -351,6 +369,18 @@ class PlacementEngine:
                               "csum_index": k * piece})
         sums = self.place_boxes(boxes, 1, stream=stream)
         return out, sums[0]
+
+    def permute_copy(self, src, dst, shape: Sequence[int], perm: Sequence[int], elem_size: int, *,
+                     src_strides: Sequence[int] | None = None, stream: int = 0, checksum: bool = True) -> str | None:
+        """``dst = src.permute(perm).contiguous()`` on the device (row gather or LDS transpose)."""
+        n = len(shape)
+        shp = (C.c_int64 * max(1, n))(*[int(v) for v in shape])
+        prm = (C.c_int32 * max(1, n))(*[int(v) for v in perm])
+        strides = None if src_strides is None else (C.c_int64 * max(1, n))(*[int(v) for v in src_strides])
+        out = C.c_uint32()
+        L.check(L.lib().mxp_permute_copy(self._h, C.c_void_p(_addr(src)), C.c_void_p(_addr(dst)), n, shp, strides, prm,
+                                         elem_size, C.byref(out) if checksum else None, C.c_void_p(stream)))
+        return format(out.value, "08x") if checksum else None
 
     def copy_batch(self, srcs: Sequence, dsts: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
                    checksums: bool = True) -> list[str] | None:

@@ -344,6 +344,60 @@ def paired_runs(overlap, src_origin, src_strides, dst_origin, dst_strides):
 
 
 # --------------------------------------------------------------------------------------
+# permuted copies: ``dest.copy_(src.permute(...))`` -- the MLA absorbed weights
+# W_UV = w_uv.transpose(0, 1), W_UK_T = w_uk.permute(1, 2, 0)
+# (engines/vllm/refit/receiver.py:244-261) and permuted box views (slice_plan.py:166-220)
+# --------------------------------------------------------------------------------------
+def permute_copy(t: OTensor, perm) -> OTensor:
+    """Contiguous copy of ``t.permute(perm)``; the element-byte axis stays last."""
+    axes = tuple(int(p) for p in perm) + (t.data.ndim - 1,)
+    return OTensor(np.ascontiguousarray(np.transpose(t.data, axes)), t.dtype)
+
+
+def mla_absorbed_weights(kv_b_proj: OTensor, num_heads: int, qk_nope: int, v_head: int) -> tuple:
+    """receiver.py:244-261: view [H, nope+v, L], split on dim 1, then W_UV = w_uv.transpose(0,1)
+    -> [v, H, L] and W_UK_T = w_uk.permute(1,2,0) -> [nope, L, H]."""
+    es = kv_b_proj.data.shape[-1]
+    v3 = _reshape_view(np.ascontiguousarray(kv_b_proj.data), (num_heads, qk_nope + v_head, -1, es))
+    w_uk = OTensor(v3[:, :qk_nope], kv_b_proj.dtype)
+    w_uv = OTensor(v3[:, qk_nope:], kv_b_proj.dtype)
+    return permute_copy(w_uv, (1, 0, 2)), permute_copy(w_uk, (1, 2, 0))
+
+
+# --------------------------------------------------------------------------------------
+# trainer-native layouts (modelexpress_rl/train/engines/megatron/aliases.py)
+# --------------------------------------------------------------------------------------
+def megatron_qkv_split(fused: OTensor, q_heads: int, kv_heads: int, head_dim: int) -> tuple:
+    """Whole q, k, v from a by-KV-group interleaved fused tensor (aliases.py:206-263: per
+    group its query rows, then one K head, then one V head)."""
+    q_rows = (q_heads // kv_heads) * head_dim
+    group_rows = q_rows + 2 * head_dim
+    q, k, v = [], [], []
+    for g in range(kv_heads):
+        lo = g * group_rows
+        q.append(fused.data[lo : lo + q_rows])
+        k.append(fused.data[lo + q_rows : lo + q_rows + head_dim])
+        v.append(fused.data[lo + q_rows + head_dim : lo + group_rows])
+    return tuple(OTensor(np.concatenate(parts), fused.dtype) for parts in (q, k, v))
+
+
+def assemble_virtual(full_shape, dtype: str, shards) -> OTensor:
+    """A full tensor assembled from shards ``(source OTensor, source_offset, shard_offset,
+    shape)``: what a receiver builds when it stages a whole logical tensor from its
+    publishers (refit/reshard/transfer_plan.py:134-189) before re-slicing it."""
+    out = OTensor.zeros(full_shape, dtype)
+    hit = np.zeros(tuple(full_shape), dtype=np.int32)
+    for src, src_off, shard_off, shape in shards:
+        s_idx = tuple(slice(o, o + n) for o, n in zip(src_off, shape))
+        d_idx = tuple(slice(o, o + n) for o, n in zip(shard_off, shape))
+        out.data[d_idx] = src.data[s_idx]
+        hit[d_idx] += 1
+    if not np.all(hit == 1):
+        raise CoverageError("virtual tensor shards leave gaps or overlap")
+    return out
+
+
+# --------------------------------------------------------------------------------------
 # a4-a8: destination map and writes (engines/vllm/refit/installer.py)
 # --------------------------------------------------------------------------------------
 STACKED_GROUPS = (  # installer.py:72-78

@@ -171,3 +171,49 @@ def test_shard_region_matches_oracle(gpu_engine, oracle):
         want = oracle.shard_region(OT.from_array(big.reshape(-1), "BF16"), big.shape, off, shp)
         assert buf.cpu().numpy().tobytes() == want.tobytes(), (off, shp)
         assert csum == oracle.safe_checksum(want)
+
+
+@pytest.mark.parametrize("shape,perm,es", [
+    ((3, 4), (1, 0), 4),                 # test_reshard_refit_slice_plan.py:155-167
+    ((2, 3, 4), (2, 0, 1), 4),           # :170-183
+    ((64, 64), (1, 0), 2),
+    ((130, 67), (1, 0), 2),              # ragged tiles, element-wise edges
+    ((257, 129), (1, 0), 1),
+    ((100, 72), (1, 0), 8),
+    ((5, 96, 80), (0, 2, 1), 2),         # batched transposes
+    ((16, 128, 512), (1, 2, 0), 2),      # W_UK_T shape of one TP=8 rank: [heads, nope, lora] -> [nope, lora, heads]
+    ((16, 128, 512), (1, 0, 2), 2),      # W_UV: keeps the innermost dim -> row gather
+    ((7, 5, 6, 9), (3, 1, 0, 2), 4),     # 4-D
+    ((6, 1, 33), (2, 1, 0), 2),          # unit dim dropped
+    ((1000,), (0,), 2),
+])
+def test_permute_copy_matches_oracle(gpu_engine, oracle, oracle_c, shape, perm, es):
+    rng = np.random.default_rng(17)
+    n = int(np.prod(shape))
+    raw = rng.integers(0, 256, n * es, dtype=np.uint8)
+    dtype = {1: "U8", 2: "BF16", 4: "F32", 8: "I64"}[es]
+    src = oracle.OTensor(raw.reshape(tuple(shape) + (es,)), dtype)
+    want = oracle.permute_copy(src, perm)
+    d = torch.full((n * es + 16,), 0xEE, dtype=torch.uint8, device="cuda")
+    csum = gpu_engine.permute_copy(_dev(raw), d, shape, perm, es)
+    assert d[: n * es].cpu().numpy().tobytes() == want.tobytes()
+    assert int((d[n * es:] != 0xEE).sum()) == 0
+    assert csum == oracle_c.checksum32(np.frombuffer(want.tobytes(), dtype=np.uint8))
+
+
+def test_mla_absorbed_weights_on_device(gpu_engine, oracle, oracle_c):
+    # engines/vllm/refit/receiver.py:244-261 on a strided view of kv_b_proj (no intermediate copy)
+    H, nope, v, L, es = 16, 128, 128, 512, 2
+    rng = np.random.default_rng(18)
+    raw = rng.integers(0, 256, H * (nope + v) * L * es, dtype=np.uint8)
+    kv_b = oracle.OTensor(raw.reshape(H * (nope + v), L, es), "BF16")
+    want_uv, want_ukt = oracle.mla_absorbed_weights(kv_b, H, nope, v)
+    d = _dev(raw)
+    strides = ((nope + v) * L, L, 1)
+    uv = torch.zeros(v * H * L * es, dtype=torch.uint8, device="cuda")
+    ukt = torch.zeros(nope * L * H * es, dtype=torch.uint8, device="cuda")
+    c_uv = gpu_engine.permute_copy(d[nope * L * es:], uv, (H, v, L), (1, 0, 2), es, src_strides=strides)
+    c_ukt = gpu_engine.permute_copy(d, ukt, (H, nope, L), (1, 2, 0), es, src_strides=strides)
+    assert uv.cpu().numpy().tobytes() == want_uv.tobytes()
+    assert ukt.cpu().numpy().tobytes() == want_ukt.tobytes()
+    assert c_uv == oracle.safe_checksum(want_uv) and c_ukt == oracle.safe_checksum(want_ukt)

@@ -66,3 +66,43 @@ def test_direct_io_ranges_match_oracle(name, oracle, tmp_path, mxp):
     with pytest.raises(mxp.MxpError, match="direct I/O"):
         PlacementEngine(0, use_o_direct=True, pack_strided_on_host=True)
     eng.close()
+
+
+def test_megatron_interleaved_qkv_refit_on_device(gpu_engine, gpu_engine_band, oracle, tmp_path, mxp):
+    """A trainer-native source (fp32, by-KV-group interleaved linear_qkv saved as two row
+    shards, fused [gate; up]) placed into a serving rank's bf16 qkv_proj / gate_up_proj:
+    de-interleave + TP slice + fuse + cast + checksum in one pass."""
+    from safetensors.torch import save_file
+    from modelexpress_amd import megatron
+    from modelexpress_amd.engine import Checkpoint, ParamSpec, PlacementPlan
+
+    q_heads, kv_heads, head_dim, hidden, ffn, src_tp, dst_tp = 8, 2, 16, 64, 96, 2, 2
+    g = torch.Generator().manual_seed(5)
+    rows = (q_heads + 2 * kv_heads) * head_dim
+    fused = torch.randn(rows, hidden, generator=g)
+    fc1 = [torch.randn(2 * ffn // src_tp, hidden, generator=g) for _ in range(src_tp)]
+    local = rows // src_tp
+    tensors = {f"l0.linear_qkv.rank{r}": fused[r * local:(r + 1) * local].clone() for r in range(src_tp)}
+    tensors.update({f"l0.linear_fc1.rank{r}": fc1[r] for r in range(src_tp)})
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    virtuals = megatron.qkv_virtuals([(f"l0.linear_qkv.rank{r}", r * local, (r + 1) * local) for r in range(src_tp)],
+                                     ("l0.q_proj.weight", "l0.k_proj.weight", "l0.v_proj.weight"), hidden,
+                                     head_dim=head_dim, q_heads=q_heads, kv_heads=kv_heads)
+    virtuals += megatron.gated_virtuals([(f"l0.linear_fc1.rank{r}", r, src_tp) for r in range(src_tp)],
+                                        ("l0.gate_proj.weight", "l0.up_proj.weight"), (hidden,), global_rows=2 * ffn)
+    ow = dict(oracle.load_checkpoint(str(tmp_path)))
+    weights = [(v.name, oracle.assemble_virtual(v.shape, "F32", [(ow[s], so, do, sh) for s, so, do, sh in v.shards]))
+               for v in virtuals]
+    ck = Checkpoint(str(tmp_path))
+    for rank in range(dst_tp):
+        params = [ParamSpec("l0.qkv_proj.weight", "BF16", ((q_heads + 2 * kv_heads) * head_dim // dst_tp, hidden)),
+                  ParamSpec("l0.gate_up_proj.weight", "BF16", (2 * ffn // dst_tp, hidden))]
+        oparams = {p.name: oracle.OTensor.zeros(p.shape, p.dtype) for p in params}
+        oracle.MdlOracle(oparams, dst_tp, rank, allow_cast=True).load_weights(weights)
+        plan = PlacementPlan(ck, params, tp_size=dst_tp, tp_rank=rank, virtual_tensors=virtuals, allow_cast=True)
+        for eng in (gpu_engine, gpu_engine_band):
+            dst = eng.allocate(plan, fill=0x77)
+            eng.execute(plan, dst)
+            for p, d, s in zip(params, dst, eng.checksums(plan)):
+                assert d.cpu().numpy().tobytes() == oparams[p.name].tobytes(), (rank, p.name)
+                assert s == oracle.safe_checksum(oparams[p.name])

@@ -303,3 +303,30 @@ def test_parse_errors_and_resolution_order(oracle, tmp_path):
     (d / "model.safetensors.index.json").write_text(json.dumps({"weight_map": {}}))
     with pytest.raises(RuntimeError, match="Empty weight_map"):
         oracle.resolve_safetensors_files(str(d))
+
+
+# ---------------------------------------------------------------- permuted copies ----
+def test_permute_copy_reference_vectors(oracle):
+    # tests/test_reshard_refit_slice_plan.py:155-197: transpose, 3-D permute, narrow+transpose
+    OT = oracle.OTensor
+    src = torch.arange(12, dtype=torch.float32).reshape(3, 4)
+    got = oracle.permute_copy(OT.from_array(src.numpy(), "F32"), (1, 0))
+    assert got.tobytes() == src.transpose(0, 1).contiguous().numpy().tobytes() and got.shape == (4, 3)
+    src = torch.arange(24, dtype=torch.float32).reshape(2, 3, 4)
+    got = oracle.permute_copy(OT.from_array(src.numpy(), "F32"), (2, 0, 1))
+    assert got.tobytes() == src.permute(2, 0, 1).contiguous().numpy().tobytes() and got.shape == (4, 2, 3)
+    src = torch.arange(20, dtype=torch.float32).reshape(4, 5)
+    got = oracle.permute_copy(OT.from_array(src.numpy(), "F32").narrow(0, 1, 2), (1, 0))
+    assert got.tobytes() == src.narrow(0, 1, 2).transpose(0, 1).contiguous().numpy().tobytes()
+
+
+def test_mla_absorbed_weights_match_torch(oracle):
+    # engines/vllm/refit/receiver.py:244-261 restated with torch ops as the reference composes them
+    H, nope, v, L = 4, 6, 5, 7
+    w = torch.arange(H * (nope + v) * L, dtype=torch.float32).reshape(H * (nope + v), L)
+    view = w.view(H, nope + v, -1)
+    w_uk, w_uv = view.split([nope, v], dim=1)
+    uv, ukt = oracle.mla_absorbed_weights(oracle.OTensor.from_array(w.numpy(), "F32"), H, nope, v)
+    assert uv.shape == (v, H, L) and ukt.shape == (nope, L, H)
+    assert uv.tobytes() == w_uv.transpose(0, 1).contiguous().numpy().tobytes()
+    assert ukt.tobytes() == w_uk.permute(1, 2, 0).contiguous().numpy().tobytes()
