@@ -336,6 +336,15 @@ int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double*
 /* blake2b-128 over the scalar list tensor_digest would hash (verify.py:152-155). */
 int mxp_digest_from_scalars(const uint64_t scalars[7], uint8_t out16[16]);
 
+/* CRC32C (Castagnoli) as the artifact manifest uses it: mxp_crc32c continues a finished
+ * CRC (`seed` = 0 to start), like crc32c_append; mxp_file_crc32c gives the whole-file
+ * checksum and one checksum per `chunk_size` piece (the last may be shorter; an empty file
+ * has no chunks) -- file_checksum / chunks_for_file of
+ * modelexpress_common/src/artifact_manifest.rs:260-324. */
+uint32_t mxp_crc32c(uint32_t seed, const void* data, uint64_t nbytes);
+int mxp_file_crc32c(const char* path, uint64_t chunk_size, uint32_t* file_crc, uint32_t* chunk_crcs,
+                    uint64_t max_chunks, uint64_t* n_chunks);
+
 /* Seeded synthetic contents (test and benchmark inputs; same bytes on host and device).
  * kind: 0 ~N(0,0.02), 1 ones, 2 zeros, 3 normal with denormal/inf/NaN/tie edge cases at
  * 1e-6 density, 4 fp8 bytes over the finite e4m3 codes, 5 fp32 scales in [1e-4,1e-2],

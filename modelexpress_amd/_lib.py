@@ -146,6 +146,8 @@ SIGNATURES = {
     "mxp_copy_batch": (C.c_int, [_P, _PP, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_digest_from_scalars": (C.c_int, [_U64P, C.POINTER(C.c_uint8)]),
+    "mxp_crc32c": (C.c_uint32, [C.c_uint32, _P, C.c_uint64]),
+    "mxp_file_crc32c": (C.c_int, [C.c_char_p, C.c_uint64, _U32P, _U32P, C.c_uint64, _U64P]),
     "mxp_synth_host": (C.c_int, [_P, C.c_uint64, C.c_int32, C.c_uint32, C.c_uint64, C.c_int32]),
     "mxp_synth_device": (C.c_int, [_P, C.c_uint64, C.c_int32, C.c_uint32, C.c_uint64, _P]),
 }

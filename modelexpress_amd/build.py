@@ -25,6 +25,7 @@ SOURCES = (
     "mxp_ckpt.cpp",
     "mxp_plan.cpp",
     "mxp_engine.cpp",
+    "mxp_crc32c.cpp",
 )
 
 # -packed-fp32-ops is switched off on purpose for every device compile: the packed fp32
