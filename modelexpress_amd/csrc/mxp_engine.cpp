@@ -110,8 +110,11 @@ struct mxp_engine {
   size_t desc_host_cap = 0;
   DevBuf<uint8_t> desc_dev;
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
+  hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
+  bool arena_recorded = false;
 
   ~mxp_engine() {
+    if (arena_busy) (void)hipEventDestroy(arena_busy);
     for (auto s : streams) (void)hipStreamDestroy(s);
     for (auto& s : slots)
       if (s->done) (void)hipEventDestroy(s->done);
@@ -339,6 +342,18 @@ void pread_full(int fd, uint8_t* dst, uint64_t n, uint64_t off, const std::strin
   }
 }
 
+// The descriptor arena (pinned staging + its device twin) is shared by the stand-alone
+// operators.  A call may only overwrite or reallocate it once the previous user's device
+// work is done, whichever stream that ran on: users record `arena_busy` after their last
+// arena-dependent operation (release_arena) and wait for it before touching the arena.
+void acquire_arena(mxp_engine& e) {
+  if (e.arena_recorded) HIP_OK(hipEventSynchronize(e.arena_busy));
+}
+void release_arena(mxp_engine& e, hipStream_t stream) {
+  HIP_OK(hipEventRecord(e.arena_busy, stream));
+  e.arena_recorded = true;
+}
+
 void ensure_desc(mxp_engine& e, size_t bytes) {
   if (bytes > e.desc_host_cap) {
     if (e.desc_host) (void)hipHostFree(e.desc_host);
@@ -366,7 +381,7 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
   const size_t o_dst = align_up(o_src + srcs.size() * sizeof(void*), 256);
   const size_t o_sum = align_up(o_dst + dsts.size() * sizeof(void*), 256);
   const size_t total = align_up(o_sum + (size_t)n_sums * 4, 256);
-  HIP_OK(hipStreamSynchronize(stream));  // the arena may still feed an earlier launch
+  acquire_arena(e);
   ensure_desc(e, total);
   std::memset(e.desc_host, 0, total);
   if (!segs.empty()) std::memcpy(e.desc_host + o_segs, segs.data(), segs.size() * sizeof(Seg));
@@ -385,9 +400,8 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
     HIP_OK(hipMemcpyAsync(e.desc_host + o_sum, d + o_sum, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
     std::memcpy(sums_out, e.desc_host + o_sum, (size_t)n_sums * 4);
-  } else {
-    // the pinned arena is read by the copy above; later calls synchronise before reuse
   }
+  release_arena(e, stream);
 }
 
 // Splits an arbitrary device pointer into a 16-byte aligned base and an offset, so the
@@ -437,6 +451,7 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     }
     HIP_OK(hipEventCreate(&e->ev_a));
     HIP_OK(hipEventCreate(&e->ev_b));
+    HIP_OK(hipEventCreateWithFlags(&e->arena_busy, hipEventDisableTiming));
     *out = e.release();
   });
 }
@@ -950,7 +965,7 @@ int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndi
     td.vec_dst = vd;
     uint32_t* sum_dev = nullptr;
     if (checksum) {
-      HIP_OK(hipStreamSynchronize(stream));
+      acquire_arena(e);
       ensure_desc(e, 256);
       sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
       HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
@@ -960,6 +975,7 @@ int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndi
       HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
       HIP_OK(hipStreamSynchronize(stream));
       std::memcpy(checksum, e.desc_host, 4);
+      release_arena(e, stream);
     }
   });
 }
@@ -1045,7 +1061,7 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
     const size_t o_jobs = 0;
     const size_t o_out = align_up(jobs.size() * sizeof(DigestJob), 256);
     const size_t total = o_out + (size_t)n * 5 * 8;
-    HIP_OK(hipStreamSynchronize(stream));
+    acquire_arena(e);
     ensure_desc(e, total);
     std::memset(e.desc_host, 0, total);
     std::memcpy(e.desc_host + o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
@@ -1054,6 +1070,7 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
                          reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_out), stream));
     HIP_OK(hipMemcpyAsync(e.desc_host + o_out, e.desc_dev.p + o_out, (size_t)n * 5 * 8, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
+    release_arena(e, stream);
     const uint64_t* sums = reinterpret_cast<const uint64_t*>(e.desc_host + o_out);
     for (int64_t k = 0; k < n; ++k) {
       uint64_t sc[7] = {nbytes[k], sums[5 * k], sums[5 * k + 1], sums[5 * k + 2], sums[5 * k + 3], sums[5 * k + 4],

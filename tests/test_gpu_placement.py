@@ -106,3 +106,67 @@ def test_megatron_interleaved_qkv_refit_on_device(gpu_engine, gpu_engine_band, o
             for p, d, s in zip(params, dst, eng.checksums(plan)):
                 assert d.cpu().numpy().tobytes() == oparams[p.name].tobytes(), (rank, p.name)
                 assert s == oracle.safe_checksum(oparams[p.name])
+
+
+def test_resident_placement_replays_from_a_hip_graph(gpu_engine, oracle, tmp_path, mxp):
+    """The resident step is two kernel launches (accumulator clear by a fill kernel, then
+    place_kernel) and no allocation or memset node, so it can be captured.  Every replay is
+    checked against the eager result, with eager work and synchronisation between replays."""
+    layout, tp, ep, shards, ck_kw = tiny_layouts()["llama_tp4"]
+    synth.write_checkpoint(layout.checkpoint(), str(tmp_path), n_shards=shards, seed=31)
+    rv = layout.rank_view(tp_size=tp, tp_rank=2)
+    ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=2)
+    staged = _stage_files(ck)
+    dst = gpu_engine.allocate(plan, fill=0)
+    gpu_engine.execute_resident(plan, staged, dst)  # eager: also caches the pointer tables
+    torch.cuda.synchronize()
+    eager_sums = gpu_engine.checksums(plan)
+    eager = [d.clone() for d in dst]
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            gpu_engine.execute_resident(plan, staged, dst, stream=torch.cuda.current_stream().cuda_stream)
+    for replay in range(3):
+        for d in dst:
+            d.fill_(replay + 1)  # eager work between replays; also proves the replay rewrites everything
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert gpu_engine.checksums(plan) == eager_sums, replay
+        assert all(torch.equal(a, b) for a, b in zip(eager, dst)), replay
+    # a replay reads the staged bytes anew: change one source byte and the output follows
+    t = [x for x in ck.tensors() if x.name == "model.norm.weight"][0]
+    staged[t.file_index][t.file_offset] ^= 0xFF
+    graph.replay()
+    torch.cuda.synchronize()
+    idx = [p.name for p in plan.params].index("model.norm.weight")
+    assert gpu_engine.checksums(plan)[idx] != eager_sums[idx]
+
+
+def test_empty_and_scalar_tensors(gpu_engine, gpu_engine_band, oracle, tmp_path, mxp):
+    """Zero-element tensors, 0-dim tensors and odd byte counts through the whole path."""
+    from safetensors.torch import save_file
+    from modelexpress_amd.engine import Checkpoint, ParamSpec, PlacementPlan
+
+    tensors = {"empty.weight": torch.zeros((0, 4)), "scalar.weight": torch.tensor(2.5),
+               "odd.weight": torch.arange(7, dtype=torch.uint8), "one.weight": torch.tensor([1.0], dtype=torch.bfloat16),
+               "a.q_proj.input_scale": torch.tensor(0.5), "a.k_proj.input_scale": torch.tensor(1.5),
+               "a.v_proj.input_scale": torch.tensor(2.5)}
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    params = [ParamSpec("empty.weight", "F32", (0, 4)), ParamSpec("scalar.weight", "F32", ()),
+              ParamSpec("odd.weight", "U8", (7,)), ParamSpec("one.weight", "BF16", (1,)),
+              ParamSpec("a.qkv_proj.input_scale", "F32", (3,))]
+    ow = oracle.load_checkpoint(str(tmp_path))
+    oparams = {p.name: oracle.OTensor.zeros(p.shape, p.dtype) for p in params}
+    oracle.MdlOracle(oparams).load_weights(ow)
+    assert oparams["a.qkv_proj.input_scale"].tobytes() == np.array([0.5, 1.5, 2.5], dtype=np.float32).tobytes()
+    ck = Checkpoint(str(tmp_path))
+    plan = PlacementPlan(ck, params)
+    for eng in (gpu_engine, gpu_engine_band):
+        dst = eng.allocate(plan, fill=0xEE)
+        eng.execute(plan, dst)
+        for p, d, s in zip(params, dst, eng.checksums(plan)):
+            assert d.cpu().numpy().tobytes() == oparams[p.name].tobytes(), p.name
+            assert s == oracle.safe_checksum(oparams[p.name]), p.name
+    assert gpu_engine.checksum32([torch.empty(0, dtype=torch.uint8, device="cuda")]) == ["00000000"]
