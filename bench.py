@@ -63,7 +63,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", type=int, default=2, choices=[1, 2, 3, 4, 5],
-                    help="BASELINE.json configuration (1-based); 2 = Llama-3-8B, the one the metric is quoted on")
+                    help="benchmark configuration (1-based); 2 = Llama-3-8B, the one the metric is quoted on")
     ap.add_argument("--rank", type=int, default=3, help="tensor-parallel (and expert-parallel) rank whose share is placed")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the configuration's own)")
     ap.add_argument("--max-file-gb", type=float, default=40.0,

@@ -963,6 +963,8 @@ int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndi
     }
     td.vec_src = vs;
     td.vec_dst = vd;
+    td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
+    for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
     uint32_t* sum_dev = nullptr;
     if (checksum) {
       acquire_arena(e);

@@ -33,6 +33,17 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
   return v;
 }
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld16_nt(const uint8_t* p) {
+  const u32x4 t = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(t.x, t.y, t.z, t.w);
+}
+__device__ __forceinline__ void st16_nt(uint8_t* p, const uint4& v) {
+  u32x4 t;
+  t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w;
+  __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
+}
+
 // Same checksum algebra as place_kernel (see mxp_kernels.hip).
 struct Csum {
   uint32_t P = 0, Q = 0, R = 0;
@@ -55,18 +66,22 @@ struct Csum {
   __device__ __forceinline__ uint32_t fold() const { return kKnuth * (P + R) + Q; }
 };
 
-template <int ES>
-__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
-                                                              uint8_t* __restrict__ dst,
-                                                              const TransposeDesc d,
-                                                              uint32_t* __restrict__ sum_out) {
-  constexpr int V = 16 / ES;                    // elements per 16-byte chunk
-  constexpr int TI = TileOf<ES>::I, TJ = TileOf<ES>::J;
-  constexpr int kPitch = TJ * ES + 4;           // LDS row pitch in bytes (dword aligned)
-  __shared__ __align__(16) uint8_t lds[TI * kPitch];
+struct TileCtx {
+  const uint8_t* sp;   // first source byte of the tile
+  uint8_t* dp;         // first destination byte of the tile
+  uint32_t ni, nj;     // valid extents inside the tile
+  uint32_t csum_base;  // checksum position of dp
+  bool valid;
+};
 
-  // blockIdx.x -> (batch, tile_j, tile_i), tile_i fastest.
-  uint64_t b = blockIdx.x;
+// Linear tile index -> (batch, tile_j, tile_i), tile_i fastest.  Workgroup-uniform.
+template <int ES>
+__device__ __forceinline__ TileCtx locate_tile(const TransposeDesc& d, uint64_t tile, const uint8_t* src, uint8_t* dst) {
+  constexpr int TI = TileOf<ES>::I, TJ = TileOf<ES>::J;
+  TileCtx c{};
+  c.valid = tile < d.n_tiles;
+  if (!c.valid) return c;
+  uint64_t b = tile;
   const uint32_t ti = (uint32_t)(b % d.tiles_i);
   b /= d.tiles_i;
   const uint32_t tj = (uint32_t)(b % d.tiles_j);
@@ -81,26 +96,38 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
     d_off += idx * d.batch_dstride[k];
   }
   const uint64_t i0 = (uint64_t)ti * TI, j0 = (uint64_t)tj * TJ;
-  const uint32_t ni = (uint32_t)min((uint64_t)TI, d.ni - i0);
-  const uint32_t nj = (uint32_t)min((uint64_t)TJ, d.nj - j0);
-  const uint8_t* sp = src + (s_off + i0 * d.si + j0) * ES;
-  uint8_t* dp = dst + (d_off + j0 * d.dj + i0) * ES;
+  c.ni = (uint32_t)min((uint64_t)TI, d.ni - i0);
+  c.nj = (uint32_t)min((uint64_t)TJ, d.nj - j0);
+  c.sp = src + (s_off + i0 * d.si + j0) * ES;
+  c.dp = dst + (d_off + j0 * d.dj + i0) * ES;
+  c.csum_base = (uint32_t)((d_off + j0 * d.dj + i0) * ES) + d.csum_bias;
+  return c;
+}
 
-  // ---- load: rows along j (contiguous in the source) ----
-  constexpr int kChunksJ = TJ / V;
-  constexpr int kLoads = TI * kChunksJ / kThreads;  // 8 for every element size
+template <int ES>
+struct TileIO {
+  static constexpr int V = 16 / ES;  // elements per 16-byte chunk
+  static constexpr int TI = TileOf<ES>::I, TJ = TileOf<ES>::J;
+  static constexpr int kPitch = TJ * ES + 4;  // LDS row pitch in bytes (dword aligned)
+  static constexpr int kChunksJ = TJ / V, kChunksI = TI / V;
+  static constexpr int kLoads = TI * kChunksJ / kThreads;  // 8 for every element size
   static_assert(kLoads * kThreads == TI * kChunksJ, "tile must divide evenly over the workgroup");
-  {
-    uint4 x[kLoads];
-    bool fast[kLoads];
-    // every 16-byte load of the tile is issued before the first LDS write
+
+  // global -> registers: rows along j (contiguous in the source), 16 bytes per lane access.
+  static __device__ __forceinline__ void issue_loads(const TileCtx& c, const TransposeDesc& d, uint4 (&x)[kLoads],
+                                                     bool (&fast)[kLoads]) {
 #pragma unroll
     for (int k = 0; k < kLoads; ++k) {
       const uint32_t q = threadIdx.x + (uint32_t)k * kThreads;
       const uint32_t ii = q / kChunksJ, cj = q % kChunksJ;
-      fast[k] = d.vec_src && ii < ni && cj * V + V <= nj;
-      if (fast[k]) x[k] = *reinterpret_cast<const uint4*>(sp + ((uint64_t)ii * d.si + cj * V) * ES);
+      fast[k] = d.vec_src && ii < c.ni && cj * V + V <= c.nj;
+      if (fast[k]) x[k] = ld16_nt(c.sp + ((uint64_t)ii * d.si + cj * V) * ES);
     }
+  }
+
+  // registers -> LDS (chunks that could not use a 16-byte load are copied element-wise here).
+  static __device__ __forceinline__ void to_lds(const TileCtx& c, const TransposeDesc& d, const uint4 (&x)[kLoads],
+                                                const bool (&fast)[kLoads], uint8_t* lds) {
 #pragma unroll
     for (int k = 0; k < kLoads; ++k) {
       const uint32_t q = threadIdx.x + (uint32_t)k * kThreads;
@@ -109,52 +136,80 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
       if (fast[k]) {
         uint32_t* lw = reinterpret_cast<uint32_t*>(l);
         lw[0] = x[k].x; lw[1] = x[k].y; lw[2] = x[k].z; lw[3] = x[k].w;
-      } else if (ii < ni && cj * V < nj) {
-        const uint8_t* g = sp + ((uint64_t)ii * d.si + cj * V) * ES;
-        const uint32_t n = min((uint32_t)V, nj - cj * V) * ES;
+      } else if (ii < c.ni && cj * V < c.nj) {
+        const uint8_t* g = c.sp + ((uint64_t)ii * d.si + cj * V) * ES;
+        const uint32_t n = min((uint32_t)V, c.nj - cj * V) * ES;
         for (uint32_t e = 0; e < n; ++e) l[e] = g[e];
       }
     }
   }
-  __syncthreads();
 
-  // ---- store: rows along i (contiguous in the destination) ----
-  Csum cs;
-  const uint32_t csum_base = (uint32_t)((d_off + j0 * d.dj + i0) * ES) + d.csum_bias;
-  constexpr int kChunksI = TI / V;
+  // LDS -> global: rows along i (contiguous in the destination), 16 bytes per lane access.
   // Work item q -> (column jj, row group ci): 16 neighbouring columns vary fastest, then 4
   // row groups, so one wavefront instruction reads 16 columns x 4 row groups from LDS.
-  for (uint32_t q = threadIdx.x; q < (uint32_t)(TJ * kChunksI); q += kThreads) {
-    const uint32_t jj = (q & 15u) + 16u * (q / (16u * kChunksI));
-    const uint32_t ci = (q >> 4) % kChunksI;
-    if (jj >= nj || ci * V >= ni) continue;
-    const uint32_t ii0 = ci * V;
-    const uint32_t n = min((uint32_t)V, ni - ii0);
-    union { uint4 v; uint8_t b[16]; } x;
-    x.v = make_uint4(0, 0, 0, 0);
+  static __device__ __forceinline__ void to_global(const TileCtx& c, const TransposeDesc& d, const uint8_t* lds, Csum& cs) {
+    for (uint32_t q = threadIdx.x; q < (uint32_t)(TJ * kChunksI); q += kThreads) {
+      const uint32_t jj = (q & 15u) + 16u * (q / (16u * kChunksI));
+      const uint32_t ci = (q >> 4) % kChunksI;
+      if (jj >= c.nj || ci * V >= c.ni) continue;
+      const uint32_t ii0 = ci * V;
+      const uint32_t n = min((uint32_t)V, c.ni - ii0);
+      union { uint4 v; uint8_t b[16]; } x;
+      x.v = make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int k = 0; k < V; ++k) {
-      if ((uint32_t)k < n) {
-        const uint8_t* l = lds + (ii0 + k) * kPitch + jj * ES;
-        if constexpr (ES == 1) x.b[k] = l[0];
-        else if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(&x.b[2 * k]) = *reinterpret_cast<const uint16_t*>(l);
-        else if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(&x.b[4 * k]) = *reinterpret_cast<const uint32_t*>(l);
-        else {
-          *reinterpret_cast<uint32_t*>(&x.b[8 * k]) = *reinterpret_cast<const uint32_t*>(l);
-          *reinterpret_cast<uint32_t*>(&x.b[8 * k + 4]) = *reinterpret_cast<const uint32_t*>(l + 4);
+      for (int k = 0; k < V; ++k) {
+        if ((uint32_t)k < n) {
+          const uint8_t* l = lds + (ii0 + k) * kPitch + jj * ES;
+          if constexpr (ES == 1) x.b[k] = l[0];
+          else if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(&x.b[2 * k]) = *reinterpret_cast<const uint16_t*>(l);
+          else if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(&x.b[4 * k]) = *reinterpret_cast<const uint32_t*>(l);
+          else {
+            *reinterpret_cast<uint32_t*>(&x.b[8 * k]) = *reinterpret_cast<const uint32_t*>(l);
+            *reinterpret_cast<uint32_t*>(&x.b[8 * k + 4]) = *reinterpret_cast<const uint32_t*>(l + 4);
+          }
+        }
+      }
+      const uint64_t off = ((uint64_t)jj * d.dj + ii0) * ES;  // bytes from dp
+      if (d.vec_dst && n == (uint32_t)V) {
+        st16_nt(c.dp + off, x.v);
+        cs.add16(x.v, c.csum_base + (uint32_t)off);
+      } else {
+        for (uint32_t k = 0; k < n * ES; ++k) {
+          c.dp[off + k] = x.b[k];
+          cs.add_byte(x.b[k], c.csum_base + (uint32_t)off + k);
         }
       }
     }
-    const uint64_t off = ((uint64_t)jj * d.dj + ii0) * ES;  // bytes from dp
-    if (d.vec_dst && n == (uint32_t)V) {
-      *reinterpret_cast<uint4*>(dp + off) = x.v;
-      cs.add16(x.v, csum_base + (uint32_t)off);
-    } else {
-      for (uint32_t k = 0; k < n * ES; ++k) {
-        dp[off + k] = x.b[k];
-        cs.add_byte(x.b[k], csum_base + (uint32_t)off + k);
-      }
-    }
+  }
+};
+
+// One workgroup walks kTilesPerGroup consecutive tiles (neighbours along i) and issues the
+// next tile's global loads before the current tile goes LDS -> global.  With more than one
+// tile per workgroup the wait before the next LDS fill also waits for the stores just
+// issued (loads and stores share one in-order counter on this target), so the overlap does
+// not materialise; one tile per workgroup, with two workgroups per CU alternating phases,
+// measured faster and is the setting used.
+template <int ES>
+__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
+                                                              uint8_t* __restrict__ dst,
+                                                              const TransposeDesc d,
+                                                              uint32_t* __restrict__ sum_out) {
+  using IO = TileIO<ES>;
+  __shared__ __align__(16) uint8_t lds[IO::TI * IO::kPitch];
+  uint4 x[IO::kLoads];
+  bool fast[IO::kLoads];
+  Csum cs;
+  const uint64_t first = (uint64_t)blockIdx.x * kTilesPerGroup;
+  TileCtx cur = locate_tile<ES>(d, first, src, dst);
+  if (cur.valid) IO::issue_loads(cur, d, x, fast);
+  for (int t = 0; t < kTilesPerGroup && cur.valid; ++t) {
+    IO::to_lds(cur, d, x, fast, lds);
+    __syncthreads();
+    const TileCtx next = (t + 1 < kTilesPerGroup) ? locate_tile<ES>(d, first + t + 1, src, dst) : TileCtx{};
+    if (next.valid) IO::issue_loads(next, d, x, fast);
+    IO::to_global(cur, d, lds, cs);
+    __syncthreads();
+    cur = next;
   }
 
   if (sum_out) {
@@ -175,9 +230,8 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
 
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
                             uint32_t* sum_out, hipStream_t stream) {
-  uint64_t blocks = (uint64_t)d.tiles_i * d.tiles_j;
-  for (int k = 0; k < kMaxBatchDims; ++k) blocks *= d.batch_size[k];
-  if (blocks == 0) return hipSuccess;
+  if (d.n_tiles == 0) return hipSuccess;
+  const uint64_t blocks = (d.n_tiles + kTilesPerGroup - 1) / kTilesPerGroup;
   if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
   const dim3 grid((uint32_t)blocks), block(kThreads);
   const uint8_t* s = static_cast<const uint8_t*>(src);

@@ -1,4 +1,4 @@
-"""Full-size checks (BASELINE configuration 2: Llama-3-8B, one TP=8 rank slice, 16 GB
+"""Full-size checks (benchmark configuration 2: Llama-3-8B, one TP=8 rank slice, 16 GB
 staged in HBM) through properties that do not need the oracle to process 16 GB:
 
 * the checkpoint is generated on the device by the seeded generator, which produces the
