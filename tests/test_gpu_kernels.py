@@ -217,3 +217,50 @@ def test_mla_absorbed_weights_on_device(gpu_engine, oracle, oracle_c):
     assert uv.cpu().numpy().tobytes() == want_uv.tobytes()
     assert ukt.cpu().numpy().tobytes() == want_ukt.tobytes()
     assert c_uv == oracle.safe_checksum(want_uv) and c_ukt == oracle.safe_checksum(want_ukt)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
+    """Random batches of pitched boxes with every alignment class (16 / 8 / 4 / 2 / 1 byte
+    units), copies and casts mixed, rows from 1 to thousands, wide rows split by columns."""
+    rng = np.random.default_rng(500 + seed)
+    src = rng.integers(0, 256, 6 << 20, dtype=np.uint8)
+    f32 = src.view(np.uint32)
+    d_src = _dev(src)
+    out_size = 8 << 20
+    want = np.full(out_size, 0xEE, dtype=np.uint8)
+    boxes, sums_want, cursor = [], [], 0
+    for g in range(int(rng.integers(1, 9))):
+        cast = bool(rng.integers(0, 3) == 0)
+        align = int(rng.choice([1, 2, 4, 8, 16])) if not cast else int(rng.choice([2, 4, 8, 16]))
+        rows = int(rng.choice([1, 1, 2, 7, 64, 513, 3000]))
+        row_bytes = int(rng.integers(1, 40)) * align if rng.integers(0, 4) else int(rng.integers(1, 5)) * 20000 // align * align
+        row_bytes = max(align, row_bytes - row_bytes % (2 if cast else 1))
+        sm = 2 if cast else 1
+        dst_pitch = row_bytes + int(rng.integers(0, 4)) * align
+        src_pitch = row_bytes * sm + int(rng.integers(0, 5)) * align * (2 if cast else 1)
+        if rows * max(dst_pitch, 1) > (1 << 20) or rows * src_pitch > (4 << 20):
+            rows = max(1, min((1 << 20) // dst_pitch, (4 << 20) // src_pitch))
+        src_off = int(rng.integers(0, 64)) * (4 if cast else 1)
+        src_off -= src_off % (4 if cast else min(align, 16))
+        dst_off = (cursor + 15) // 16 * 16
+        if rows == 1 and not cast and align < 16 and rng.integers(0, 2):
+            dst_off += align  # a byte/dword-granular start inside the buffer
+        csum = 0
+        for r in range(rows):
+            s = src[src_off + r * src_pitch: src_off + r * src_pitch + row_bytes * sm]
+            if cast:
+                s = oracle.cast_f32_bf16_bits(s.view(np.uint32)).view(np.uint8)
+            want[dst_off + r * dst_pitch: dst_off + r * dst_pitch + row_bytes] = s
+            csum += int(oracle_c.checksum32(s, first_index=1000 + r * dst_pitch), 16)
+        sums_want.append(format(csum & 0xFFFFFFFF, "08x"))
+        boxes.append({"src": d_src.data_ptr() + src_off, "dst": dst_off, "src_pitch": src_pitch, "dst_pitch": dst_pitch,
+                      "rows": rows, "row_bytes": row_bytes, "csum_index": 1000, "csum_group": g, "cast": int(cast)})
+        cursor = dst_off + rows * dst_pitch + 64
+        assert cursor < out_size
+    out = torch.full((out_size,), 0xEE, dtype=torch.uint8, device="cuda")
+    for b in boxes:
+        b["dst"] = out.data_ptr() + b["dst"]
+    sums = gpu_engine.place_boxes(boxes, len(boxes))
+    assert np.array_equal(out.cpu().numpy(), want)
+    assert sums == sums_want
