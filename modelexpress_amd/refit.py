@@ -29,6 +29,7 @@ import torch
 
 from .adapter import PlacementLayout
 from .engine import Checkpoint, PlacementEngine, PlacementPlan
+from .timing import RefitTimingRecorder
 
 
 @dataclass(frozen=True)
@@ -65,6 +66,13 @@ class StagedWeights:
     in_place: bool
 
 
+import contextlib
+
+
+def _null():
+    return contextlib.nullcontext()
+
+
 class HipRefitAdapter:
     """Refit executor for one rank's resident parameters."""
 
@@ -72,6 +80,8 @@ class HipRefitAdapter:
 
     def __init__(self, layout: PlacementLayout, *, device: int = 0, engine: PlacementEngine | None = None,
                  in_place: bool = False):
+        self.timing: RefitTimingRecorder | None = None  # the record of the cycle in progress
+        self._plans_built = 0
         self.layout = layout
         self.device = device
         self.in_place = in_place
@@ -79,11 +89,15 @@ class HipRefitAdapter:
         self.engine = engine or PlacementEngine(device)
 
     def create_transfer_plan(self, inputs: RefitInputs) -> RefitPlan:
-        ck = Checkpoint(inputs.checkpoint_path)
         lay = self.layout
-        plan = PlacementPlan(ck, lay.params, tp_size=lay.tp_size, tp_rank=lay.tp_rank,
-                             stacked_params_mapping=lay.stacked_params_mapping, expert_mapping=lay.expert_mapping,
-                             skip_prefixes=lay.skip_prefixes, allow_cast=True)
+        self.timing = RefitTimingRecorder(backend="hip_placement", version=inputs.version_id, tp_rank=lay.tp_rank,
+                                          tp_size=lay.tp_size, cold=self._plans_built == 0)
+        with self.timing.span("transfer_planning"):
+            ck = Checkpoint(inputs.checkpoint_path)
+            plan = PlacementPlan(ck, lay.params, tp_size=lay.tp_size, tp_rank=lay.tp_rank,
+                                 stacked_params_mapping=lay.stacked_params_mapping, expert_mapping=lay.expert_mapping,
+                                 skip_prefixes=lay.skip_prefixes, allow_cast=True)
+        self._plans_built += 1
         return RefitPlan(inputs, ck, plan, inputs.physical_fingerprint)
 
     def validate_transfer_plan(self, plan: Any, inputs: RefitInputs) -> bool:
@@ -91,13 +105,19 @@ class HipRefitAdapter:
 
     def stage_weight(self, plan: RefitPlan) -> StagedWeights:
         eng = self.engine
-        buffers = list(self.layout.destinations) if self.in_place else eng.allocate(plan.plan)
-        stats = eng.execute(plan.plan, buffers)
-        sums = eng.checksums(plan.plan)
-        sizes = [p.nbytes for p in plan.plan.params]
-        digests = eng.digest(buffers, sizes)
-        staged = StagedWeights(plan, buffers, sums, digests, stats, self.in_place)
-        self._verify(staged)
+        rec = self.timing or RefitTimingRecorder(backend="hip_placement", version=plan.inputs.version_id, cold=False)
+        self.timing = rec
+        with rec.span("setup_registration"):
+            buffers = list(self.layout.destinations) if self.in_place else eng.allocate(plan.plan)
+        with rec.span("wire_transfer"):
+            stats = eng.execute(plan.plan, buffers)
+            sums = eng.checksums(plan.plan)
+        rec.bytes = stats["placed_bytes"]
+        with rec.span("receive_sync"):
+            sizes = [p.nbytes for p in plan.plan.params]
+            digests = eng.digest(buffers, sizes)
+            staged = StagedWeights(plan, buffers, sums, digests, stats, self.in_place)
+            self._verify(staged)
         return staged
 
     def _verify(self, staged: StagedWeights) -> None:
@@ -115,14 +135,20 @@ class HipRefitAdapter:
 
     def apply_weight(self, staged: StagedWeights) -> dict:
         names = [p.name for p in staged.plan.plan.params]
-        if staged.in_place:
-            return dict(zip(names, staged.checksums))
-        sizes = [p.nbytes for p in staged.plan.plan.params]
-        sums = self.engine.copy_batch(staged.buffers, list(self.layout.destinations), sizes)
-        torch.cuda.synchronize(self.device)
-        if sums != staged.checksums:
-            raise RuntimeError(f"refit {staged.plan.inputs.version_id}: installed bytes differ from the staged ones")
-        return dict(zip(names, sums))
+        rec = self.timing
+        try:
+            if staged.in_place:
+                return dict(zip(names, staged.checksums))
+            sizes = [p.nbytes for p in staged.plan.plan.params]
+            with (rec.span("installation") if rec else _null()):
+                sums = self.engine.copy_batch(staged.buffers, list(self.layout.destinations), sizes)
+                torch.cuda.synchronize(self.device)
+            if sums != staged.checksums:
+                raise RuntimeError(f"refit {staged.plan.inputs.version_id}: installed bytes differ from the staged ones")
+            return dict(zip(names, sums))
+        finally:
+            if rec is not None:
+                rec.emit()
 
     def release_staged_weight(self, staged: StagedWeights) -> None:
         if not staged.in_place:

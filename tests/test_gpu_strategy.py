@@ -193,5 +193,9 @@ def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
     for n, p in model.named_parameters():
         assert p.data.view(torch.uint8).cpu().numpy().tobytes() == want[n].tobytes(), n
         assert sums[n] == oracle.safe_checksum(want[n])
+    rec = ad.timing.as_dict()
+    assert rec["backend"] == "hip_placement" and rec["version"] == "v1" and rec["bytes"] == sum(p.nbytes for p in rv.params)
+    assert {"transfer_planning", "wire_transfer", "receive_sync", "installation"} <= set(rec["stages"])
+    assert ad.timing.emit().startswith("MX_REFIT_TIMING {")
     ad.release_staged_weight(staged)
     ad.close()

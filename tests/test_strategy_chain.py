@@ -182,3 +182,28 @@ def test_accelerator_backend_selection():
     assert b.torch_device(1) == torch.device("cuda", 1)
     with pytest.raises(ValueError, match="Unsupported accelerator backend"):
         accelerator_backend_for("xpu:0")
+
+
+def test_refit_timing_vocabulary():
+    # modelexpress/refit/timing.py:23-35: ten fixed stages, one JSON record with a fixed prefix
+    import json
+
+    from modelexpress_amd.timing import MX_REFIT_TIMING_PREFIX, REFIT_TIMING_STAGES, RefitTimingRecorder
+
+    assert REFIT_TIMING_STAGES == ("control_discovery", "source_preparation", "setup_registration", "transfer_planning",
+                                   "wire_transfer", "receive_sync", "transformation", "installation", "post_install",
+                                   "rollout_readiness")
+    ticks = iter([0.0, 1.0, 3.0, 3.0, 3.5, 10.0, 10.0])
+    rec = RefitTimingRecorder(backend="test", version=7, cold=True, clock=lambda: next(ticks))
+    with rec.span("wire_transfer"):
+        pass
+    with pytest.raises(RuntimeError):
+        with rec.span("installation"):
+            raise RuntimeError("boom")
+    with pytest.raises(ValueError):
+        rec.add_duration("not_a_stage", 1.0)
+    line = rec.emit()
+    assert line.startswith(MX_REFIT_TIMING_PREFIX + " ")
+    payload = json.loads(line[len(MX_REFIT_TIMING_PREFIX) + 1:])
+    assert payload["cold_warm"] == "cold" and payload["stages"]["wire_transfer"] == {"duration_s": 2.0, "count": 1, "statuses": ["ok"]}
+    assert payload["stages"]["installation"]["statuses"] == ["error"]
