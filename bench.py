@@ -217,8 +217,9 @@ def main() -> int:
                                 "gbps_wall": round(placed / dt / 1e9, 1),
                                 "note": "one batched launch; wall time includes descriptor upload, result copy and sync"}
             ops["checksum32"]["matches_fused"] = eng.checksum32(dst, sizes) == resident_sums
-            # LDS-tiled transpose (permuted copies): a square bf16 matrix and the MLA W_UK_T shape
+            # LDS transpose (permuted copies): a square bf16 matrix, a batch of smaller ones and the MLA W_UK_T shape
             for label, shape, perm in (("transpose_bf16_16384x16384", (16384, 16384), (1, 0)),
+                                       ("transpose_bf16_16x4096x4096", (16, 4096, 4096), (0, 2, 1)),
                                        ("mla_w_uk_t_bf16_128x128x512", (128, 128, 512), (1, 2, 0))):
                 nbytes = 2
                 for v in shape:

@@ -74,7 +74,12 @@ hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_
 // Batched 2-D transpose (mxp_permute.hip).  "i" = the destination's innermost dimension,
 // "j" = the source's innermost dimension; strides are in elements.
 constexpr int kMaxBatchDims = 6;
-constexpr int kTilesPerGroup = 1;  // consecutive tiles one transpose workgroup walks (4 measured 12% slower)
+// Transpose tiling.  One wavefront owns a sub-tile of 64 (128 for 1-byte elements) source rows
+// (i) x 128 source bytes (j); a workgroup is kTransposeWaves wavefronts arranged
+// waves_i x (kTransposeWaves / waves_i), chosen per call from the extents.
+constexpr int kTransposeWaves = 8;
+constexpr int transpose_sub_rows(int elem_size) { return elem_size == 1 ? 128 : 64; }
+constexpr int transpose_sub_cols(int elem_size) { return 128 / elem_size; }
 struct TransposeDesc {
   uint64_t ni, nj;   // extents
   uint64_t si;       // source stride of i (source stride of j is 1)
@@ -85,7 +90,8 @@ struct TransposeDesc {
   uint64_t batch_sstride[kMaxBatchDims];
   uint64_t batch_dstride[kMaxBatchDims];
   uint32_t vec_src, vec_dst;  // 16-byte accesses are aligned on that side
-  uint32_t csum_bias, pad;
+  uint32_t csum_bias;
+  uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides kTransposeWaves)
 };
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
                             uint32_t* sum_out, hipStream_t stream);

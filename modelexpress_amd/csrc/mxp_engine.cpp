@@ -945,7 +945,13 @@ int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndi
     td.si = ss[nd - 1];
     td.nj = size[c];
     td.dj = ds[c];
-    const uint64_t tile_i = 512, tile_j = es == 1 ? 128 : es == 2 ? 64 : es == 4 ? 32 : 16;  // TileOf<ES>
+    // Workgroup shape: as many wavefronts along i (long destination runs) as the extent can
+    // use, the rest along j.
+    uint32_t waves_i = 1;
+    while (waves_i < (uint32_t)kTransposeWaves && (uint64_t)waves_i * transpose_sub_rows(elem_size) < td.ni) waves_i *= 2;
+    td.waves_i = waves_i;
+    const uint64_t tile_i = (uint64_t)waves_i * transpose_sub_rows(elem_size);
+    const uint64_t tile_j = (uint64_t)(kTransposeWaves / waves_i) * transpose_sub_cols(elem_size);
     td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
     td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
     bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * es) % 16 == 0;

@@ -1,5 +1,5 @@
-// Batched LDS-tiled transpose: dst = src.permute(...).contiguous() when the permutation
-// moves the source's contiguous dimension away from the innermost position.
+// Batched LDS transpose: dst = src.permute(...).contiguous() when the permutation moves the
+// source's contiguous dimension away from the innermost position.
 //
 // Reference call sites: the MLA absorbed weights  W_UK_T = w_uk.permute(1, 2, 0)
 // (modelexpress/engines/vllm/refit/receiver.py:252-261) and permuted box views
@@ -9,23 +9,36 @@
 //
 // Naming: "i" is the destination's innermost dimension (strided in the source), "j" the
 // source's innermost dimension (strided in the destination); every other dimension is a
-// batch index.  A workgroup moves one tile of 512 (i) x 128 bytes (j): source rows are read
-// with 16-byte loads (eight per lane, all issued before the first LDS write) into LDS, and
-// columns are read back out of LDS so that every store is 16 contiguous destination bytes.
-// The transposition happens in LDS; the row pitch is a whole row plus one dword, and in the
-// store phase one wavefront covers 16 neighbouring columns x 4 row groups so that its 64
-// column reads spread over the banks.  HBM traffic: every element read once, written once.
+// batch index.
+//
+// Every wavefront moves its own sub-tile and never waits for another one (no workgroup
+// barrier on the data path): 64 or 128 source rows (i) x 128 source bytes (j).
+//   1. global -> registers: lane = (row mod 8, 16-byte chunk); 8 (16 for 1-byte elements)
+//      128-bit loads per lane, all issued before anything else; a wavefront load covers eight
+//      whole 128-byte lines.
+//   2. registers -> LDS, row major, with the chunk index XOR-swizzled by the row group, one
+//      ds_write_b128 per load, conflict free.
+//   3. LDS -> registers: a lane owns a dword column (two bf16 / four fp8 columns) and reads it
+//      down the V = 16 / elem_size rows that make one 16-byte destination chunk; the swizzle
+//      makes the 32 lanes of an LDS cycle hit 32 different banks.  Bytes are regrouped with
+//      v_perm_b32.
+//   4. registers -> global: eight consecutive lanes write one whole 128-byte destination
+//      line, so a wavefront store is eight full lines.  The checksum is taken from the
+//      registers being stored.
+// HBM traffic: every element read once and written once, in whole lines.
+//
+// A workgroup is eight such wavefronts, waves_i of them side by side along i (so the
+// workgroup writes runs of up to 1 KiB per destination row) and the rest along j; the host
+// picks waves_i from the extent of i.  The workgroup only exists to share an LDS allocation
+// and one checksum atomic.  Measured on 2-byte elements: 16384 x 16384 5.4 TB/s, sixteen
+// 4096 x 4096 matrices 6.2 TB/s (a plain copy of the same bytes through place_kernel: 5.7);
+// the rate falls as the destination pitch grows (65536 x 4096: 4.6-5.0 TB/s).  Visiting
+// tiles in compact super-tiles or in bands along j measured no better than plain order.
 #include "mxp_device.h"
 
 namespace mxp {
 
 namespace {
-
-constexpr int kThreads = 512;
-// Tile extents per element size: 66 KiB of LDS (two workgroups per CU), eight 16-byte loads
-// per lane in flight.  Long destination runs matter most: 512 x 64 bf16 elements (1 KiB
-// written per destination row) measured 4.56 TB/s on a 16384^2 transpose, 128 x 128 4.0 TB/s.
-template <int ES> struct TileOf { static constexpr int I = 512, J = (ES == 1) ? 128 : (ES == 2) ? 64 : (ES == 4) ? 32 : 16; };
 
 __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
 #pragma unroll
@@ -66,22 +79,169 @@ struct Csum {
   __device__ __forceinline__ uint32_t fold() const { return kKnuth * (P + R) + Q; }
 };
 
-struct TileCtx {
-  const uint8_t* sp;   // first source byte of the tile
-  uint8_t* dp;         // first destination byte of the tile
-  uint32_t ni, nj;     // valid extents inside the tile
-  uint32_t csum_base;  // checksum position of dp
-  bool valid;
+constexpr int kWaves = kTransposeWaves;
+constexpr int kThreads = kWaves * 64;
+
+template <int ES>
+struct Sub {
+  static constexpr int kLoads = transpose_sub_rows(ES) / 8;  // 16-byte loads per lane
+  static constexpr int RI = transpose_sub_rows(ES);          // rows (i) of a wavefront's sub-tile
+  static constexpr int TJ = 128 / ES;                        // columns (j): 128 source bytes per row
+  static constexpr int V = 16 / ES;                          // rows gathered into one 16-byte destination chunk
+  static constexpr int G = ES == 8 ? 8 : 4;                  // bytes per LDS read
+  static constexpr int DPC = 16 / G;                         // LDS reads across one 16-byte source chunk
+  static constexpr int CPR = G / ES;                         // destination rows fed by one LDS column
+  static constexpr int NW = V * G / 4;                       // dwords a lane gathers per iteration
+  static constexpr int NCI = RI / V;                         // 16-byte chunks per destination row
+  static constexpr int RESTN = 64 / (8 * DPC);               // (chunk column, row group) pairs per iteration
+  static constexpr int kIters = NCI / RESTN;
+  static constexpr int kLdsBytes = RI * 128;
+  static_assert(NCI % 8 == 0 && kIters * RESTN == NCI, "sub-tile does not divide over the wavefront");
+  static_assert(kWaves * kLdsBytes <= 160 * 1024, "workgroup exceeds the LDS of a compute unit");
 };
 
-// Linear tile index -> (batch, tile_j, tile_i), tile_i fastest.  Workgroup-uniform.
+// Byte e of a 16-byte register value, without indexing memory (a dynamically indexed local
+// array would be placed in LDS and cost occupancy).
+__device__ __forceinline__ uint32_t get_byte(const uint4& v, uint32_t e) {
+  const uint64_t lo = (uint64_t)v.x | ((uint64_t)v.y << 32), hi = (uint64_t)v.z | ((uint64_t)v.w << 32);
+  return (uint32_t)(((e < 8u) ? lo : hi) >> ((e & 7u) * 8u)) & 0xFFu;
+}
+__device__ __forceinline__ void or_byte(uint4& v, uint32_t e, uint32_t byte) {
+  const uint32_t s = byte << ((e & 3u) * 8u);
+  v.x |= (e < 4u) ? s : 0u;
+  v.y |= (e >= 4u && e < 8u) ? s : 0u;
+  v.z |= (e >= 8u && e < 12u) ? s : 0u;
+  v.w |= (e >= 12u) ? s : 0u;
+}
+
+// Destination chunk p (0 <= p < CPR) out of the NW gathered dwords: element p of every row.
+template <int ES, int P>
+__device__ __forceinline__ uint4 regroup(const uint32_t (&w)[Sub<ES>::NW]) {
+  if constexpr (ES >= 4) {
+    return make_uint4(w[0], w[1], w[2], w[3]);
+  } else if constexpr (ES == 2) {
+    constexpr uint32_t sel = P == 0 ? 0x05040100u : 0x07060302u;
+    return make_uint4(__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel),
+                      __builtin_amdgcn_perm(w[5], w[4], sel), __builtin_amdgcn_perm(w[7], w[6], sel));
+  } else {
+    constexpr uint32_t sel = (uint32_t)P | ((uint32_t)(4 + P) << 8) | 0x0c0c0000u;  // byte P of both operands, low half
+    uint32_t o[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t a = __builtin_amdgcn_perm(w[4 * d + 1], w[4 * d], sel);
+      const uint32_t b = __builtin_amdgcn_perm(w[4 * d + 3], w[4 * d + 2], sel);
+      o[d] = a | (b << 16);
+    }
+    return make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
+template <int ES, bool FULL>
+__device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_t ci, uint8_t* __restrict__ dp, uint32_t ni,
+                                            uint32_t nj, uint64_t dj_bytes, uint32_t csum_base, bool vec_dst, Csum& cs) {
+  using S = Sub<ES>;
+  const uint64_t off = (uint64_t)jj * dj_bytes + ci * 16u;
+  const uint32_t pos = csum_base + (uint32_t)off;
+  if constexpr (FULL) {
+    st16_nt(dp + off, v);
+    cs.add16(v, pos);
+  } else {
+    if (jj < nj && ci * S::V < ni) {
+      const uint32_t n = min((uint32_t)S::V, ni - ci * S::V);
+      if (vec_dst && n == (uint32_t)S::V) {
+        st16_nt(dp + off, v);
+        cs.add16(v, pos);
+      } else {
+        for (uint32_t e = 0; e < n * ES; ++e) {
+          const uint32_t byte = get_byte(v, e);
+          dp[off + e] = (uint8_t)byte;
+          cs.add_byte(byte, pos + e);
+        }
+      }
+    }
+  }
+}
+
+// Moves one sub-tile.  FULL: the sub-tile is complete and both sides allow 16-byte accesses,
+// so nothing is predicated.  Otherwise rows / columns beyond (ni, nj) are skipped and chunks
+// that cannot use a 16-byte access are moved byte-wise.
+template <int ES, bool FULL>
+__device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uint8_t* __restrict__ dp, uint32_t ni,
+                                             uint32_t nj, uint64_t si_bytes, uint64_t dj_bytes, uint32_t csum_base,
+                                             bool vec_src, bool vec_dst, uint8_t* lds, Csum& cs) {
+  using S = Sub<ES>;
+  const uint32_t lane = threadIdx.x & 63u;
+  {
+    const uint32_t lrow = lane >> 3, c = lane & 7u;
+    uint4 x[S::kLoads];
+#pragma unroll
+    for (int k = 0; k < S::kLoads; ++k) {
+      const uint32_t row = (uint32_t)k * 8u + lrow;
+      const uint8_t* g = sp + (uint64_t)row * si_bytes + c * 16u;
+      if constexpr (FULL) {
+        x[k] = ld16_nt(g);
+      } else {
+        x[k] = make_uint4(0, 0, 0, 0);
+        if (row < ni && c * S::V < nj) {
+          if (vec_src && c * S::V + S::V <= nj) {
+            x[k] = ld16_nt(g);
+          } else {
+            const uint32_t n = min((uint32_t)S::V, nj - c * S::V) * ES;
+            for (uint32_t e = 0; e < n; ++e) or_byte(x[k], e, g[e]);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < S::kLoads; ++k) {
+      const uint32_t row = (uint32_t)k * 8u + lrow;
+      const uint32_t f = (row / S::V) & 7u;
+      *reinterpret_cast<uint4*>(lds + row * 128u + ((c ^ f) << 4)) = x[k];
+    }
+  }
+  // Only this wavefront touches its LDS region and its LDS operations complete in issue
+  // order: no barrier, the fence just stops the compiler from moving reads above the writes.
+  __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+
+  const uint32_t ci_lo = lane & 7u, dlo = (lane >> 3) % S::DPC, rest = lane / (8u * S::DPC);
+#pragma unroll
+  for (int it = 0; it < S::kIters; ++it) {
+    const uint32_t m = (uint32_t)it * S::RESTN + rest;
+    const uint32_t a = m & 7u, ci = (m >> 3) * 8u + ci_lo;
+    const uint8_t* l = lds + (ci * S::V) * 128u + ((a ^ ci_lo) << 4) + dlo * S::G;
+    uint32_t w[S::NW];
+#pragma unroll
+    for (int k = 0; k < S::V; ++k) {
+      if constexpr (S::G == 8) {
+        const uint2 t = *reinterpret_cast<const uint2*>(l + k * 128);
+        w[2 * k] = t.x;
+        w[2 * k + 1] = t.y;
+      } else {
+        w[k] = *reinterpret_cast<const uint32_t*>(l + k * 128);
+      }
+    }
+    const uint32_t jj0 = a * (16u / ES) + dlo * S::CPR;
+    store_chunk<ES, FULL>(regroup<ES, 0>(w), jj0, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+    if constexpr (S::CPR >= 2) store_chunk<ES, FULL>(regroup<ES, 1>(w), jj0 + 1, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+    if constexpr (S::CPR == 4) {
+      store_chunk<ES, FULL>(regroup<ES, 2>(w), jj0 + 2, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+      store_chunk<ES, FULL>(regroup<ES, 3>(w), jj0 + 3, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+    }
+  }
+}
+
 template <int ES>
-__device__ __forceinline__ TileCtx locate_tile(const TransposeDesc& d, uint64_t tile, const uint8_t* src, uint8_t* dst) {
-  constexpr int TI = TileOf<ES>::I, TJ = TileOf<ES>::J;
-  TileCtx c{};
-  c.valid = tile < d.n_tiles;
-  if (!c.valid) return c;
-  uint64_t b = tile;
+__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
+                                                              uint8_t* __restrict__ dst,
+                                                              const TransposeDesc d,
+                                                              uint32_t* __restrict__ sum_out) {
+  using S = Sub<ES>;
+  __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  Csum cs;
+  // Linear tile index -> (batch, tile_j, tile_i), tile_i fastest.  Workgroup-uniform.
+  uint64_t b = blockIdx.x;
   const uint32_t ti = (uint32_t)(b % d.tiles_i);
   b /= d.tiles_i;
   const uint32_t tj = (uint32_t)(b % d.tiles_j);
@@ -95,132 +255,32 @@ __device__ __forceinline__ TileCtx locate_tile(const TransposeDesc& d, uint64_t 
     s_off += idx * d.batch_sstride[k];
     d_off += idx * d.batch_dstride[k];
   }
-  const uint64_t i0 = (uint64_t)ti * TI, j0 = (uint64_t)tj * TJ;
-  c.ni = (uint32_t)min((uint64_t)TI, d.ni - i0);
-  c.nj = (uint32_t)min((uint64_t)TJ, d.nj - j0);
-  c.sp = src + (s_off + i0 * d.si + j0) * ES;
-  c.dp = dst + (d_off + j0 * d.dj + i0) * ES;
-  c.csum_base = (uint32_t)((d_off + j0 * d.dj + i0) * ES) + d.csum_bias;
-  return c;
-}
-
-template <int ES>
-struct TileIO {
-  static constexpr int V = 16 / ES;  // elements per 16-byte chunk
-  static constexpr int TI = TileOf<ES>::I, TJ = TileOf<ES>::J;
-  static constexpr int kPitch = TJ * ES + 4;  // LDS row pitch in bytes (dword aligned)
-  static constexpr int kChunksJ = TJ / V, kChunksI = TI / V;
-  static constexpr int kLoads = TI * kChunksJ / kThreads;  // 8 for every element size
-  static_assert(kLoads * kThreads == TI * kChunksJ, "tile must divide evenly over the workgroup");
-
-  // global -> registers: rows along j (contiguous in the source), 16 bytes per lane access.
-  static __device__ __forceinline__ void issue_loads(const TileCtx& c, const TransposeDesc& d, uint4 (&x)[kLoads],
-                                                     bool (&fast)[kLoads]) {
-#pragma unroll
-    for (int k = 0; k < kLoads; ++k) {
-      const uint32_t q = threadIdx.x + (uint32_t)k * kThreads;
-      const uint32_t ii = q / kChunksJ, cj = q % kChunksJ;
-      fast[k] = d.vec_src && ii < c.ni && cj * V + V <= c.nj;
-      if (fast[k]) x[k] = ld16_nt(c.sp + ((uint64_t)ii * d.si + cj * V) * ES);
-    }
-  }
-
-  // registers -> LDS (chunks that could not use a 16-byte load are copied element-wise here).
-  static __device__ __forceinline__ void to_lds(const TileCtx& c, const TransposeDesc& d, const uint4 (&x)[kLoads],
-                                                const bool (&fast)[kLoads], uint8_t* lds) {
-#pragma unroll
-    for (int k = 0; k < kLoads; ++k) {
-      const uint32_t q = threadIdx.x + (uint32_t)k * kThreads;
-      const uint32_t ii = q / kChunksJ, cj = q % kChunksJ;
-      uint8_t* l = lds + ii * kPitch + cj * 16;
-      if (fast[k]) {
-        uint32_t* lw = reinterpret_cast<uint32_t*>(l);
-        lw[0] = x[k].x; lw[1] = x[k].y; lw[2] = x[k].z; lw[3] = x[k].w;
-      } else if (ii < c.ni && cj * V < c.nj) {
-        const uint8_t* g = c.sp + ((uint64_t)ii * d.si + cj * V) * ES;
-        const uint32_t n = min((uint32_t)V, c.nj - cj * V) * ES;
-        for (uint32_t e = 0; e < n; ++e) l[e] = g[e];
-      }
-    }
-  }
-
-  // LDS -> global: rows along i (contiguous in the destination), 16 bytes per lane access.
-  // Work item q -> (column jj, row group ci): 16 neighbouring columns vary fastest, then 4
-  // row groups, so one wavefront instruction reads 16 columns x 4 row groups from LDS.
-  static __device__ __forceinline__ void to_global(const TileCtx& c, const TransposeDesc& d, const uint8_t* lds, Csum& cs) {
-    for (uint32_t q = threadIdx.x; q < (uint32_t)(TJ * kChunksI); q += kThreads) {
-      const uint32_t jj = (q & 15u) + 16u * (q / (16u * kChunksI));
-      const uint32_t ci = (q >> 4) % kChunksI;
-      if (jj >= c.nj || ci * V >= c.ni) continue;
-      const uint32_t ii0 = ci * V;
-      const uint32_t n = min((uint32_t)V, c.ni - ii0);
-      union { uint4 v; uint8_t b[16]; } x;
-      x.v = make_uint4(0, 0, 0, 0);
-#pragma unroll
-      for (int k = 0; k < V; ++k) {
-        if ((uint32_t)k < n) {
-          const uint8_t* l = lds + (ii0 + k) * kPitch + jj * ES;
-          if constexpr (ES == 1) x.b[k] = l[0];
-          else if constexpr (ES == 2) *reinterpret_cast<uint16_t*>(&x.b[2 * k]) = *reinterpret_cast<const uint16_t*>(l);
-          else if constexpr (ES == 4) *reinterpret_cast<uint32_t*>(&x.b[4 * k]) = *reinterpret_cast<const uint32_t*>(l);
-          else {
-            *reinterpret_cast<uint32_t*>(&x.b[8 * k]) = *reinterpret_cast<const uint32_t*>(l);
-            *reinterpret_cast<uint32_t*>(&x.b[8 * k + 4]) = *reinterpret_cast<const uint32_t*>(l + 4);
-          }
-        }
-      }
-      const uint64_t off = ((uint64_t)jj * d.dj + ii0) * ES;  // bytes from dp
-      if (d.vec_dst && n == (uint32_t)V) {
-        st16_nt(c.dp + off, x.v);
-        cs.add16(x.v, c.csum_base + (uint32_t)off);
-      } else {
-        for (uint32_t k = 0; k < n * ES; ++k) {
-          c.dp[off + k] = x.b[k];
-          cs.add_byte(x.b[k], c.csum_base + (uint32_t)off + k);
-        }
-      }
-    }
-  }
-};
-
-// One workgroup walks kTilesPerGroup consecutive tiles (neighbours along i) and issues the
-// next tile's global loads before the current tile goes LDS -> global.  With more than one
-// tile per workgroup the wait before the next LDS fill also waits for the stores just
-// issued (loads and stores share one in-order counter on this target), so the overlap does
-// not materialise; one tile per workgroup, with two workgroups per CU alternating phases,
-// measured faster and is the setting used.
-template <int ES>
-__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
-                                                              uint8_t* __restrict__ dst,
-                                                              const TransposeDesc d,
-                                                              uint32_t* __restrict__ sum_out) {
-  using IO = TileIO<ES>;
-  __shared__ __align__(16) uint8_t lds[IO::TI * IO::kPitch];
-  uint4 x[IO::kLoads];
-  bool fast[IO::kLoads];
-  Csum cs;
-  const uint64_t first = (uint64_t)blockIdx.x * kTilesPerGroup;
-  TileCtx cur = locate_tile<ES>(d, first, src, dst);
-  if (cur.valid) IO::issue_loads(cur, d, x, fast);
-  for (int t = 0; t < kTilesPerGroup && cur.valid; ++t) {
-    IO::to_lds(cur, d, x, fast, lds);
-    __syncthreads();
-    const TileCtx next = (t + 1 < kTilesPerGroup) ? locate_tile<ES>(d, first + t + 1, src, dst) : TileCtx{};
-    if (next.valid) IO::issue_loads(next, d, x, fast);
-    IO::to_global(cur, d, lds, cs);
-    __syncthreads();
-    cur = next;
+  const uint32_t waves_j = (uint32_t)kWaves / d.waves_i;
+  const uint64_t i0 = ((uint64_t)ti * d.waves_i + wave % d.waves_i) * S::RI;
+  const uint64_t j0 = ((uint64_t)tj * waves_j + wave / d.waves_i) * S::TJ;
+  if (i0 < d.ni && j0 < d.nj) {
+    const uint32_t ni = (uint32_t)min((uint64_t)S::RI, d.ni - i0), nj = (uint32_t)min((uint64_t)S::TJ, d.nj - j0);
+    const uint64_t d_el = d_off + j0 * d.dj + i0;
+    const uint8_t* sp = src + (s_off + i0 * d.si + j0) * ES;
+    uint8_t* dp = dst + d_el * ES;
+    const uint32_t csum_base = (uint32_t)(d_el * ES) + d.csum_bias;
+    uint8_t* my_lds = lds + wave * S::kLdsBytes;
+    if (d.vec_src && d.vec_dst && ni == (uint32_t)S::RI && nj == (uint32_t)S::TJ)
+      move_subtile<ES, true>(sp, dp, ni, nj, d.si * ES, d.dj * ES, csum_base, true, true, my_lds, cs);
+    else
+      move_subtile<ES, false>(sp, dp, ni, nj, d.si * ES, d.dj * ES, csum_base, d.vec_src != 0, d.vec_dst != 0, my_lds, cs);
   }
 
   if (sum_out) {
-    __shared__ uint32_t part[kThreads / 64];
+    // Each wavefront leaves its partial sum in the first dword of its own LDS region (its
+    // data-path accesses to that region are complete in issue order).
     const uint32_t w = wave_sum_u32(cs.fold());
-    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = w;
+    if ((threadIdx.x & 63) == 0) *reinterpret_cast<uint32_t*>(lds + wave * S::kLdsBytes) = w;
     __syncthreads();
     if (threadIdx.x == 0) {
       uint32_t t = 0;
 #pragma unroll
-      for (int k = 0; k < kThreads / 64; ++k) t += part[k];
+      for (int k = 0; k < kWaves; ++k) t += *reinterpret_cast<const uint32_t*>(lds + k * S::kLdsBytes);
       atomicAdd(sum_out, t);
     }
   }
@@ -231,9 +291,8 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
                             uint32_t* sum_out, hipStream_t stream) {
   if (d.n_tiles == 0) return hipSuccess;
-  const uint64_t blocks = (d.n_tiles + kTilesPerGroup - 1) / kTilesPerGroup;
-  if (blocks > 0x7FFFFFFFull) return hipErrorInvalidValue;
-  const dim3 grid((uint32_t)blocks), block(kThreads);
+  if (d.n_tiles > 0x7FFFFFFFull || d.waves_i == 0 || kWaves % d.waves_i) return hipErrorInvalidValue;
+  const dim3 grid((uint32_t)d.n_tiles), block(kThreads);
   const uint8_t* s = static_cast<const uint8_t*>(src);
   uint8_t* t = static_cast<uint8_t*>(dst);
   switch (elem_size) {

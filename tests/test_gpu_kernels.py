@@ -186,6 +186,18 @@ def test_shard_region_matches_oracle(gpu_engine, oracle):
     ((7, 5, 6, 9), (3, 1, 0, 2), 4),     # 4-D
     ((6, 1, 33), (2, 1, 0), 2),          # unit dim dropped
     ((1000,), (0,), 2),
+    ((256, 384), (1, 0), 1),             # whole sub-tiles only, every element size
+    ((1024, 192), (1, 0), 2),
+    ((192, 96), (1, 0), 4),
+    ((128, 48), (1, 0), 8),
+    ((200, 300), (1, 0), 1),             # ragged in both directions
+    ((600, 200), (1, 0), 2),             # ragged, 16-byte accesses on both sides
+    ((600, 201), (1, 0), 2),             # source rows not 16-byte aligned
+    ((601, 200), (1, 0), 2),             # destination rows not 16-byte aligned
+    ((3, 520, 136), (0, 2, 1), 4),
+    ((16, 1024), (1, 0), 2),             # destination rows shorter than a sub-tile
+    ((1024, 16), (1, 0), 2),             # source rows shorter than a sub-tile
+    ((2, 3, 70, 130), (1, 3, 0, 2), 2),  # two batch dimensions, transposed inner pair
 ])
 def test_permute_copy_matches_oracle(gpu_engine, oracle, oracle_c, shape, perm, es):
     rng = np.random.default_rng(17)
@@ -197,6 +209,25 @@ def test_permute_copy_matches_oracle(gpu_engine, oracle, oracle_c, shape, perm, 
     d = torch.full((n * es + 16,), 0xEE, dtype=torch.uint8, device="cuda")
     csum = gpu_engine.permute_copy(_dev(raw), d, shape, perm, es)
     assert d[: n * es].cpu().numpy().tobytes() == want.tobytes()
+    assert int((d[n * es:] != 0xEE).sum()) == 0
+    assert csum == oracle_c.checksum32(np.frombuffer(want.tobytes(), dtype=np.uint8))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_permute_copy_random(gpu_engine, oracle, oracle_c, seed):
+    """Random shapes, permutations and element sizes against the element-enumerating oracle."""
+    rng = np.random.default_rng(900 + seed)
+    nd = int(rng.integers(2, 5))
+    es = int(rng.choice([1, 2, 4, 8]))
+    shape = tuple(int(x) for x in rng.integers(1, {2: 700, 3: 90, 4: 30}[nd], nd))
+    perm = tuple(int(x) for x in rng.permutation(nd))
+    n = int(np.prod(shape))
+    raw = rng.integers(0, 256, n * es, dtype=np.uint8)
+    src = oracle.OTensor(raw.reshape(shape + (es,)), {1: "U8", 2: "BF16", 4: "F32", 8: "I64"}[es])
+    want = oracle.permute_copy(src, perm)
+    d = torch.full((n * es + 16,), 0xEE, dtype=torch.uint8, device="cuda")
+    csum = gpu_engine.permute_copy(_dev(raw), d, shape, perm, es)
+    assert d[: n * es].cpu().numpy().tobytes() == want.tobytes(), (shape, perm, es)
     assert int((d[n * es:] != 0xEE).sum()) == 0
     assert csum == oracle_c.checksum32(np.frombuffer(want.tobytes(), dtype=np.uint8))
 
