@@ -66,6 +66,9 @@ def main() -> int:
                     help="benchmark configuration (1-based); 2 = Llama-3-8B, the one the metric is quoted on")
     ap.add_argument("--rank", type=int, default=3, help="tensor-parallel (and expert-parallel) rank whose share is placed")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the configuration's own)")
+    ap.add_argument("--rank-local", action="store_true",
+                    help="keep only the tensors this rank reads in the checkpoint (an expert-parallel rank never "
+                         "opens the other ranks' experts): lets the full-depth DeepSeek-V3 share fit one GPU")
     ap.add_argument("--max-file-gb", type=float, default=40.0,
                     help="write real checkpoint files (ingest and CPU legs) only below this size")
     ap.add_argument("--tile-kib", type=int, default=0, help="destination KiB per workgroup (0 = library default)")
@@ -100,7 +103,7 @@ def main() -> int:
         layout.dims["layers"] = args.layers
         if args.config == 5:
             n_shards = max(1, round(163 * args.layers / 61))
-    elif args.config == 5:
+    elif args.config == 5 and not args.rank_local:
         # The whole 681 GB model cannot be staged on one GPU: 3 dense + 8 MoE layers are run
         # at their real shapes (per-layer work is identical across the 58 MoE layers).
         layout.dims["layers"] = 11
@@ -116,6 +119,26 @@ def main() -> int:
     ep_rank = rank % ep
     rv = layout.rank_view(tp_size=tp, tp_rank=rank, ep_size=ep, ep_rank=ep_rank, param_dtype="BF16" if cast else None)
     host_threads = min(16, os.cpu_count() or 1)
+    dropped = 0
+    if args.rank_local:
+        # Plan once against headers of the whole checkpoint, then keep what the plan reads.
+        hdr_dir = tempfile.mkdtemp(prefix="mxp_bench_full_hdr_")
+        try:
+            synth.write_headers_only(tensors, hdr_dir, n_shards=n_shards)
+            full_ck = Checkpoint(hdr_dir)
+            full_plan = PlacementPlan(full_ck, rv.params, tp_size=tp, tp_rank=rank,
+                                      stacked_params_mapping=rv.stacked_params_mapping,
+                                      expert_mapping=rv.expert_mapping, allow_cast=cast)
+            used = {w.tensor for w in full_plan.writes()}
+            full_plan.close()
+            full_ck.close()
+        finally:
+            shutil.rmtree(hdr_dir, ignore_errors=True)
+        dropped = sum(t.nbytes for t in tensors if t.name not in used)
+        tensors = [t for t in tensors if t.name in used]
+        _log(f"rank-local checkpoint: {len(tensors)} tensors kept, {dropped / 1e9:.1f} GB of other ranks' tensors dropped")
+        total_bytes = sum(t.nbytes for t in tensors)
+        n_shards = max(1, min(n_shards, round(total_bytes / 4.3e9)))
     workloads = {
         1: "configs[0]: GPT-2-small-shaped fp16 checkpoint, one safetensors file; every tensor placed unsliced (TP=1) "
            "with its checksum",
@@ -196,7 +219,8 @@ def main() -> int:
             "dtype": "f32->bf16" if cast else "u8", "data": "synthetic",
             "config": {"workload": workloads[args.config], "family": layout.family,
                        "layers": n_layers, "tp_size": tp, "tp_rank": rank, "ep_size": ep, "ep_rank": ep_rank,
-                       "checkpoint_bytes": total_bytes,
+                       "checkpoint_bytes": total_bytes, "rank_local_checkpoint": bool(args.rank_local),
+                       "other_ranks_bytes_dropped": dropped,
                        "placed_bytes": placed, "buffers": len(plan.params), "timed": "device placement, one launch per step"},
             "roofline": roofline,
         }
