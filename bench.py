@@ -261,6 +261,24 @@ def main() -> int:
                 ops[label] = {"bytes": nbytes, "ms": round(ms, 4), "gbps_algorithmic": round(2 * nbytes / ms / 1e6, 1),
                               "frac_of_hbm_peak": round(2 * nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
                 del a, b
+            # the other conversions of copy_ on 2^28 elements (6 bytes of traffic per element)
+            n_el = 1 << 28
+            for src_dt, dst_dt in (("BF16", "F32"), ("F32", "F16")):
+                se, de = (2, 4) if src_dt == "BF16" else (4, 2)
+                a = torch.empty(n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256)
+                b = torch.empty(n_el * de, dtype=torch.uint8, device="cuda")
+                eng.cast(a, b, n_el, src_dt, dst_dt, checksum=False)
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ev0.record()
+                for _ in range(10):
+                    eng.cast(a, b, n_el, src_dt, dst_dt, checksum=False)
+                ev1.record()
+                torch.cuda.synchronize()
+                ms = ev0.elapsed_time(ev1) / 10
+                ops[f"cast_{src_dt.lower()}_{dst_dt.lower()}"] = {
+                    "elements": n_el, "ms": round(ms, 4), "gbps_algorithmic": round(6 * n_el / ms / 1e6, 1),
+                    "frac_of_hbm_peak": round(6 * n_el / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                del a, b
             out["ops"] = ops
 
         # ---- end-to-end ingest from files through the pinned ring ----

@@ -4,7 +4,7 @@
  * The library turns safetensors byte ranges on local storage into one serving rank's
  * parameter buffers in HBM: host-staged ingest through a bounded ring of pinned
  * buffers, then hand-written gfx950 kernels for tensor-parallel slicing, QKV / gate_up
- * fusing, MoE expert stacking, fp32->bf16 refit casts, fp8 block-scale tile slicing and
+ * fusing, MoE expert stacking, fp32->bf16 refit casts (and the receive-side widening ones), fp8 block-scale tile slicing and
  * per-tensor checksums.
  *
  * The boundary is plain C: opaque handles, pointers and sizes.  Device pointers are
@@ -121,7 +121,8 @@ int64_t mxp_ckpt_find(const mxp_ckpt* ckpt, const char* name);
  * ========================================================================= */
 typedef struct mxp_plan mxp_plan;
 
-#define MXP_PLAN_ALLOW_CAST_F32_BF16 0x1u /* F32 source into BF16 parameter (refit)       */
+#define MXP_PLAN_ALLOW_CAST_F32_BF16 0x1u /* plan a dtype conversion where source and       */
+#define MXP_PLAN_ALLOW_CAST MXP_PLAN_ALLOW_CAST_F32_BF16 /* parameter dtypes differ (MXP_CAST_*) */
 #define MXP_PLAN_ALLOW_UNMAPPED 0x2u      /* skip checkpoint tensors with no destination  */
 #define MXP_PLAN_ALLOW_UNCOVERED 0x4u     /* allow parameters no tensor writes            */
 #define MXP_PLAN_NO_FP8_BLOCK_CHECK 0x8u  /* do not require 128-aligned fp8 scale slicing */
@@ -158,6 +159,17 @@ int mxp_plan_add_virtual_shard(mxp_plan* plan, int64_t virtual_index, const char
                                const int64_t* source_offset, const int64_t* shard_offset, const int64_t* shape);
 int mxp_plan_build(mxp_plan* plan);
 
+/* dtype conversions of dest.copy_(src): trainer fp32 -> wire bf16
+ * (modelexpress_rl/train/engines/fsdp/adapter.py:203-206, publisher.py:44), served bf16 staging
+ * -> fp32 receive buffer (refit/reshard/receiver.py:962-969), and their fp16 counterparts.
+ * Narrowing rounds to nearest even; fp32 -> bf16 maps every NaN to mxp_engine_options.nan_bits;
+ * the fp16 conversions keep a NaN's top payload bits and make it quiet. */
+#define MXP_CAST_NONE 0
+#define MXP_CAST_F32_BF16 1
+#define MXP_CAST_BF16_F32 2
+#define MXP_CAST_F16_F32 3
+#define MXP_CAST_F32_F16 4
+
 #define MXP_WRITE_DIRECT 0
 #define MXP_WRITE_FUSED 1
 #define MXP_WRITE_EXPERT 2
@@ -167,7 +179,7 @@ typedef struct mxp_write_info {
   int64_t tensor_index; /* source tensor in the checkpoint */
   int64_t param_index;  /* destination parameter */
   int32_t kind;         /* MXP_WRITE_* */
-  int32_t cast;         /* 1 when fp32 -> bf16 */
+  int32_t cast;         /* MXP_CAST_* */
   /* The write as a pitched box, in bytes of the respective dtype. */
   uint64_t src_offset;  /* from the start of the source tensor's data */
   uint64_t src_pitch;
@@ -285,6 +297,10 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
  * checksum of the bf16 bytes in *checksum when not NULL. */
 int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems,
                       uint32_t* checksum, void* stream);
+/* Any MXP_CAST_* conversion of `n_elems` contiguous elements (same call sites), with the
+ * checksum of the destination bytes in *checksum when not NULL. */
+int mxp_cast(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems, int32_t cast,
+             uint32_t* checksum, void* stream);
 /* Pitched 2-D byte gather, the device form of narrow(axis, r*n, n).contiguous()
  * (installer.py:317) and of the as_strided re-slice (receiver.py:919-960). */
 int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* dst,
@@ -300,7 +316,7 @@ typedef struct mxp_box {
   uint64_t row_bytes;  /* destination bytes per row */
   uint64_t csum_index; /* checksum position of the first destination byte */
   uint32_t csum_group; /* which output checksum this box adds to, 0 .. n_groups-1 */
-  uint32_t cast;       /* 1: source is fp32, destination bf16 */
+  uint32_t cast;       /* MXP_CAST_*; row_bytes counts destination bytes */
 } mxp_box;
 /* n boxes in one launch: the batched form of the staged re-slice of
  * refit/reshard/receiver.py:919-960 (as_strided + copy_ per view) and of shard_region

@@ -139,6 +139,7 @@ SIGNATURES = {
     "mxp_checksum32": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_digest": (C.c_int, [_P, _PP, _U64P, C.c_int64, C.POINTER(C.c_uint8), _U64P, _P]),
     "mxp_cast_f32_bf16": (C.c_int, [_P, _P, _P, C.c_uint64, _U32P, _P]),
+    "mxp_cast": (C.c_int, [_P, _P, _P, C.c_uint64, C.c_int32, _U32P, _P]),
     "mxp_gather2d": (C.c_int, [_P, _P, C.c_uint64, _P, C.c_uint64, C.c_uint64, C.c_uint64, _U32P, _P]),
     "mxp_place_boxes": (C.c_int, [_P, C.POINTER(Box), C.c_int64, C.c_uint32, _U32P, _P]),
     "mxp_permute_copy": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64),

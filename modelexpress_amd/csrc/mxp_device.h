@@ -3,7 +3,7 @@
 // Everything the device executes is driven by flat descriptor tables built on
 // the host: a "segment" is one pitched 2-D byte box (rows x row_bytes) moving
 // from a source buffer to a destination buffer, optionally through the
-// fp32->bf16 cast, with the position-weighted checksum of the bytes it writes
+// dtype conversion, with the position-weighted checksum of the bytes it writes
 // accumulated on the way.  A "work item" is one tile (a band of rows) of one
 // segment; one workgroup executes one work item, so one launch covers an
 // arbitrary mix of tensors with thousands of workgroups.
@@ -16,8 +16,27 @@ namespace mxp {
 enum SegOp : uint32_t {
   kOpCopy = 0,       // dst bytes = src bytes
   kOpCastF32Bf16 = 1,  // src is fp32, dst is bf16 (round to nearest even)
-  kOpChecksumOnly = 2  // read src, write nothing, accumulate checksum at dst_off indices
+  kOpChecksumOnly = 2,  // read src, write nothing, accumulate checksum at dst_off indices
+  kOpCastBf16F32 = 3,  // src is bf16, dst is fp32 (exact)
+  kOpCastF16F32 = 4,   // src is fp16, dst is fp32 (exact; NaNs made quiet)
+  kOpCastF32F16 = 5    // src is fp32, dst is fp16 (round to nearest even)
 };
+constexpr bool op_narrows(uint32_t op) { return op == kOpCastF32Bf16 || op == kOpCastF32F16; }
+constexpr bool op_widens(uint32_t op) { return op == kOpCastBf16F32 || op == kOpCastF16F32; }
+// Source bytes that produce `dst_bytes` destination bytes.
+constexpr uint64_t op_src_bytes(uint32_t op, uint64_t dst_bytes) {
+  return op_narrows(op) ? dst_bytes * 2 : op_widens(op) ? dst_bytes / 2 : dst_bytes;
+}
+// Destination bytes produced from `src_bytes` source bytes.
+constexpr uint64_t op_dst_bytes(uint32_t op, uint64_t src_bytes) {
+  return op_narrows(op) ? src_bytes / 2 : op_widens(op) ? src_bytes * 2 : src_bytes;
+}
+// Public conversion code of a write record (0 none, 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32,
+// 4 fp32->fp16) -> segment operation.
+constexpr uint32_t seg_op_of_cast(int cast) {
+  return cast == 1 ? kOpCastF32Bf16 : cast == 2 ? kOpCastBf16F32 : cast == 3 ? kOpCastF16F32
+       : cast == 4 ? kOpCastF32F16 : kOpCopy;
+}
 
 // 80 bytes, 16-byte aligned; the index is workgroup-uniform, so the whole record
 // arrives through scalar loads.
@@ -28,11 +47,11 @@ struct alignas(16) Seg {
   uint64_t src_pitch;  // bytes between consecutive rows in the source
   uint64_t dst_pitch;  // bytes between consecutive rows in the destination
   uint32_t rows;
-  uint32_t row_bytes;  // DESTINATION bytes per row (source bytes are 2x for the cast)
+  uint32_t row_bytes;  // DESTINATION bytes per row (source bytes: op_src_bytes)
   uint32_t src_buf;    // index into the source base-pointer table
   uint32_t dst_buf;    // index into the destination base-pointer table
   uint32_t op;         // SegOp
-  uint32_t unit;       // bytes per lane access on the destination side: 16, 8 (cast), 4, 2 or 1
+  uint32_t unit;       // bytes per lane access on the destination side: 16, 8 (narrowing cast), 4, 2 or 1
   uint32_t rows_per_tile;
   uint32_t csum_slot;  // index into the checksum accumulator array, ~0u = none
   uint32_t units_per_row;  // row_bytes / unit

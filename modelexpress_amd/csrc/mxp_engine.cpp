@@ -167,11 +167,11 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       b.dst_pitch = w.dst_pitch;
       b.rows = w.rows;
       b.row_bytes = w.row_bytes;
-      b.op = w.cast ? kOpCastF32Bf16 : kOpCopy;
+      b.op = seg_op_of_cast(w.cast);
       b.csum_slot = (uint32_t)w.param;
       lower_box(b, lo, segs, work);
       L->placed_bytes += w.rows * w.row_bytes;
-      L->algo_bytes += w.rows * w.row_bytes * (w.cast ? 3 : 2);
+      L->algo_bytes += w.rows * (w.row_bytes + op_src_bytes(b.op, w.row_bytes));
     }
     L->res_n_segs = (uint32_t)segs.size();
     L->res_n_work = (uint32_t)work.size();
@@ -190,26 +190,26 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   const uint64_t slot = L->direct_io ? eng.opt.slot_bytes - 2 * blk : eng.opt.slot_bytes;
   for (const auto& w : pl.writes) {
     const TensorRec& t = ck.tensors[w.tensor];
-    const uint64_t sm = w.cast ? 2 : 1;
-    const uint64_t row_src = w.row_bytes * sm;
+    const uint32_t op = seg_op_of_cast(w.cast);
+    const uint64_t row_src = op_src_bytes(op, w.row_bytes);
     BoxCopy b;
     b.src_buf = 0;
     b.dst_buf = (uint32_t)w.param;
-    b.op = w.cast ? kOpCastF32Bf16 : kOpCopy;
+    b.op = op;
     b.csum_slot = (uint32_t)w.param;
     const uint64_t t0 = t.file_offset + w.src_offset;
     if (w.rows == 1 || (w.src_pitch == row_src && w.dst_pitch == w.row_bytes)) {
       // contiguous run: split on 4 KiB multiples of destination bytes
       const uint64_t total = w.rows * w.row_bytes;
-      const uint64_t max_dst = (slot / sm) / 4096 * 4096;
+      const uint64_t max_dst = std::min(slot, op_dst_bytes(op, slot)) / 4096 * 4096;
       for (uint64_t done = 0; done < total; done += max_dst) {
         const uint64_t n = std::min(max_dst, total - done);
-        Piece p{t.file_index, t0 + done * sm, n * sm, b};
+        Piece p{t.file_index, t0 + op_src_bytes(op, done), op_src_bytes(op, n), b};
         p.box.src_off = 0;
         p.box.dst_off = w.dst_offset + done;
         p.box.rows = 1;
         p.box.row_bytes = n;
-        p.box.src_pitch = n * sm;
+        p.box.src_pitch = op_src_bytes(op, n);
         p.box.dst_pitch = n;
         pieces.push_back(p);
       }
@@ -700,7 +700,7 @@ int mxp_plan_totals(const mxp_plan* plan, uint64_t* file_bytes, uint64_t* h2d_by
     uint64_t placed = 0, algo = 0;
     for (const auto& w : plan->writes) {
       placed += w.rows * w.row_bytes;
-      algo += w.rows * w.row_bytes * (w.cast ? 3 : 2);
+      algo += w.rows * (w.row_bytes + op_src_bytes(seg_op_of_cast(w.cast), w.row_bytes));
     }
     if (placed_bytes) *placed_bytes = placed;
     if (kernel_algorithmic_bytes) *kernel_algorithmic_bytes = algo;
@@ -736,23 +736,25 @@ int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* 
   });
 }
 
-int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems, uint32_t* checksum,
-                      void* stream) {
+int mxp_cast(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems, int32_t cast, uint32_t* checksum,
+             void* stream) {
   return guard([&] {
-    if (!engine || (n_elems && (!src || !dst))) throw Error(MXP_ERR_ARG, "mxp_cast_f32_bf16: bad argument");
+    if (!engine || (n_elems && (!src || !dst))) throw Error(MXP_ERR_ARG, "mxp_cast: bad argument");
+    if (cast < MXP_CAST_F32_BF16 || cast > MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_cast: unknown conversion code");
     if (checksum) *checksum = 0;
     if (n_elems == 0) return;
     HIP_OK(hipSetDevice(engine->opt.device));
-    if ((reinterpret_cast<uintptr_t>(src) & 3u) || (reinterpret_cast<uintptr_t>(dst) & 1u))
-      throw Error(MXP_ERR_ARG, "mxp_cast_f32_bf16: pointers must be element aligned");
-    if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_cast_f32_bf16: dst must be 16-byte aligned");
+    const uint32_t op = seg_op_of_cast(cast);
+    const uint64_t dst_es = op_widens(op) ? 4 : 2, src_es = op_widens(op) ? 2 : 4;
+    if (reinterpret_cast<uintptr_t>(src) % src_es) throw Error(MXP_ERR_ARG, "mxp_cast: src must be element aligned");
+    if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_cast: dst must be 16-byte aligned");
     const void* sb;
     uint64_t so;
     split_ptr(src, sb, so);
     BoxCopy b;
     b.src_off = so;
-    b.row_bytes = n_elems * 2;
-    b.op = kOpCastF32Bf16;
+    b.row_bytes = n_elems * dst_es;
+    b.op = op;
     b.csum_slot = 0;
     std::vector<BoxCopy> boxes{b};
     uint32_t sum = 0;
@@ -760,6 +762,11 @@ int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n
               static_cast<hipStream_t>(stream));
     if (checksum) *checksum = sum;
   });
+}
+
+int mxp_cast_f32_bf16(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems, uint32_t* checksum,
+                      void* stream) {
+  return mxp_cast(engine, src, dst, n_elems, MXP_CAST_F32_BF16, checksum, stream);
 }
 
 int mxp_gather2d(mxp_engine* engine, const void* src, uint64_t src_pitch, void* dst, uint64_t dst_pitch,
@@ -807,8 +814,11 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n
       if (x.rows == 0 || x.row_bytes == 0) continue;
       if (!x.src || !x.dst) throw Error(MXP_ERR_ARG, "mxp_place_boxes: null pointer");
       if (x.csum_group >= (n_groups ? n_groups : 1)) throw Error(MXP_ERR_ARG, "mxp_place_boxes: csum_group out of range");
-      const uint64_t sm = x.cast ? 2 : 1;
-      if (x.rows > 1 && (x.src_pitch < x.row_bytes * sm || x.dst_pitch < x.row_bytes))
+      if (x.cast > (uint32_t)MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_place_boxes: unknown conversion code");
+      const uint32_t op = seg_op_of_cast((int)x.cast);
+      if ((op_narrows(op) && x.row_bytes % 2) || (op_widens(op) && x.row_bytes % 4))
+        throw Error(MXP_ERR_ARG, "mxp_place_boxes: row_bytes is not a whole number of elements");
+      if (x.rows > 1 && (x.src_pitch < op_src_bytes(op, x.row_bytes) || x.dst_pitch < x.row_bytes))
         throw Error(MXP_ERR_ARG, "mxp_place_boxes: pitch smaller than the row");
       const void* sb;
       const void* db;
@@ -826,7 +836,7 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n
       b.dst_pitch = x.dst_pitch;
       b.rows = x.rows;
       b.row_bytes = x.row_bytes;
-      b.op = x.cast ? kOpCastF32Bf16 : kOpCopy;
+      b.op = op;
       b.csum_slot = out_checksums ? x.csum_group : 0xFFFFFFFFu;
       b.csum_bias = x.csum_index - d_o;  // positions are relative to the caller's buffer, not the aligned base
       boxes.push_back(b);

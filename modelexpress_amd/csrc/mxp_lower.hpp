@@ -12,7 +12,8 @@
 namespace mxp {
 
 // One logical box of any size: `rows` rows of `row_bytes` DESTINATION bytes each.
-// For kOpCastF32Bf16 the source row is 2 * row_bytes long.
+// The source row is op_src_bytes(op, row_bytes) long (twice as long for a narrowing cast,
+// half as long for a widening one).
 struct BoxCopy {
   uint32_t src_buf = 0, dst_buf = 0;
   uint64_t src_off = 0, dst_off = 0;
@@ -29,14 +30,12 @@ struct LowerOptions {
   uint32_t max_row_bytes = 32768;   // wider pitched rows are split by columns
 };
 
-inline uint32_t src_mul(uint32_t op) { return op == kOpCastF32Bf16 ? 2u : 1u; }
-
 inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& segs,
                      std::vector<WorkItem>& work) {
   if (b.rows == 0 || b.row_bytes == 0) return;
   if (b.rows > 0xFFFFFFFFull || b.row_bytes > o.max_row_bytes)
     throw std::logic_error("emit_seg: box not normalised");
-  const uint64_t sm = src_mul(b.op);
+  const uint64_t src_row = op_src_bytes(b.op, b.row_bytes);
   const bool pitched = b.rows > 1;
   auto all_mult = [&](uint64_t m_dst, uint64_t m_src) {
     if (b.dst_off % m_dst || b.row_bytes % m_dst) return false;
@@ -45,20 +44,24 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
     return true;
   };
   uint32_t unit;
-  if (b.op == kOpCastF32Bf16) {
+  if (op_narrows(b.op)) {
     if (all_mult(8, 16)) unit = 8;
     else if (all_mult(2, 4)) unit = 2;
+    else throw std::invalid_argument("cast box is not element aligned");
+  } else if (op_widens(b.op)) {
+    if (all_mult(16, 8)) unit = 16;
+    else if (all_mult(4, 2)) unit = 4;
     else throw std::invalid_argument("cast box is not element aligned");
   } else {
     unit = all_mult(16, 16) ? 16 : all_mult(4, 4) ? 4 : 1;
   }
-  const uint64_t max_pitch = pitched ? std::max(b.src_pitch, b.dst_pitch) : b.row_bytes * sm;
+  const uint64_t max_pitch = pitched ? std::max(b.src_pitch, b.dst_pitch) : std::max(b.row_bytes, src_row);
   if (max_pitch >= (1ull << 31)) throw std::invalid_argument("row pitch of 2 GiB or more is not supported");
 
   Seg s{};
   s.src_off = b.src_off;
   s.dst_off = b.dst_off;
-  s.src_pitch = pitched ? b.src_pitch : b.row_bytes * sm;
+  s.src_pitch = pitched ? b.src_pitch : src_row;
   s.dst_pitch = pitched ? b.dst_pitch : b.row_bytes;
   s.rows = (uint32_t)b.rows;
   s.row_bytes = (uint32_t)b.row_bytes;
@@ -70,7 +73,7 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
   s.csum_bias = (uint32_t)b.csum_bias;
   s.units_per_row = s.row_bytes / unit;
   s.div_magic = s.units_per_row > 1 ? (uint32_t)((1ull << 32) / s.units_per_row) + 1u : 0u;
-  uint64_t rpt = std::max<uint64_t>(1, o.tile_bytes / (b.row_bytes * sm));
+  uint64_t rpt = std::max<uint64_t>(1, o.tile_bytes / std::max(b.row_bytes, src_row));
   rpt = std::min<uint64_t>(rpt, b.rows);
   // In-tile byte offsets are 32-bit on the device, and the reciprocal division is exact
   // only while (units in tile) * (units per row) < 2^32.
@@ -90,10 +93,11 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
 inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>& segs,
                       std::vector<WorkItem>& work) {
   if (in.rows == 0 || in.row_bytes == 0) return;
-  const uint64_t sm = src_mul(in.op);
+  const uint32_t op = in.op;
+  const bool is_cast = op_narrows(op) || op_widens(op);
   BoxCopy b = in;
   // Rows that abut in both layouts are one contiguous run.
-  if (b.rows > 1 && b.src_pitch == b.row_bytes * sm && b.dst_pitch == b.row_bytes) {
+  if (b.rows > 1 && b.src_pitch == op_src_bytes(op, b.row_bytes) && b.dst_pitch == b.row_bytes) {
     b.row_bytes *= b.rows;
     b.rows = 1;
   }
@@ -105,11 +109,11 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
     while (full) {
       const uint64_t n = std::min<uint64_t>(full, 0x80000000ull);
       BoxCopy m = b;
-      m.src_off = b.src_off + done * sm;
+      m.src_off = b.src_off + op_src_bytes(op, done);
       m.dst_off = b.dst_off + done;
       m.rows = n;
       m.row_bytes = W;
-      m.src_pitch = W * sm;
+      m.src_pitch = op_src_bytes(op, W);
       m.dst_pitch = W;
       emit_seg(m, o, segs, work);
       done += n * W;
@@ -118,17 +122,17 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
     const uint64_t rem = b.row_bytes - done;
     if (rem) {
       // Keep the 16-byte path for as much of the remainder as possible.
-      const uint64_t body = (b.op == kOpCastF32Bf16) ? rem : (rem / 16) * 16;
+      const uint64_t body = is_cast ? rem : (rem / 16) * 16;
       BoxCopy m = b;
       m.rows = 1;
       if (body) {
-        m.src_off = b.src_off + done * sm;
+        m.src_off = b.src_off + op_src_bytes(op, done);
         m.dst_off = b.dst_off + done;
         m.row_bytes = body;
         emit_seg(m, o, segs, work);
       }
       if (rem - body) {
-        m.src_off = b.src_off + (done + body) * sm;
+        m.src_off = b.src_off + op_src_bytes(op, done + body);
         m.dst_off = b.dst_off + done + body;
         m.row_bytes = rem - body;
         emit_seg(m, o, segs, work);
@@ -141,7 +145,7 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
     const uint64_t cw = std::min<uint64_t>(o.max_row_bytes, b.row_bytes - c);
     for (uint64_t r = 0; r < b.rows; r += 0x80000000ull) {
       BoxCopy m = b;
-      m.src_off = b.src_off + r * b.src_pitch + c * sm;
+      m.src_off = b.src_off + r * b.src_pitch + op_src_bytes(op, c);
       m.dst_off = b.dst_off + r * b.dst_pitch + c;
       m.rows = std::min<uint64_t>(0x80000000ull, b.rows - r);
       m.row_bytes = cw;

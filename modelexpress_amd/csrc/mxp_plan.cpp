@@ -283,9 +283,13 @@ struct Planner {
     ParamRec& p = pl.params[dst.param];
     int cast = 0;
     if (t.dtype != p.dtype) {
-      if (t.dtype == MXP_DTYPE_F32 && p.dtype == MXP_DTYPE_BF16 && (pl.flags & MXP_PLAN_ALLOW_CAST_F32_BF16))
-        cast = 1;
-      else
+      if (pl.flags & MXP_PLAN_ALLOW_CAST) {
+        if (t.dtype == MXP_DTYPE_F32 && p.dtype == MXP_DTYPE_BF16) cast = MXP_CAST_F32_BF16;
+        else if (t.dtype == MXP_DTYPE_BF16 && p.dtype == MXP_DTYPE_F32) cast = MXP_CAST_BF16_F32;
+        else if (t.dtype == MXP_DTYPE_F16 && p.dtype == MXP_DTYPE_F32) cast = MXP_CAST_F16_F32;
+        else if (t.dtype == MXP_DTYPE_F32 && p.dtype == MXP_DTYPE_F16) cast = MXP_CAST_F32_F16;
+      }
+      if (!cast)
         throw Error(MXP_ERR_UNSUPPORTED, "tensor '" + t.name + "' is " + mxp_dtype_name(t.dtype) +
                                              " but parameter '" + p.name + "' is " +
                                              mxp_dtype_name(p.dtype) + "; no conversion is planned");
@@ -309,7 +313,7 @@ struct Planner {
     w.row_bytes = (uint64_t)run * ed;
     auto finish = [&](const WriteRec& r) {
       const uint64_t span = r.dst_offset + (r.rows - 1) * r.dst_pitch + r.row_bytes;
-      const uint64_t sspan = r.src_offset + (r.rows - 1) * r.src_pitch + r.row_bytes * (cast ? 2 : 1);
+      const uint64_t sspan = r.src_offset + (r.rows - 1) * r.src_pitch + r.row_bytes / ed * es;
       if (span > p.nbytes || sspan > t.nbytes)
         throw Error(MXP_ERR_STATE, "internal: write for '" + t.name + "' leaves its buffers");
       p.bytes_written += r.rows * r.row_bytes;
@@ -320,7 +324,7 @@ struct Planner {
       w.rows = 1;
       w.src_offset = (uint64_t)src.base * es;
       w.dst_offset = (uint64_t)dst.base * ed;
-      w.src_pitch = w.row_bytes * (cast ? 2 : 1);
+      w.src_pitch = w.row_bytes / ed * es;
       w.dst_pitch = w.row_bytes;
       w.paired_runs = 1;
       finish(w);

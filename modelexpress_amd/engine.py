@@ -50,12 +50,16 @@ class VirtualTensor:
     shards: tuple
 
 
+# MXP_CAST_* of include/mxp.h
+CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4}
+
+
 @dataclass(frozen=True)
 class WriteEntry:
     tensor: str
     param: str
     kind: str
-    cast: bool
+    cast: int  # 0 or a CAST_CODES value
     src_offset: int
     src_pitch: int
     dst_offset: int
@@ -179,7 +183,7 @@ class PlacementPlan:
         for i in range(int(lib.mxp_plan_write_count(self._h))):
             L.check(lib.mxp_plan_write_info(self._h, i, C.byref(info)))
             out.append(WriteEntry(tensors[info.tensor_index].name, self.params[info.param_index].name,
-                                  L.WRITE_KINDS[info.kind], bool(info.cast), info.src_offset, info.src_pitch,
+                                  L.WRITE_KINDS[info.kind], int(info.cast), info.src_offset, info.src_pitch,
                                   info.dst_offset, info.dst_pitch, info.rows, info.row_bytes, info.paired_runs))
         return out
 
@@ -301,6 +305,17 @@ class PlacementEngine:
         out = C.c_uint32()
         L.check(L.lib().mxp_cast_f32_bf16(self._h, C.c_void_p(_addr(src)), C.c_void_p(_addr(dst)), n_elems,
                                           C.byref(out) if checksum else None, C.c_void_p(stream)))
+        return format(out.value, "08x") if checksum else None
+
+    def cast(self, src, dst, n_elems: int, src_dtype: str, dst_dtype: str, *, stream: int = 0,
+             checksum: bool = True) -> str | None:
+        """``dst.copy_(src)`` across dtypes for the supported pairs (``CAST_CODES``)."""
+        code = CAST_CODES.get((src_dtype, dst_dtype))
+        if code is None:
+            raise ValueError(f"no conversion from {src_dtype} to {dst_dtype}")
+        out = C.c_uint32()
+        L.check(L.lib().mxp_cast(self._h, C.c_void_p(_addr(src)), C.c_void_p(_addr(dst)), n_elems, code,
+                                 C.byref(out) if checksum else None, C.c_void_p(stream)))
         return format(out.value, "08x") if checksum else None
 
     def gather2d(self, src, src_pitch: int, dst, dst_pitch: int, rows: int, row_bytes: int, *, stream: int = 0,

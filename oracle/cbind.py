@@ -33,6 +33,8 @@ class OracleC:
         h.orc_checksum32_at.argtypes = [C.c_void_p, C.c_uint64, C.c_uint64]
         h.orc_digest_scalars.restype = None
         h.orc_digest_scalars.argtypes = [C.c_void_p, C.c_uint64, C.POINTER(C.c_uint64)]
+        h.orc_cast.restype = None
+        h.orc_cast.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint16]
         h.orc_cast_f32_bf16.restype = None
         h.orc_cast_f32_bf16.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint16]
         h.orc_copy2d.restype = None
@@ -55,6 +57,14 @@ class OracleC:
         src = np.ascontiguousarray(u32, dtype=np.uint32)
         dst = np.empty(src.shape, dtype=np.uint16)
         self.h.orc_cast_f32_bf16(src.ctypes.data, dst.ctypes.data, src.size, nan_bits)
+        return dst
+
+    def cast(self, code: int, bits: np.ndarray, nan_bits: int = 0x7FC0) -> np.ndarray:
+        """Conversion ``code`` (1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16) on bit patterns."""
+        widen = code in (2, 3)
+        src = np.ascontiguousarray(bits, dtype=np.uint16 if widen else np.uint32)
+        dst = np.empty(src.shape, dtype=np.uint32 if widen else np.uint16)
+        self.h.orc_cast(code, src.ctypes.data, dst.ctypes.data, src.size, nan_bits)
         return dst
 
     def run_writes(self, writes: list, n_params: int, threads: int, nan_bits: int = 0x7FC0) -> list:

@@ -63,7 +63,8 @@ def run(ckpt_dir: str, rank_params: list, *, tp_size=1, tp_rank=0, stacked=None,
     recs = []
     placed = 0
     for _kind, dest, src in writes:
-        cast = src.dtype != dest.dtype
+        cast = O.CAST_CODES[(src.dtype, dest.dtype)] if src.dtype != dest.dtype else 0
+        se, de = src.data.shape[-1], dest.data.shape[-1]
         base = dest.data
         while base.base is not None and isinstance(base.base, np.ndarray):
             base = base.base
@@ -77,7 +78,7 @@ def run(ckpt_dir: str, rank_params: list, *, tp_size=1, tp_rank=0, stacked=None,
                 step = 4 << 20
                 for lo in range(0, row_bytes, step):
                     n = min(step, row_bytes - lo)
-                    recs.append(cbind.OrcWrite(src=s0 + s_off + lo * (2 if cast else 1), dst=d0 + d_off + lo, src_pitch=0,
+                    recs.append(cbind.OrcWrite(src=s0 + s_off + lo * se // de, dst=d0 + d_off + lo, src_pitch=0,
                                                dst_pitch=0, rows=1, row_bytes=n,
                                                dst_index=d0 + d_off + lo - base_addr[pname], param=index[pname],
                                                cast=int(cast)))

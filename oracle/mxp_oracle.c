@@ -69,6 +69,46 @@ void orc_cast_f32_bf16(const uint32_t* src, uint16_t* dst, uint64_t n, uint16_t 
   for (uint64_t i = 0; i < n; ++i) dst[i] = bf16_bits(src[i], nan_bits);
 }
 
+/* The other conversions of the same copy_ (receive side: refit/reshard/receiver.py:962-969).
+ * Codes: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16. */
+static inline uint32_t f16_to_f32_bits(uint16_t h) {
+  const uint32_t sign = ((uint32_t)h & 0x8000u) << 16, e = (h >> 10) & 0x1Fu, m = h & 0x3FFu;
+  if (e == 31u) return sign | 0x7F800000u | (m << 13) | (m ? 0x400000u : 0u);
+  if (e != 0u) return sign | ((e + 112u) << 23) | (m << 13);
+  if (m == 0u) return sign;
+  uint32_t top = 9;
+  while (!(m >> top)) --top;
+  return sign | ((top + 103u) << 23) | ((m << (23u - top)) & 0x7FFFFFu);
+}
+
+static inline uint16_t f32_to_f16_bits(uint32_t u) {
+  const uint32_t sign = (u >> 16) & 0x8000u, a = u & 0x7FFFFFFFu;
+  if (a > 0x7F800000u) return (uint16_t)(sign | 0x7E00u | ((a >> 13) & 0x3FFu));
+  if (a >= 0x38800000u) {
+    const uint32_t r = a - 0x38000000u;
+    uint32_t h = (r + 0xFFFu + ((r >> 13) & 1u)) >> 13;
+    if (h > 0x7C00u) h = 0x7C00u;
+    return (uint16_t)(sign | h);
+  }
+  const uint32_t e = a >> 23, m = (a & 0x7FFFFFu) | 0x800000u;
+  uint32_t shift = 126u - e;
+  if (shift > 25u) shift = 25u;
+  const uint32_t q = m >> shift, rem = m & ((1u << shift) - 1u), half = 1u << (shift - 1u);
+  return (uint16_t)(sign | (q + ((rem > half) || (rem == half && (q & 1u)))));
+}
+
+/* n elements; returns nothing, dst holds the converted elements */
+void orc_cast(uint32_t code, const void* src, void* dst, uint64_t n, uint16_t nan_bits) {
+  uint64_t i;
+  switch (code) {
+    case 1: orc_cast_f32_bf16((const uint32_t*)src, (uint16_t*)dst, n, nan_bits); break;
+    case 2: for (i = 0; i < n; ++i) ((uint32_t*)dst)[i] = (uint32_t)((const uint16_t*)src)[i] << 16; break;
+    case 3: for (i = 0; i < n; ++i) ((uint32_t*)dst)[i] = f16_to_f32_bits(((const uint16_t*)src)[i]); break;
+    case 4: for (i = 0; i < n; ++i) ((uint16_t*)dst)[i] = f32_to_f16_bits(((const uint32_t*)src)[i]); break;
+    default: break;
+  }
+}
+
 void orc_copy2d(const uint8_t* src, uint64_t src_pitch, uint8_t* dst, uint64_t dst_pitch, uint64_t rows,
                 uint64_t row_bytes) {
   for (uint64_t r = 0; r < rows; ++r) memcpy(dst + r * dst_pitch, src + r * src_pitch, row_bytes);
@@ -81,7 +121,7 @@ typedef struct orc_write {
   uint64_t src_pitch, dst_pitch, rows, row_bytes; /* row_bytes in destination bytes */
   uint64_t dst_index;  /* byte offset of dst inside its parameter (checksum position) */
   uint32_t param;      /* which checksum accumulator */
-  uint32_t cast;       /* 1: fp32 -> bf16 */
+  uint32_t cast;       /* 0 copy, else a conversion code of orc_cast */
 } orc_write;
 
 typedef struct {
@@ -97,7 +137,7 @@ static void run_one(const orc_write* w, uint32_t* sums, uint16_t nan_bits) {
   for (uint64_t r = 0; r < w->rows; ++r) {
     const uint8_t* s = w->src + r * w->src_pitch;
     uint8_t* d = w->dst + r * w->dst_pitch;
-    if (w->cast) orc_cast_f32_bf16((const uint32_t*)s, (uint16_t*)d, w->row_bytes / 2, nan_bits);
+    if (w->cast) orc_cast(w->cast, s, d, w->row_bytes / ((w->cast == 2 || w->cast == 3) ? 4 : 2), nan_bits);
     else memcpy(d, s, w->row_bytes);
     sums[w->param] += orc_checksum32_at(d, w->row_bytes, w->dst_index + r * w->dst_pitch);
   }

@@ -198,6 +198,72 @@ def cast_tensor_f32_bf16(t: OTensor, nan_bits: int = 0x7FC0) -> OTensor:
     return OTensor.from_array(cast_f32_bf16_bits(u32, nan_bits).astype("<u2"), "BF16")
 
 
+# The receive side of the same path converts the other way: "Cast the served bf16 staging
+# into the (fp32) receive buffer - a torch op" (refit/reshard/receiver.py:962-969), and a
+# half-precision engine takes fp32 trainer weights as fp16.  Conversion codes, shared with
+# the product's write records: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16.
+CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4}
+
+
+def cast_bf16_f32_bits(u16: np.ndarray) -> np.ndarray:
+    """Exact: bf16 is the upper half of the fp32 pattern (NaN payloads are kept)."""
+    return u16.astype(np.uint32) << np.uint32(16)
+
+
+_F16_TOP_BIT = np.array([0] + [int(m).bit_length() - 1 for m in range(1, 1024)], dtype=np.uint32)
+
+
+def cast_f16_f32_bits(u16: np.ndarray) -> np.ndarray:
+    """Exact widening.  Subnormal halves are renormalised; a NaN keeps its payload and is
+    made quiet (what hardware converters and torch's CPU path produce)."""
+    h = u16.astype(np.uint32)
+    sign = (h & 0x8000) << 16
+    e = (h >> 10) & 0x1F
+    m = h & 0x3FF
+    normal = sign | ((e + 112) << 23) | (m << 13)
+    top = _F16_TOP_BIT[m]
+    sub = np.where(m == 0, sign, sign | ((top + 103) << 23) | ((m << (23 - top)) & 0x7FFFFF))
+    special = sign | 0x7F800000 | (m << 13) | np.where(m != 0, np.uint32(0x400000), np.uint32(0))
+    return np.where(e == 31, special, np.where(e == 0, sub, normal)).astype(np.uint32)
+
+
+def cast_f32_f16_bits(u32: np.ndarray) -> np.ndarray:
+    """fp32 -> fp16, round to nearest even; overflow goes to infinity, values below half
+    the smallest subnormal to (signed) zero; a NaN keeps the top ten payload bits and is made
+    quiet (the hardware converters' rule, which torch's CPU path follows)."""
+    u = u32.astype(np.uint64)
+    sign = (u >> 16) & 0x8000
+    a = u & 0x7FFFFFFF
+    # normal half range: re-bias the exponent, round the 13 dropped bits to nearest even
+    r = (a - 0x38000000) & 0xFFFFFFFF
+    hn = np.minimum((r + 0xFFF + ((r >> 13) & 1)) >> 13, 0x7C00)
+    # subnormal half: shift the 24-bit significand right, round to nearest even
+    e = a >> 23
+    m = (a & 0x7FFFFF) | 0x800000
+    shift = np.minimum(126 - np.minimum(e, 126), 25).astype(np.uint64)
+    q = m >> shift
+    rem = m & ((np.uint64(1) << shift) - 1)
+    half = np.uint64(1) << (shift - 1)
+    hs = q + ((rem > half) | ((rem == half) & ((q & 1) == 1)))
+    out = np.where(a >= 0x38800000, hn, hs)
+    out = np.where(a > 0x7F800000, 0x7E00 | ((a >> 13) & 0x3FF), out)
+    return (sign | out).astype(np.uint16)
+
+
+def cast_tensor(t: OTensor, dst_dtype: str, nan_bits: int = 0x7FC0) -> OTensor:
+    """dtype conversion of ``dest.copy_(src)`` for the supported pairs."""
+    code = CAST_CODES.get((t.dtype, dst_dtype))
+    if code is None:
+        raise ValueError(f"no conversion from {t.dtype} to {dst_dtype}")
+    src = np.ascontiguousarray(t.data)
+    if code == 1:
+        return cast_tensor_f32_bf16(t, nan_bits)
+    if code == 4:
+        return OTensor.from_array(cast_f32_f16_bits(src.view("<u4").reshape(t.shape)).astype("<u2"), "F16")
+    fn = cast_bf16_f32_bits if code == 2 else cast_f16_f32_bits
+    return OTensor.from_array(fn(src.view("<u2").reshape(t.shape)).astype("<u4"), "F32")
+
+
 # --------------------------------------------------------------------------------------
 # a10: safe_checksum (tensor_utils.py:27-44) over the row-major flat byte stream
 # --------------------------------------------------------------------------------------
@@ -691,8 +757,8 @@ class MdlOracle:
     def _copy(self, dest: OTensor, src: OTensor) -> None:
         if src.dtype == dest.dtype:
             dest.data[...] = src.data
-        elif src.dtype == "F32" and dest.dtype == "BF16" and self.allow_cast:
-            dest.data[...] = cast_tensor_f32_bf16(src, self.nan_bits).data
+        elif (src.dtype, dest.dtype) in CAST_CODES and self.allow_cast:
+            dest.data[...] = cast_tensor(src, dest.dtype, self.nan_bits).data
         else:
             raise RuntimeError(f"no conversion from {src.dtype} to {dest.dtype}")
 

@@ -50,21 +50,46 @@ def apply_plan_numpy(ck: Checkpoint, plan: PlacementPlan, nan_bits=0x7FC0) -> di
         t = tensors[w.tensor]
         src = files[t.file_index][t.file_offset : t.file_offset + t.nbytes]
         dst = out[w.param]
-        mul = 2 if w.cast else 1
+        src_row = {0: w.row_bytes, 1: w.row_bytes * 2, 4: w.row_bytes * 2, 2: w.row_bytes // 2, 3: w.row_bytes // 2}[w.cast]
         for r in range(w.rows):
-            s = src[w.src_offset + r * w.src_pitch : w.src_offset + r * w.src_pitch + w.row_bytes * mul]
-            if w.cast:
+            s = src[w.src_offset + r * w.src_pitch : w.src_offset + r * w.src_pitch + src_row]
+            if w.cast == 1:
                 u = s.view("<u4").astype(np.uint64)
                 b = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
                 b[(u & 0x7FFFFFFF) > 0x7F800000] = nan_bits
                 s = b.view(np.uint8)
+            elif w.cast == 2:
+                s = (s.view("<u2").astype(np.uint32) << 16).view(np.uint8)
+            elif w.cast in (3, 4):  # torch is the library the reference converts with
+                import torch
+                src_t, dst_t = (torch.float16, torch.float32) if w.cast == 3 else (torch.float32, torch.float16)
+                s = torch.from_numpy(s.copy()).view(src_t).to(dst_t).view(torch.uint8).numpy()
             dst[w.dst_offset + r * w.dst_pitch : w.dst_offset + r * w.dst_pitch + w.row_bytes] = s
     return out
 
 
+def cast_setup(ck_kw: dict):
+    """Splits a ``tiny_layouts`` kwargs dict: ``(checkpoint kwargs, param dtype or None, cast?, source bytes per
+    destination byte)``.  An F32 checkpoint without an explicit ``param_dtype`` is the refit into BF16."""
+    kw = dict(ck_kw)
+    param_dtype = kw.pop("param_dtype", None)
+    if param_dtype is None and kw.get("dtype") == "F32":
+        param_dtype = "BF16"
+    size = {"F32": 4, "BF16": 2, "F16": 2}
+    ratio = size[kw.get("dtype") or "BF16"] / size[param_dtype] if param_dtype else 1
+    return kw, param_dtype, param_dtype is not None, ratio
+
+
 def tiny_layouts():
-    """Small instances of the five benchmark families: ``name -> (layout, tp, ep, shards, ckpt kwargs)``."""
+    """Small instances of the five benchmark families: ``name -> (layout, tp, ep, shards, ckpt kwargs)``;
+    a ``param_dtype`` among the kwargs asks for a converting placement (see ``cast_setup``)."""
     return {
+        "llama_bf16_into_f32": (models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
+                                4, 1, 2, {"dtype": "BF16", "edge_cases": models.NORMAL_EDGE_DENSE, "param_dtype": "F32"}),
+        "llama_f16_into_f32": (models.Llama(layers=1, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
+                               2, 1, 1, {"dtype": "F16", "edge_cases": models.NORMAL_EDGE_DENSE, "param_dtype": "F32"}),
+        "llama_f32_into_f16": (models.Llama(layers=1, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
+                               2, 1, 2, {"dtype": "F32", "edge_cases": models.NORMAL_EDGE_DENSE, "param_dtype": "F16"}),
         "gpt2": (models.Gpt2(layers=2, hidden=32, ffn=64, vocab=97, positions=16), 1, 1, 1, {}),
         "llama_tp4": (models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256), 4, 1, 3, {}),
         "llama_f32_refit": (models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),

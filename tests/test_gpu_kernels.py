@@ -86,6 +86,36 @@ def test_cast_f32_bf16_matches_oracle(gpu_engine, oracle, oracle_c):
         assert int(d[src.size * 2:].sum()) == 0  # nothing written past the end
 
 
+@pytest.mark.parametrize("src_dtype,dst_dtype", [("BF16", "F32"), ("F16", "F32"), ("F32", "F16")])
+def test_cast_pairs_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dtype):
+    """The other conversions of dest.copy_(src) (refit/reshard/receiver.py:962-969): every 16-bit
+    pattern for the widening ones, every rounding class for fp32 -> fp16, odd sizes and offsets."""
+    rng = np.random.default_rng(14)
+    code = oracle.CAST_CODES[(src_dtype, dst_dtype)]
+    if src_dtype == "F32":
+        hi = np.arange(1 << 16, dtype=np.uint32) << 16
+        lows = np.array([0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF, 0x2000, 0x3000, 0xFFFF], dtype=np.uint32)
+        full = np.concatenate([(hi[:, None] | lows[None, :]).reshape(-1),
+                               rng.integers(0, 1 << 32, (1 << 20) + 3, dtype=np.uint64).astype(np.uint32)])
+        fn, se, de = oracle.cast_f32_f16_bits, 4, 2
+    else:
+        full = np.concatenate([np.arange(1 << 16, dtype=np.uint16), rng.integers(0, 1 << 16, (1 << 20) + 5, dtype=np.uint16)])
+        fn, se, de = (oracle.cast_bf16_f32_bits if src_dtype == "BF16" else oracle.cast_f16_f32_bits), 2, 4
+    dev = _dev(full)
+    for off, n in ((0, full.size), (0, 1), (1, 7), (3, 8), (5, 4099), (2, 65536 + 11)):
+        src = full[off: off + n]
+        d = torch.zeros(n * de + 16, dtype=torch.uint8, device="cuda")
+        csum = gpu_engine.cast(dev.view(torch.uint8)[off * se:], d, n, src_dtype, dst_dtype)
+        want = fn(src)
+        got = d[: n * de].cpu().numpy().view(want.dtype)
+        assert np.array_equal(got, want), (off, n)
+        assert np.array_equal(oracle_c.cast(code, src), want)
+        assert csum == oracle_c.checksum32(want.view(np.uint8))
+        assert int(d[n * de:].sum()) == 0  # nothing written past the end
+    with pytest.raises(ValueError):
+        gpu_engine.cast(dev, dev, 1, "BF16", "F16")
+
+
 def test_cast_nan_image_is_a_parameter(mxp, oracle):
     from modelexpress_amd.engine import PlacementEngine
 
@@ -262,31 +292,39 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
     want = np.full(out_size, 0xEE, dtype=np.uint8)
     boxes, sums_want, cursor = [], [], 0
     for g in range(int(rng.integers(1, 9))):
-        cast = bool(rng.integers(0, 3) == 0)
-        align = int(rng.choice([1, 2, 4, 8, 16])) if not cast else int(rng.choice([2, 4, 8, 16]))
+        cast = int(rng.choice([0, 0, 0, 1, 2, 3, 4]))  # MXP_CAST_* code
+        narrow, widen = cast in (1, 4), cast in (2, 3)
+        align = int(rng.choice([1, 2, 4, 8, 16])) if not cast else int(rng.choice([4, 8, 16]) if widen else rng.choice([2, 4, 8, 16]))
         rows = int(rng.choice([1, 1, 2, 7, 64, 513, 3000]))
         row_bytes = int(rng.integers(1, 40)) * align if rng.integers(0, 4) else int(rng.integers(1, 5)) * 20000 // align * align
-        row_bytes = max(align, row_bytes - row_bytes % (2 if cast else 1))
-        sm = 2 if cast else 1
+        row_bytes = max(align, row_bytes - row_bytes % (4 if widen else 2 if narrow else 1))
+        src_row = row_bytes * 2 if narrow else row_bytes // 2 if widen else row_bytes
+        src_align = align * 2 if narrow else align // 2 if widen else align
         dst_pitch = row_bytes + int(rng.integers(0, 4)) * align
-        src_pitch = row_bytes * sm + int(rng.integers(0, 5)) * align * (2 if cast else 1)
+        src_pitch = src_row + int(rng.integers(0, 5)) * src_align
         if rows * max(dst_pitch, 1) > (1 << 20) or rows * src_pitch > (4 << 20):
             rows = max(1, min((1 << 20) // dst_pitch, (4 << 20) // src_pitch))
-        src_off = int(rng.integers(0, 64)) * (4 if cast else 1)
-        src_off -= src_off % (4 if cast else min(align, 16))
+        src_off = int(rng.integers(0, 64)) * (4 if narrow else 2 if widen else 1)
+        src_off -= src_off % (min(src_align, 16) if cast else min(align, 16))
         dst_off = (cursor + 15) // 16 * 16
         if rows == 1 and not cast and align < 16 and rng.integers(0, 2):
             dst_off += align  # a byte/dword-granular start inside the buffer
         csum = 0
         for r in range(rows):
-            s = src[src_off + r * src_pitch: src_off + r * src_pitch + row_bytes * sm]
-            if cast:
+            s = src[src_off + r * src_pitch: src_off + r * src_pitch + src_row]
+            if cast == 1:
                 s = oracle.cast_f32_bf16_bits(s.view(np.uint32)).view(np.uint8)
+            elif cast == 4:
+                s = oracle.cast_f32_f16_bits(s.view(np.uint32)).view(np.uint8)
+            elif cast == 2:
+                s = oracle.cast_bf16_f32_bits(s.view(np.uint16)).view(np.uint8)
+            elif cast == 3:
+                s = oracle.cast_f16_f32_bits(s.view(np.uint16)).view(np.uint8)
             want[dst_off + r * dst_pitch: dst_off + r * dst_pitch + row_bytes] = s
             csum += int(oracle_c.checksum32(s, first_index=1000 + r * dst_pitch), 16)
         sums_want.append(format(csum & 0xFFFFFFFF, "08x"))
         boxes.append({"src": d_src.data_ptr() + src_off, "dst": dst_off, "src_pitch": src_pitch, "dst_pitch": dst_pitch,
-                      "rows": rows, "row_bytes": row_bytes, "csum_index": 1000, "csum_group": g, "cast": int(cast)})
+                      "rows": rows, "row_bytes": row_bytes, "csum_index": 1000, "csum_group": g, "cast": cast})
         cursor = dst_off + rows * dst_pitch + 64
         assert cursor < out_size
     out = torch.full((out_size,), 0xEE, dtype=torch.uint8, device="cuda")

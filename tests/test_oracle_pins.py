@@ -204,6 +204,49 @@ def test_cast_matches_torch_cpu_on_every_rounding_class(oracle, oracle_c):
     assert np.array_equal(oracle_c.cast_f32_bf16(rnd), oracle.cast_f32_bf16_bits(rnd))
 
 
+def _torch_convert(bits: np.ndarray, src: str, dst: str) -> np.ndarray:
+    st = {"F32": (torch.float32, np.int32), "BF16": (torch.bfloat16, np.int16), "F16": (torch.float16, np.int16)}
+    ut = {"F32": np.uint32, "BF16": np.uint16, "F16": np.uint16}
+    t = torch.from_numpy(bits.view(st[src][1]).copy()).view(st[src][0]).to(st[dst][0])
+    return t.view(torch.int32 if dst == "F32" else torch.int16).numpy().view(ut[dst])
+
+
+def test_widening_casts_match_torch_on_every_pattern(oracle, oracle_c):
+    # refit/reshard/receiver.py:962-969: recv (fp32) .copy_(staging (bf16)); torch is the library the reference calls
+    h = np.arange(1 << 16, dtype=np.uint16)
+    assert np.array_equal(oracle.cast_bf16_f32_bits(h), _torch_convert(h, "BF16", "F32"))
+    assert np.array_equal(oracle.cast_f16_f32_bits(h), _torch_convert(h, "F16", "F32"))
+    assert np.array_equal(oracle_c.cast(2, h), oracle.cast_bf16_f32_bits(h))
+    assert np.array_equal(oracle_c.cast(3, h), oracle.cast_f16_f32_bits(h))
+    # hand values: 1.0, -2.0, smallest subnormal half (2^-24), largest subnormal, inf, a signalling NaN made quiet
+    hv = np.array([0x3C00, 0xC000, 0x0001, 0x03FF, 0x7C00, 0x7C01], dtype=np.uint16)
+    assert oracle.cast_f16_f32_bits(hv).tolist() == [0x3F800000, 0xC0000000, 0x33800000, 0x387FC000, 0x7F800000, 0x7FC02000]
+    assert oracle.cast_bf16_f32_bits(np.array([0x3F80, 0x7FC1], dtype=np.uint16)).tolist() == [0x3F800000, 0x7FC10000]
+    # exactness: widening then narrowing is the identity on every non-NaN pattern
+    not_nan16 = (h & 0x7FFF) <= 0x7C00
+    assert np.array_equal(oracle.cast_f32_f16_bits(oracle.cast_f16_f32_bits(h))[not_nan16], h[not_nan16])
+    not_nan_bf = (h & 0x7FFF) <= 0x7F80
+    assert np.array_equal(oracle.cast_f32_bf16_bits(oracle.cast_bf16_f32_bits(h))[not_nan_bf], h[not_nan_bf])
+
+
+def test_f32_to_f16_matches_torch_and_numpy(oracle, oracle_c):
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    lows = np.array([0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF, 0x2000, 0x2FFF, 0x3000, 0x7FFF, 0x8000, 0x8001, 0xFFFF],
+                    dtype=np.uint32)
+    u = (hi[:, None] | lows[None, :]).reshape(-1)
+    u = np.concatenate([u, np.random.default_rng(4).integers(0, 1 << 32, 1 << 21, dtype=np.uint64).astype(np.uint32)])
+    got = oracle.cast_f32_f16_bits(u)
+    assert np.array_equal(got, _torch_convert(u, "F32", "F16"))  # NaN payload rule included
+    not_nan = (u & 0x7FFFFFFF) <= 0x7F800000
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got[not_nan], u.view(np.float32).astype(np.float16).view(np.uint16)[not_nan])
+    assert np.array_equal(oracle_c.cast(4, u), got)
+    # hand values: 1.0; 65504 (max half); 65520 -> inf (tie to even overflows); 2^-25 -> 0 (tie to even);
+    # just above 2^-25 -> smallest subnormal; 2^-14 (smallest normal); -0.0
+    hv = np.array([0x3F800000, 0x477FE000, 0x477FF000, 0x33000000, 0x33000001, 0x38800000, 0x80000000], dtype=np.uint32)
+    assert oracle.cast_f32_f16_bits(hv).tolist() == [0x3C00, 0x7BFF, 0x7C00, 0x0000, 0x0001, 0x0400, 0x8000]
+
+
 # ---------------------------------------------------------------- paired_runs --------
 def test_paired_runs_reference_vectors(oracle):
     # tests/test_reshard_refit_slice_plan.py:54-65: narrow(1,0,4) of (4,8) into (4,4)

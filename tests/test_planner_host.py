@@ -5,21 +5,20 @@ oracle's parameter buffers.  No device work happens here."""
 import numpy as np
 import pytest
 
-from helpers import apply_plan_numpy, make_plan, oracle_place, tiny_layouts
+from helpers import apply_plan_numpy, cast_setup, make_plan, oracle_place, tiny_layouts
 from modelexpress_amd import synth
 
 
 @pytest.mark.parametrize("name", list(tiny_layouts()))
 def test_plan_matches_oracle_for_every_rank(name, mxp, oracle, tmp_path):
     layout, tp, ep, shards, ck_kw = tiny_layouts()[name]
-    cast = ck_kw.get("dtype") == "F32"
+    ck_kw, param_dtype, cast, _ratio = cast_setup(ck_kw)
     synth.write_checkpoint(layout.checkpoint(**ck_kw), str(tmp_path), n_shards=shards, seed=3)
     for tp_rank in range(tp):
         for ep_rank in range(ep):
             if ep > 1 and ep_rank != tp_rank % ep:
                 continue
-            rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=ep_rank,
-                                  param_dtype="BF16" if cast else None)
+            rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=ep_rank, param_dtype=param_dtype)
             want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
             ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
             got = apply_plan_numpy(ck, plan)

@@ -266,4 +266,24 @@ def test_dtype_mismatch_needs_the_cast_flag(mxp, tmp_path):
         PlacementPlan(Checkpoint(str(tmp_path)), [ParamSpec("w.weight", "BF16", (4, 4))])
     assert e.value.code == ERR_UNSUPPORTED
     plan = PlacementPlan(Checkpoint(str(tmp_path)), [ParamSpec("w.weight", "BF16", (4, 4))], allow_cast=True)
-    assert plan.writes()[0].cast and plan.writes()[0].row_bytes == 32
+    assert plan.writes()[0].cast == 1 and plan.writes()[0].row_bytes == 32
+
+
+def test_widening_and_half_conversions_are_planned(mxp, oracle, tmp_path):
+    # receiver.py:962-969 converts the served bf16 staging into an fp32 receive buffer
+    w = torch.arange(32, dtype=torch.float32).reshape(4, 8)
+    save_file({"a.weight": w.to(torch.bfloat16), "b.weight": w.to(torch.float16), "c.weight": w},
+              str(tmp_path / "model.safetensors"))
+    ck = Checkpoint(str(tmp_path))
+    specs = [ParamSpec("a.weight", "F32", (4, 4)), ParamSpec("b.weight", "F32", (4, 4)), ParamSpec("c.weight", "F16", (4, 4))]
+    with pytest.raises(MxpError, match="no conversion"):
+        PlacementPlan(ck, specs, tp_size=2, tp_rank=1)
+    plan = PlacementPlan(ck, specs, tp_size=2, tp_rank=1, allow_cast=True)
+    by = {x.tensor: x for x in plan.writes()}
+    # column slice [:, 4:8]: 4 rows; destination rows are 16 B (fp32) from 8 B of bf16 / fp16, 8 B (fp16) from 16 B of fp32
+    a, b, c = by["a.weight"], by["b.weight"], by["c.weight"]
+    assert (a.cast, a.rows, a.row_bytes, a.src_offset, a.src_pitch, a.dst_pitch) == (2, 4, 16, 8, 16, 16)
+    assert (b.cast, b.rows, b.row_bytes, b.src_offset, b.src_pitch, b.dst_pitch) == (3, 4, 16, 8, 16, 16)
+    assert (c.cast, c.rows, c.row_bytes, c.src_offset, c.src_pitch, c.dst_pitch) == (4, 4, 8, 16, 32, 8)
+    with pytest.raises(MxpError, match="no conversion"):  # pairs outside the table stay refused
+        PlacementPlan(ck, [ParamSpec("a.weight", "F16", (4, 8))], allow_cast=True, allow_uncovered=True, allow_unmapped=True)
