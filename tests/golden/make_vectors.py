@@ -6,7 +6,9 @@ digest and the cast, produced WITHOUT the oracle (oracle/) and without the produ
 * tensor_digest   a big-integer loop written from refit/reshard/verify.py:112-155 and
                   hashlib.blake2b, the library the reference calls;
 * cast            torch's CPU float32 -> bfloat16 conversion (non-NaN inputs only: the NaN
-                  image depends on the host's instruction set).
+                  image depends on the host's instruction set), and its float32 -> float16,
+                  bfloat16 -> float32 and float16 -> float32 conversions (the widening ones on
+                  every 64th 16-bit pattern plus the special ones).
 
 Inputs come from a fixed linear congruential generator so the file is reproducible with
 nothing but the standard library and torch.  Run: python tests/golden/make_vectors.py
@@ -76,6 +78,20 @@ def main():
     t = torch.tensor([b - (1 << 32) if b >= (1 << 31) else b for b in bits], dtype=torch.int32).view(torch.float32)
     out = t.to(torch.bfloat16).view(torch.int16).tolist()
     vec["cast"] = {"f32_bits": bits, "bf16_bits": [v & 0xFFFF for v in out]}
+    extra16 = [0x33000000, 0x33000001, 0x337FFFFF, 0x33800000, 0x387FC000, 0x387FE000, 0x38800000, 0x477FE000,
+               0x477FEFFF, 0x477FF000, 0x47800000, 0xC77FF000, 0x3F801000, 0x3F803000, 0x3F801001]
+    bits16 = [b for b in bits + extra16 if (b & 0x7FFFFFFF) <= 0x7F800000]
+    t = torch.tensor([b - (1 << 32) if b >= (1 << 31) else b for b in bits16], dtype=torch.int32).view(torch.float32)
+    vec["cast_f32_f16"] = {"f32_bits": bits16, "f16_bits": [v & 0xFFFF for v in t.to(torch.float16).view(torch.int16).tolist()]}
+    halves = sorted(set(list(range(0, 1 << 16, 64)) + [0x0001, 0x03FF, 0x0400, 0x7BFF, 0x7C00, 0xFC00, 0x8001, 0x83FF,
+                                                       0x3C00, 0x3F80, 0x7F80, 0xFF80, 0x7F7F, 0x0080, 0x007F]))
+    h = torch.tensor([v - (1 << 16) if v >= (1 << 15) else v for v in halves], dtype=torch.int16)
+    not_nan16 = [i for i, v in enumerate(halves) if (v & 0x7FFF) <= 0x7C00]
+    not_nan_bf = [i for i, v in enumerate(halves) if (v & 0x7FFF) <= 0x7F80]
+    f = h.view(torch.float16).to(torch.float32).view(torch.int32).tolist()
+    g = h.view(torch.bfloat16).to(torch.float32).view(torch.int32).tolist()
+    vec["cast_f16_f32"] = {"f16_bits": [halves[i] for i in not_nan16], "f32_bits": [f[i] & M32 for i in not_nan16]}
+    vec["cast_bf16_f32"] = {"bf16_bits": [halves[i] for i in not_nan_bf], "f32_bits": [g[i] & M32 for i in not_nan_bf]}
     Path(__file__).with_name("vectors.json").write_text(json.dumps(vec, indent=0, separators=(",", ":")))
     print("wrote", Path(__file__).with_name("vectors.json"))
 
