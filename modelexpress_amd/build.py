@@ -85,6 +85,27 @@ def build_library(force: bool = True, jobs: int = 4) -> Path:
     return LIB_PATH
 
 
+ABI_DRIVER_SRC = PKG_DIR.parent / "tests" / "c" / "abi_driver.c"
+ABI_DRIVER = ABI_DRIVER_SRC.with_suffix("")
+
+
+def build_abi_driver() -> Path:
+    """Compile the plain-C caller of the library (tests/c/abi_driver.c) with gcc: it includes
+    only include/mxp.h and the HIP runtime API header, and links libmxplace.so and libamdhip64."""
+    rocm = Path(os.environ.get("ROCM_PATH", "/opt/rocm"))
+    cmd = ["gcc", "-std=c11", "-O1", "-Wall", "-Wextra", "-D__HIP_PLATFORM_AMD__", f"-I{INCLUDE}", f"-I{rocm / 'include'}",
+           str(ABI_DRIVER_SRC), "-o", str(ABI_DRIVER), f"-L{PKG_DIR}", "-lmxplace", f"-L{rocm / 'lib'}", "-lamdhip64",
+           "-Wl,-rpath,$ORIGIN/../../modelexpress_amd", f"-Wl,-rpath,{rocm / 'lib'}"]
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"gcc failed on {ABI_DRIVER_SRC.name}:\n{proc.stderr}")
+    if proc.stderr.strip():
+        sys.stderr.write(proc.stderr)
+    return ABI_DRIVER
+
+
 if __name__ == "__main__":
     path = build_library(force="--incremental" not in sys.argv)
     print(path)
+    if "--abi-driver" in sys.argv:
+        print(build_abi_driver())
