@@ -79,6 +79,7 @@ struct mxp_plan::Lowered {
   uint64_t slot_bytes = 0;
   uint32_t tile_bytes = 0;
   bool host_pack = false;
+  int reader_threads = 0;  // the chunk-size ramp depends on it
   bool direct_io = false;
   // resident tables: source buffer index = shard file index
   DevBuf<Seg> res_segs;
@@ -137,7 +138,8 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   if (!pl.built) throw Error(MXP_ERR_STATE, "plan has not been built");
   const bool host_pack = eng.opt.pack_strided_on_host == 1;
   if (pl.lowered && pl.lowered->slot_bytes == eng.opt.slot_bytes && pl.lowered->tile_bytes == eng.opt.tile_bytes &&
-      pl.lowered->host_pack == host_pack && pl.lowered->direct_io == (eng.opt.use_o_direct != 0))
+      pl.lowered->host_pack == host_pack && pl.lowered->direct_io == (eng.opt.use_o_direct != 0) &&
+      pl.lowered->reader_threads == eng.opt.reader_threads)
     return;
   if (pl.lowered) { free_lowered(pl.lowered); pl.lowered = nullptr; }
   auto L = std::make_unique<mxp_plan::Lowered>();
@@ -145,6 +147,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   L->tile_bytes = eng.opt.tile_bytes;
   L->host_pack = host_pack;
   L->direct_io = eng.opt.use_o_direct != 0;
+  L->reader_threads = eng.opt.reader_threads;
   // Direct I/O reads whole 4 KiB blocks at 4 KiB offsets into 4 KiB aligned memory: every
   // range is widened to block boundaries and the box starts that many bytes into the slot.
   const uint64_t blk = L->direct_io ? 4096 : 1;
@@ -262,33 +265,77 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       L->chunks.push_back(cur);
       cur = Chunk();
     };
-    for (auto& p : pieces) {
-      uint64_t at = align_up(cur.used_bytes, L->direct_io ? blk : 256);
-      uint64_t lead = 0, need = 0;
-      if (L->direct_io) {
-        const uint64_t a0 = p.file_off / blk * blk, a1 = align_up(p.file_off + p.nbytes, blk);
-        lead = p.file_off - a0;
-        need = lead + p.nbytes;
-        p.file_off = a0;
-        p.nbytes = a1 - a0;
+    // Chunk capacity ramps up: every reader thread starts on a small chunk, so the first
+    // host-to-device copy is issued after a 2 MiB read instead of a whole slot's, and the
+    // copies already queued hide the longer reads that follow.
+    const uint64_t threads = (uint64_t)std::max(1, eng.opt.reader_threads);
+    auto capacity = [&](size_t chunk_index) -> uint64_t {
+      if (L->direct_io) return eng.opt.slot_bytes;
+      const uint64_t step = chunk_index / threads;
+      const uint64_t cap = step >= 3 ? eng.opt.slot_bytes : (uint64_t)(2u << 20) << step;
+      return std::min<uint64_t>(eng.opt.slot_bytes, std::max<uint64_t>(cap, 64 * 1024));
+    };
+    for (size_t pi = 0; pi < pieces.size(); ++pi) {
+      Piece p = pieces[pi];
+      for (;;) {
+        const uint64_t cap = capacity(L->chunks.size());
+        uint64_t at = align_up(cur.used_bytes, L->direct_io ? blk : 256);
+        // A contiguous run that does not fit what is left of this chunk is cut at a 4 KiB
+        // multiple of destination bytes; the remainder goes on into the next chunk.
+        Piece rest;
+        bool have_rest = false;
+        if (!L->direct_io && p.rows == 1 && p.box.rows == 1 && at + p.nbytes > cap) {
+          const uint64_t room_src = cap > at ? cap - at : 0;
+          const uint64_t k = op_dst_bytes(p.box.op, room_src) / 4096 * 4096;  // destination bytes that fit
+          if (k == 0 && !cur.ranges.empty()) {
+            close();
+            continue;
+          }
+          if (k > 0 && k < p.box.row_bytes) {
+            rest = p;
+            have_rest = true;
+            const uint64_t ks = op_src_bytes(p.box.op, k);
+            rest.file_off += ks;
+            rest.nbytes -= ks;
+            rest.box.dst_off += k;
+            rest.box.row_bytes -= k;
+            rest.box.src_pitch = rest.nbytes;
+            rest.box.dst_pitch = rest.box.row_bytes;
+            p.nbytes = ks;
+            p.box.row_bytes = k;
+            p.box.src_pitch = ks;
+            p.box.dst_pitch = k;
+          }
+        }
+        uint64_t lead = 0, need = 0;
+        if (L->direct_io) {
+          const uint64_t a0 = p.file_off / blk * blk, a1 = align_up(p.file_off + p.nbytes, blk);
+          lead = p.file_off - a0;
+          need = lead + p.nbytes;
+          p.file_off = a0;
+          p.nbytes = a1 - a0;
+        }
+        const uint64_t in_slot = p.nbytes * p.rows;
+        if (!cur.ranges.empty() && at + in_slot > cap) {
+          close();
+          at = 0;
+        }
+        if (at + in_slot > eng.opt.slot_bytes) throw Error(MXP_ERR_STATE, "internal: a piece does not fit a staging slot");
+        if (cur.ranges.empty()) {
+          cur.seg_begin = (uint32_t)segs.size();
+          cur.work_begin = (uint32_t)work.size();
+        }
+        cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at, p.rows, p.file_pitch, need});
+        cur.used_bytes = at + in_slot;
+        L->file_bytes += in_slot;
+        p.box.src_off = at + lead;
+        const size_t w0 = work.size();
+        lower_box(p.box, lo, segs, work);
+        // work items index segments relative to the chunk's first segment
+        for (size_t k = w0; k < work.size(); ++k) work[k].seg -= cur.seg_begin;
+        if (!have_rest) break;
+        p = rest;
       }
-      const uint64_t in_slot = p.nbytes * p.rows;
-      if (!cur.ranges.empty() && at + in_slot > eng.opt.slot_bytes) {
-        close();
-        at = 0;
-      }
-      if (cur.ranges.empty()) {
-        cur.seg_begin = (uint32_t)segs.size();
-        cur.work_begin = (uint32_t)work.size();
-      }
-      cur.ranges.push_back(FileRange{p.file, p.file_off, p.nbytes, at, p.rows, p.file_pitch, need});
-      cur.used_bytes = at + in_slot;
-      L->file_bytes += in_slot;
-      p.box.src_off = at + lead;
-      const size_t w0 = work.size();
-      lower_box(p.box, lo, segs, work);
-      // work items index segments relative to the chunk's first segment
-      for (size_t k = w0; k < work.size(); ++k) work[k].seg -= cur.seg_begin;
     }
     close();
     L->ing_n_segs = (uint32_t)segs.size();
