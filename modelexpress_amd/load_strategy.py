@@ -38,6 +38,8 @@ logger = logging.getLogger("modelexpress_amd.load_strategy")
 
 T = TypeVar("T")
 
+from .manifest import TensorRecord  # noqa: E402
+
 _TORCH_DTYPE = {
     "F64": torch.float64, "F32": torch.float32, "F16": torch.float16, "BF16": torch.bfloat16,
     "F8_E4M3": torch.float8_e4m3fn, "F8_E5M2": torch.float8_e5m2, "I64": torch.int64, "I32": torch.int32,
@@ -221,6 +223,7 @@ class HipPlacementStrategy(LoadStrategy):
         try:
             result.metadata["placement_stats"] = stats
             result.metadata["checksums"] = sums
+            result.metadata["manifest"] = [TensorRecord(p.name, p.nbytes, p.dtype, sums[p.name]) for p in layout.params]
             log_tensor_summary(sums, f"worker{ctx.global_rank}",
                                {p.name: (tuple(p.shape), p.dtype) for p in layout.params})
             logger.info(f"[Worker {ctx.global_rank}] HIP placement complete: "

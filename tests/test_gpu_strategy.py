@@ -84,6 +84,34 @@ def test_chain_places_into_param_data(oracle, tmp_path, monkeypatch, mxp):
     assert set(ctx.tensors) == set(want)
 
 
+def test_manifest_of_a_placed_rank_matches_a_source_manifest(oracle, tmp_path, monkeypatch, mxp):
+    """Source side: names, sizes, dtypes, checksums and digests computed by the oracle.  Target
+    side: the manifest the strategy leaves in the result plus device digests of the live
+    parameters.  One flipped byte on the target must fail the comparison."""
+    from modelexpress_amd.engine import PlacementEngine
+    from modelexpress_amd.manifest import ManifestMismatchError, TensorRecord, build_manifest, compare_manifests
+
+    synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=2, seed=23)
+    rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
+    want = oracle_place(oracle, str(tmp_path), rv, tp_size=TP, tp_rank=RANK)
+    source = [TensorRecord(p.name, p.nbytes, p.dtype, oracle.safe_checksum(want[p.name]), oracle.tensor_digest(want[p.name]))
+              for p in rv.params]
+    monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
+    model = ToyModel(rv)
+    ad = ToyAdapter(rv)
+    result = HipPlacementStrategy().load(LoadResult(value=model, model=model), _ctx(ad, str(tmp_path)))
+    assert compare_manifests(source, result.metadata["manifest"], require_exact_match=True) == len(rv.params)
+    eng = PlacementEngine(0)
+    live = dict(model.named_parameters())
+    local = build_manifest(eng, rv.params, [live[p.name].data for p in rv.params])
+    assert compare_manifests(source, local, require_exact_match=True) == len(rv.params)
+    victim = rv.params[1]
+    live[victim.name].data.view(torch.uint8).view(-1)[3] ^= 1
+    with pytest.raises(ManifestMismatchError, match=f"'{victim.name}' checksum mismatch"):
+        compare_manifests(source, build_manifest(eng, rv.params, [live[p.name].data for p in rv.params]))
+    eng.close()
+
+
 def test_truncated_shard_fails_the_strategy_and_the_chain_recovers(tmp_path, monkeypatch, mxp):
     """A shard that shrinks between planning and ingest: the read error surfaces as
     StrategyFailed (mutated once any chunk reached the GPU), the chain rolls back,

@@ -207,3 +207,30 @@ def test_refit_timing_vocabulary():
     payload = json.loads(line[len(MX_REFIT_TIMING_PREFIX) + 1:])
     assert payload["cold_warm"] == "cold" and payload["stages"]["wire_transfer"] == {"duration_s": 2.0, "count": 1, "statuses": ["ok"]}
     assert payload["stages"]["installation"]["statuses"] == ["error"]
+
+
+def test_manifest_comparison_rules(caplog):
+    # modelexpress/nixl_transfer.py:835-897: size and dtype must agree per shared name; a name diff
+    # fails closed only when an exact match is required; nothing matched is an error in that mode
+    from modelexpress_amd.manifest import ManifestMismatchError, TensorRecord, compare_manifests, dumps, loads
+
+    a = [TensorRecord("w", 64, "BF16", "0000abcd", "00" * 16), TensorRecord("b", 8, "F32", "00000001")]
+    assert compare_manifests(a, loads(dumps(a)), require_exact_match=True) == 2
+    with pytest.raises(ManifestMismatchError, match="size mismatch: source=64 bytes, local=32 bytes"):
+        compare_manifests(a, [TensorRecord("w", 32, "BF16")])
+    with pytest.raises(ManifestMismatchError, match="dtype mismatch: source='BF16', local='F16'"):
+        compare_manifests(a, [TensorRecord("w", 64, "F16")])
+    with pytest.raises(ManifestMismatchError, match="checksum mismatch"):
+        compare_manifests(a, [TensorRecord("w", 64, "BF16", "0000abce")])
+    with pytest.raises(ManifestMismatchError, match="digest mismatch"):
+        compare_manifests(a, [TensorRecord("w", 64, "BF16", "0000abcd", "11" * 16)])
+    assert compare_manifests(a, [TensorRecord("w", 64, "BF16", "0000abce")], check_content=False) == 1
+    assert compare_manifests(a, [TensorRecord("w", 64, "BF16")]) == 1  # a side without content fields is not compared
+    with caplog.at_level("WARNING", logger="modelexpress_amd.manifest"):
+        assert compare_manifests(a, [TensorRecord("w", 64, "BF16"), TensorRecord("extra", 4, "F32")]) == 1
+    assert "1 local-only, 1 source-only" in caplog.text
+    with pytest.raises(ManifestMismatchError, match="1 local-only .first: .'extra'.., 1 source-only"):
+        compare_manifests(a, [TensorRecord("w", 64, "BF16"), TensorRecord("extra", 4, "F32")], require_exact_match=True)
+    with pytest.raises(ManifestMismatchError, match="No matching tensors"):
+        compare_manifests([], [], require_exact_match=True)
+    assert compare_manifests([], []) == 0
