@@ -112,6 +112,8 @@ struct TransposeDesc {
   uint32_t csum_bias;
   uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides kTransposeWaves)
 };
+// Per-device set-up of the placement kernels (idempotent; also done lazily by launch_place).
+hipError_t configure_place_kernels();
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
                             uint32_t* sum_out, hipStream_t stream);
 

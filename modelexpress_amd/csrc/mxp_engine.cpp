@@ -484,13 +484,15 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     if (o.use_o_direct && o.pack_strided_on_host == 1)
       throw Error(MXP_ERR_ARG, "direct I/O reads whole blocks; it cannot be combined with per-row host packing");
     if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
-    if (o.tile_bytes < 1024 || o.tile_bytes > (1u << 20)) throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 1 MiB]");
+    if (o.tile_bytes < 1024 || o.tile_bytes > (uint32_t)(kPlaceThreads * kPlaceBatch * 16))
+      throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 128 KiB]");
     if (o.ring_slots > 256 || o.reader_threads > 256 || o.streams > 64) throw Error(MXP_ERR_ARG, "ring, thread or stream count too large");
     int n_dev = 0;
     HIP_OK(hipGetDeviceCount(&n_dev));
     if (n_dev <= 0) throw Error(MXP_ERR_DEVICE, "no HIP device is visible");
     if (o.device < 0 || o.device >= n_dev) throw Error(MXP_ERR_ARG, "device ordinal out of range");
     HIP_OK(hipSetDevice(o.device));
+    HIP_OK(configure_place_kernels());
     for (int s = 0; s < o.streams; ++s) {
       hipStream_t st;
       HIP_OK(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));

@@ -12,6 +12,8 @@
 //  digest_kernel  int32-word row sums for the blake2b-hashed tensor digest
 //                 (reads each byte once)
 #include "mxp_device.h"
+#include <atomic>
+#include <type_traits>
 
 namespace mxp {
 
@@ -167,88 +169,72 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
     d_o = row * dp + col * (uint32_t)UNIT;
   };
 
-  if constexpr (NARROW && UNIT == 8) {
-    // Narrowing cast: a unit is four elements, one 16-byte load and one 8-byte store per lane, so a
-    // wavefront load covers 1 KiB of contiguous source and a store 512 B of contiguous
-    // destination.  As in the copy path, eight loads per lane (a 128 KiB read burst per
-    // workgroup) are in flight before the first store; sixteen measured 6% slower.
+  constexpr bool BATCHED = (NARROW && UNIT == 8) || (!NARROW && UNIT == 16);
+  if constexpr (BATCHED) {
+    // The wide paths.  A lane moves kPlaceBatch units: 16 bytes in and out for a copy, 16 in /
+    // 8 out for a narrowing cast, 8 in / 16 out for a widening one, so a wavefront access is
+    // 1 KiB (512 B on the narrow side) of contiguous memory.  A tile is at most one batch (the
+    // host bounds it): a single pass in four phases that the scheduler may not interleave -
+    // all addresses, all loads, all stores, then the checksum arithmetic - so the workgroup
+    // presents the memory system with one burst of reads over a contiguous region followed by
+    // one burst of writes over another.  Measured on the Llama rank: 256 lanes x 4 loads
+    // 5.16 TB/s, 1024 x 8 5.98 TB/s; sixteen loads per lane are slower.
     constexpr int U = kPlaceBatch;
-    for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += (uint32_t)U * kPlaceThreads) {
-      uint32_t d_o[U];
-      uint4 a[U];
+    using In = typename std::conditional<WIDEN, uint2, uint4>::type;
+    using Out = typename std::conditional<NARROW, uint2, uint4>::type;
+    auto load = [&](uint32_t off) -> In {
+      if constexpr (WIDEN) return ld8(src + off);
+      else return ld16(src + off);
+    };
+    auto convert = [&](const In& a) -> Out {
+      if constexpr (NARROW) return narrow4<OP>(a, nan_bits);
+      else if constexpr (WIDEN) return widen4<OP>(a);
+      else return a;
+    };
+    auto store = [&](uint32_t off, const Out& x) {
+      if constexpr (OP == kOpChecksumOnly) return;
+      else if constexpr (NARROW) st8(dst + off, x);
+      else st16(dst + off, x);
+    };
+    auto sum = [&](uint32_t off, const Out& x) {
+      if constexpr (NARROW) cs.add8(x.x, x.y, csum_base + off);
+      else cs.add16(x, csum_base + off);
+    };
+    uint32_t so[U], d_o[U];
+    In a[U];
+    if (n_units == (uint32_t)U * kPlaceThreads) {  // full tile: nothing is predicated
+#pragma unroll
+      for (int k = 0; k < U; ++k) locate(threadIdx.x + (uint32_t)k * kPlaceThreads, so[k], d_o[k]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int k = 0; k < U; ++k) a[k] = load(so[k]);
+      __builtin_amdgcn_sched_barrier(0);
+      Out x[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        x[k] = convert(a[k]);
+        store(d_o[k], x[k]);
+      }
+      if constexpr (OP != kOpChecksumOnly) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int k = 0; k < U; ++k) sum(d_o[k], x[k]);
+    } else {
       bool ok[U];
 #pragma unroll
       for (int k = 0; k < U; ++k) {
-        const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
+        const uint32_t v = threadIdx.x + (uint32_t)k * kPlaceThreads;
         ok[k] = v < n_units;
-        if (ok[k]) {
-          uint32_t so;
-          locate(v, so, d_o[k]);
-          a[k] = ld16(src + so);
-        }
+        locate(ok[k] ? v : 0u, so[k], d_o[k]);
       }
+#pragma unroll
+      for (int k = 0; k < U; ++k)
+        if (ok[k]) a[k] = load(so[k]);
 #pragma unroll
       for (int k = 0; k < U; ++k) {
         if (ok[k]) {
-          const uint2 x = narrow4<OP>(a[k], nan_bits);
-          st8(dst + d_o[k], x);
-          cs.add8(x.x, x.y, csum_base + d_o[k]);
-        }
-      }
-    }
-  } else if constexpr (WIDEN && UNIT == 16) {
-    // Widening cast: a unit is four elements, one 8-byte load and one 16-byte store per lane
-    // (a wavefront load covers 512 B of contiguous source, a store 1 KiB of destination).
-    constexpr int U = kPlaceBatch;
-    for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += (uint32_t)U * kPlaceThreads) {
-      uint32_t d_o[U];
-      uint2 a[U];
-      bool ok[U];
-#pragma unroll
-      for (int k = 0; k < U; ++k) {
-        const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
-        ok[k] = v < n_units;
-        if (ok[k]) {
-          uint32_t so;
-          locate(v, so, d_o[k]);
-          a[k] = ld8(src + so);
-        }
-      }
-#pragma unroll
-      for (int k = 0; k < U; ++k) {
-        if (ok[k]) {
-          const uint4 x = widen4<OP>(a[k]);
-          st16(dst + d_o[k], x);
-          cs.add16(x, csum_base + d_o[k]);
-        }
-      }
-    }
-  } else if constexpr (UNIT == 16) {
-    // One batch = kPlaceBatch units per lane: every load of the batch is issued before its
-    // first store, so a workgroup presents the memory system with a burst of reads over
-    // one contiguous region followed by a burst of writes over another.  With the default
-    // tile (kPlaceThreads * kPlaceBatch * 16 B = 128 KiB) a workgroup runs exactly one
-    // batch; that shape measured fastest (5.98 TB/s against 5.16 TB/s for 256 lanes x 4).
-    constexpr int U = kPlaceBatch;
-    for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += (uint32_t)U * kPlaceThreads) {
-      uint32_t d_o[U];
-      uint4 x[U];
-      bool ok[U];
-#pragma unroll
-      for (int k = 0; k < U; ++k) {
-        const uint32_t v = v0 + (uint32_t)k * kPlaceThreads;
-        ok[k] = v < n_units;
-        if (ok[k]) {
-          uint32_t so;
-          locate(v, so, d_o[k]);
-          x[k] = ld16(src + so);
-        }
-      }
-#pragma unroll
-      for (int k = 0; k < U; ++k) {
-        if (ok[k]) {
-          if constexpr (OP != kOpChecksumOnly) st16(dst + d_o[k], x[k]);
-          cs.add16(x[k], csum_base + d_o[k]);
+          const Out x = convert(a[k]);
+          store(d_o[k], x);
+          sum(d_o[k], x);
         }
       }
     }
@@ -351,16 +337,39 @@ __global__ __launch_bounds__(kPlaceThreads) void checksum_kernel(
   place_body<true>(segs, work, src_bases, nullptr, sums, 0u);
 }
 
+// One workgroup per compute unit: a unit then alternates between one 128 KiB read burst and
+// one 128 KiB write burst instead of mixing the two.  Two resident workgroups measured 4-10%
+// slower on every configuration.  The limit is imposed with an otherwise unused dynamic LDS
+// allocation of more than half a unit's LDS, which needs the attribute below once per device.
+constexpr uint32_t kOnePerCu = 96 * 1024;
+
+hipError_t configure_place_kernels() {
+  static std::atomic<uint64_t> configured{0};  // bit per device
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (configured.load(std::memory_order_acquire) & bit) return hipSuccess;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(place_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)kOnePerCu);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(checksum_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kOnePerCu);
+  if (e == hipSuccess) configured.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
                         uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only) {
   if (n_work == 0) return hipSuccess;
+  if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
+  const uint32_t lds_place = kOnePerCu, lds_csum = kOnePerCu;
   if (checksum_only) {
-    hipLaunchKernelGGL(checksum_kernel, dim3(n_work), dim3(kPlaceThreads), 0, stream, segs_dev, work_dev,
+    hipLaunchKernelGGL(checksum_kernel, dim3(n_work), dim3(kPlaceThreads), lds_csum, stream, segs_dev, work_dev,
                        src_bases_dev, sums_dev);
     return hipGetLastError();
   }
-  hipLaunchKernelGGL(place_kernel, dim3(n_work), dim3(kPlaceThreads), 0, stream, segs_dev,
+  hipLaunchKernelGGL(place_kernel, dim3(n_work), dim3(kPlaceThreads), lds_place, stream, segs_dev,
                      work_dev, src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits);
   return hipGetLastError();
 }

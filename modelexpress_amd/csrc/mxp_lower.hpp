@@ -82,6 +82,9 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
     rpt = (rpt + 1) / 2;
   if ((uint64_t)s.units_per_row * s.units_per_row >= (1ull << 32))
     throw std::logic_error("emit_seg: row too wide for its unit");
+  // The 16-byte (8-byte for narrowing casts) paths of place_kernel run one batch per tile.
+  if ((unit == 16 || unit == 8) && rpt * s.units_per_row > (uint64_t)kPlaceThreads * kPlaceBatch)
+    throw std::logic_error("emit_seg: tile larger than one batch");
   s.rows_per_tile = (uint32_t)rpt;
   const uint32_t seg_idx = (uint32_t)segs.size();
   segs.push_back(s);
