@@ -338,6 +338,19 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* boxes, int64_t n, uint32_
 int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
                      const int64_t* src_strides, const int32_t* perm, int32_t elem_size, uint32_t* checksum,
                      void* stream);
+/* dst_view[...] = src_view[...] for two strided views of one `shape` (ndim <= 8, strides in
+ * elements, NULL = contiguous row-major): the device form of one RecordedCopy
+ * (refit/reshard/types.py:57-71) once its op-chain has been replayed to a strided source view
+ * (refit/reshard/slice_plan.py:136-164) - destination.as_strided(shape, dst_strides).copy_(
+ * source.as_strided(shape, src_strides)).  Rows contiguous on both sides run as pitched boxes,
+ * a transposed innermost dimension through the LDS transpose, anything else element by
+ * element (the run length paired_runs would find).  A destination view that overlaps itself
+ * is refused.  `cast` is an MXP_CAST_* code (then `elem_size` is the destination element's and the
+ * transpose route is not taken).  *checksum, when not NULL, receives the position-weighted checksum of the
+ * written bytes, positions counted from `dst`. */
+int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
+                  const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_size,
+                  int32_t cast, uint32_t* checksum, void* stream);
 /* n independent contiguous device copies in one launch, with the checksum of each
  * destination in out_checksums[k] when not NULL: the device form of the batched
  * torch._foreach_copy_ install (refit/reshard/receiver.py:939-955).  Destinations must

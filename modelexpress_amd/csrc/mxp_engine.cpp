@@ -897,153 +897,217 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n
   });
 }
 
+extern "C++" {
+namespace {
+
+// dst_view[...] = src_view[...] for two strided views of one shape (strides in elements).
+// Dimensions are put in destination order (largest destination stride first) and merged
+// where both sides allow; then
+//   * innermost dimension contiguous on both sides  -> pitched row boxes through place_kernel,
+//   * contiguous in the destination only, with another dimension contiguous in the source
+//                                                   -> transpose_kernel (other dims = batch),
+//   * anything else                                 -> one element per box row (the run length
+//     the reference's paired_runs finds for such a view: slice_plan.py:259-294).
+// The checksum, when asked for, weights every written byte by its offset from `dst`.
+void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
+               std::vector<uint64_t> ds, int elem_size, int cast, uint32_t* checksum, hipStream_t stream,
+               const char* what) {
+  const uint32_t op = seg_op_of_cast(cast);
+  const uint64_t es = (uint64_t)elem_size;          // destination element
+  const uint64_t es_s = op_src_bytes(op, es);       // source element
+  auto fail = [&](int code, const std::string& msg) { throw Error(code, std::string(what) + ": " + msg); };
+  uint64_t total = 1;
+  for (auto n : size) total *= n;
+  if (checksum) *checksum = 0;
+  if (total == 0) return;
+  if (!src || !dst) fail(MXP_ERR_ARG, "null pointer");
+  if (reinterpret_cast<uintptr_t>(src) % es_s || reinterpret_cast<uintptr_t>(dst) % es) fail(MXP_ERR_ARG, "pointer is not element aligned");
+  HIP_OK(hipSetDevice(e.opt.device));
+  {
+    // drop unit dims, order by destination stride, refuse a self-overlapping destination, merge
+    std::vector<size_t> order;
+    for (size_t d = 0; d < size.size(); ++d)
+      if (size[d] != 1) order.push_back(d);
+    std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) { return ds[x] > ds[y]; });
+    std::vector<uint64_t> n2, s2, d2;
+    for (size_t d : order) { n2.push_back(size[d]); s2.push_back(ss[d]); d2.push_back(ds[d]); }
+    for (size_t d = 0; d + 1 < n2.size(); ++d)
+      if (d2[d] < d2[d + 1] * n2[d + 1]) fail(MXP_ERR_UNSUPPORTED, "the destination view overlaps itself");
+    if (!n2.empty() && d2.back() == 0) fail(MXP_ERR_UNSUPPORTED, "the destination view overlaps itself");
+    size.clear(); ss.clear(); ds.clear();
+    for (size_t d = 0; d < n2.size(); ++d) {
+      if (!size.empty() && ss.back() == s2[d] * n2[d] && ds.back() == d2[d] * n2[d]) {
+        size.back() *= n2[d];
+        ss.back() = s2[d];
+        ds.back() = d2[d];
+      } else {
+        size.push_back(n2[d]); ss.push_back(s2[d]); ds.push_back(d2[d]);
+      }
+    }
+    if (size.empty()) { size.push_back(1); ss.push_back(1); ds.push_back(1); }
+  }
+  const size_t nd = size.size();
+  int c = -1;  // a dimension other than the innermost that is contiguous in the source
+  for (size_t d = 0; d + 1 < nd; ++d)
+    if (ss[d] == 1) c = (int)d;
+  const bool dst_inner = ds[nd - 1] == 1 || total == 1;
+  const bool transpose = op == kOpCopy && dst_inner && ss[nd - 1] != 1 && total != 1 && c >= 0 && nd - 2 <= (size_t)kMaxBatchDims;
+
+  if (!transpose) {
+    // Row boxes: whole innermost rows when both sides are contiguous there, else one element per row.
+    const bool rows_ok = dst_inner && (ss[nd - 1] == 1 || total == 1);
+    std::vector<uint64_t> n = size, s = ss, d = ds;
+    if (!rows_ok) { n.push_back(1); s.push_back(1); d.push_back(1); }  // a virtual innermost dimension of one element
+    const size_t m = n.size();
+    const void* sb;
+    const void* db;
+    uint64_t so, d_o;
+    split_ptr(src, sb, so);
+    split_ptr(dst, db, d_o);
+    std::vector<BoxCopy> boxes;
+    BoxCopy b;
+    b.row_bytes = n[m - 1] * es;
+    b.op = op;
+    b.csum_slot = checksum ? 0u : 0xFFFFFFFFu;
+    b.csum_bias = (uint64_t)0 - d_o;
+    if (m == 1) {
+      b.src_off = so;
+      b.dst_off = d_o;
+      boxes.push_back(b);
+    } else {
+      b.rows = n[m - 2];
+      b.src_pitch = s[m - 2] * es_s;
+      b.dst_pitch = d[m - 2] * es;
+      uint64_t outer = 1;
+      for (size_t q = 0; q + 2 < m; ++q) outer *= n[q];
+      if (outer > (1u << 20)) fail(MXP_ERR_UNSUPPORTED, "too many row bands");
+      std::vector<uint64_t> idx(m, 0);
+      for (uint64_t o = 0; o < outer; ++o) {
+        uint64_t s_el = 0, d_el = 0;
+        for (size_t q = 0; q + 2 < m; ++q) { s_el += idx[q] * s[q]; d_el += idx[q] * d[q]; }
+        BoxCopy x = b;
+        x.src_off = so + s_el * es_s;
+        x.dst_off = d_o + d_el * es;
+        boxes.push_back(x);
+        for (int q = (int)m - 3; q >= 0; --q) { if (++idx[q] < n[q]) break; idx[q] = 0; }
+      }
+    }
+    uint32_t sum = 0;
+    run_boxes(e, boxes, {sb}, {const_cast<void*>(db)}, 1, checksum ? &sum : nullptr, stream);
+    if (checksum) *checksum = sum;
+    return;
+  }
+
+  // True transpose: i = destination innermost, j = the source's unit-stride dimension.
+  TransposeDesc td{};
+  td.ni = size[nd - 1];
+  td.si = ss[nd - 1];
+  td.nj = size[c];
+  td.dj = ds[c];
+  // Workgroup shape: as many wavefronts along i (long destination runs) as the extent can
+  // use, the rest along j.
+  uint32_t waves_i = 1;
+  while (waves_i < (uint32_t)kTransposeWaves && (uint64_t)waves_i * transpose_sub_rows(elem_size) < td.ni) waves_i *= 2;
+  td.waves_i = waves_i;
+  const uint64_t tile_i = (uint64_t)waves_i * transpose_sub_rows(elem_size);
+  const uint64_t tile_j = (uint64_t)(kTransposeWaves / waves_i) * transpose_sub_cols(elem_size);
+  td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
+  td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
+  bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * es) % 16 == 0;
+  bool vd = (reinterpret_cast<uintptr_t>(dst) % 16 == 0) && (td.dj * es) % 16 == 0;
+  int k = kMaxBatchDims - 1;
+  for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
+  for (int d = (int)nd - 2; d >= 0; --d) {
+    if (d == c) continue;
+    td.batch_size[k] = size[d];
+    td.batch_sstride[k] = ss[d];
+    td.batch_dstride[k] = ds[d];
+    vs = vs && (ss[d] * es) % 16 == 0;
+    vd = vd && (ds[d] * es) % 16 == 0;
+    --k;
+  }
+  td.vec_src = vs;
+  td.vec_dst = vd;
+  td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
+  for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
+  uint32_t* sum_dev = nullptr;
+  if (checksum) {
+    acquire_arena(e);
+    ensure_desc(e, 256);
+    sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
+    HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
+  }
+  HIP_OK(launch_transpose(src, dst, td, elem_size, sum_dev, stream));
+  if (checksum) {
+    HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::memcpy(checksum, e.desc_host, 4);
+    release_arena(e, stream);
+  }
+}
+
+std::vector<uint64_t> strides_or_row_major(const int64_t* strides, const int64_t* shape, int32_t ndim, const char* what) {
+  std::vector<uint64_t> out((size_t)ndim, 1);
+  if (!strides) {
+    for (int d = ndim - 2; d >= 0; --d) out[d] = out[d + 1] * (uint64_t)shape[d + 1];
+    return out;
+  }
+  for (int d = 0; d < ndim; ++d) {
+    if (strides[d] < 0) throw Error(MXP_ERR_UNSUPPORTED, std::string(what) + ": negative strides are not supported");
+    out[d] = (uint64_t)strides[d];
+  }
+  return out;
+}
+
+void check_view_args(const mxp_engine* engine, int32_t ndim, const int64_t* shape, int32_t elem_size, const char* what) {
+  if (!engine || ndim < 0 || ndim > MXP_MAX_DIMS || (ndim && !shape)) throw Error(MXP_ERR_ARG, std::string(what) + ": bad argument");
+  if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8)
+    throw Error(MXP_ERR_ARG, std::string(what) + ": elem_size must be 1, 2, 4 or 8");
+  for (int d = 0; d < ndim; ++d)
+    if (shape[d] < 0) throw Error(MXP_ERR_ARG, std::string(what) + ": negative extent");
+}
+
+}  // namespace
+}  // extern "C++"
+
 int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
                      const int64_t* src_strides, const int32_t* perm, int32_t elem_size, uint32_t* checksum,
                      void* stream_v) {
   return guard([&] {
-    if (!engine || ndim < 0 || ndim > MXP_MAX_DIMS || (ndim && (!shape || !perm)))
-      throw Error(MXP_ERR_ARG, "mxp_permute_copy: bad argument");
-    if (elem_size != 1 && elem_size != 2 && elem_size != 4 && elem_size != 8)
-      throw Error(MXP_ERR_ARG, "mxp_permute_copy: elem_size must be 1, 2, 4 or 8");
-    if (checksum) *checksum = 0;
-    mxp_engine& e = *engine;
-    hipStream_t stream = static_cast<hipStream_t>(stream_v);
-    const uint64_t es = (uint64_t)elem_size;
-    // Dimensions in destination order.
+    const char* what = "mxp_permute_copy";
+    check_view_args(engine, ndim, shape, elem_size, what);
+    if (ndim && !perm) throw Error(MXP_ERR_ARG, "mxp_permute_copy: bad argument");
+    if (dst && (reinterpret_cast<uintptr_t>(dst) & 15u)) throw Error(MXP_ERR_ARG, "mxp_permute_copy: dst must be 16-byte aligned");
+    const std::vector<uint64_t> st = strides_or_row_major(src_strides, shape, ndim, what);
+    // Dimensions in destination order; the destination is contiguous.
     std::vector<uint64_t> size, ss;
-    {
-      std::vector<int64_t> rm((size_t)ndim, 1);
-      for (int d = ndim - 2; d >= 0; --d) rm[d] = rm[d + 1] * shape[d + 1];
-      std::vector<bool> seen((size_t)ndim, false);
-      for (int d = 0; d < ndim; ++d) {
-        if (perm[d] < 0 || perm[d] >= ndim || seen[perm[d]]) throw Error(MXP_ERR_ARG, "mxp_permute_copy: perm is not a permutation");
-        seen[perm[d]] = true;
-        if (shape[perm[d]] < 0) throw Error(MXP_ERR_ARG, "mxp_permute_copy: negative extent");
-        const int64_t st = src_strides ? src_strides[perm[d]] : rm[perm[d]];
-        if (st < 0) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: negative strides are not supported");
-        size.push_back((uint64_t)shape[perm[d]]);
-        ss.push_back((uint64_t)st);
-      }
+    std::vector<bool> seen((size_t)ndim, false);
+    for (int d = 0; d < ndim; ++d) {
+      if (perm[d] < 0 || perm[d] >= ndim || seen[perm[d]]) throw Error(MXP_ERR_ARG, "mxp_permute_copy: perm is not a permutation");
+      seen[perm[d]] = true;
+      size.push_back((uint64_t)shape[perm[d]]);
+      ss.push_back(st[perm[d]]);
     }
-    uint64_t total = 1;
-    for (auto n : size) total *= n;
-    if (total == 0) return;
-    if (!src || !dst) throw Error(MXP_ERR_ARG, "mxp_permute_copy: null pointer");
-    if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_permute_copy: dst must be 16-byte aligned");
-    if (reinterpret_cast<uintptr_t>(src) % es) throw Error(MXP_ERR_ARG, "mxp_permute_copy: src is not element aligned");
-    HIP_OK(hipSetDevice(e.opt.device));
-    // Drop unit dims; merge neighbours that are contiguous in the source too (the
-    // destination is contiguous, so it always merges).
-    {
-      std::vector<uint64_t> n2, s2;
-      for (size_t d = 0; d < size.size(); ++d)
-        if (size[d] != 1) { n2.push_back(size[d]); s2.push_back(ss[d]); }
-      size.clear();
-      ss.clear();
-      for (size_t d = 0; d < n2.size(); ++d) {
-        if (!size.empty() && ss.back() == s2[d] * n2[d]) {
-          size.back() *= n2[d];
-          ss.back() = s2[d];
-        } else {
-          size.push_back(n2[d]);
-          ss.push_back(s2[d]);
-        }
-      }
-      if (size.empty()) { size.push_back(1); ss.push_back(1); }
-    }
-    const size_t nd = size.size();
-    std::vector<uint64_t> ds(nd, 1);
-    for (int d = (int)nd - 2; d >= 0; --d) ds[d] = ds[d + 1] * size[d + 1];
+    std::vector<uint64_t> ds(size.size(), 1);
+    for (int d = (int)size.size() - 2; d >= 0; --d) ds[d] = ds[d + 1] * size[d + 1];
+    copy_view(*engine, src, dst, size, ss, ds, elem_size, MXP_CAST_NONE, checksum, static_cast<hipStream_t>(stream_v), what);
+  });
+}
 
-    if (ss[nd - 1] == 1 || total == 1) {
-      // The innermost dimension is kept: rows of size[last] elements, gathered.
-      const uint64_t row_bytes = size[nd - 1] * es;
-      const void* sb;
-      uint64_t so;
-      split_ptr(src, sb, so);
-      std::vector<BoxCopy> boxes;
-      BoxCopy b;
-      b.row_bytes = row_bytes;
-      b.op = kOpCopy;
-      b.csum_slot = checksum ? 0u : 0xFFFFFFFFu;
-      if (nd == 1) {
-        b.src_off = so;
-        boxes.push_back(b);
-      } else {
-        b.rows = size[nd - 2];
-        b.src_pitch = ss[nd - 2] * es;
-        b.dst_pitch = row_bytes;
-        uint64_t outer = 1;
-        for (size_t d = 0; d + 2 < nd; ++d) outer *= size[d];
-        if (outer > (1u << 20)) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: too many row bands");
-        std::vector<uint64_t> idx(nd, 0);
-        for (uint64_t o = 0; o < outer; ++o) {
-          uint64_t s_el = 0, d_el = 0;
-          for (size_t d = 0; d + 2 < nd; ++d) { s_el += idx[d] * ss[d]; d_el += idx[d] * ds[d]; }
-          BoxCopy x = b;
-          x.src_off = so + s_el * es;
-          x.dst_off = d_el * es;
-          boxes.push_back(x);
-          for (int d = (int)nd - 3; d >= 0; --d) { if (++idx[d] < size[d]) break; idx[d] = 0; }
-        }
-      }
-      uint32_t sum = 0;
-      run_boxes(e, boxes, {sb}, {dst}, 1, checksum ? &sum : nullptr, stream);
-      if (checksum) *checksum = sum;
-      return;
-    }
-
-    // True transpose: i = destination innermost, j = the source's unit-stride dimension.
-    int c = -1;
-    for (size_t d = 0; d + 1 < nd; ++d)
-      if (ss[d] == 1) c = (int)d;
-    if (c < 0) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: the source has no unit-stride dimension");
-    if (nd - 2 > (size_t)kMaxBatchDims) throw Error(MXP_ERR_UNSUPPORTED, "mxp_permute_copy: too many batch dimensions");
-    TransposeDesc td{};
-    td.ni = size[nd - 1];
-    td.si = ss[nd - 1];
-    td.nj = size[c];
-    td.dj = ds[c];
-    // Workgroup shape: as many wavefronts along i (long destination runs) as the extent can
-    // use, the rest along j.
-    uint32_t waves_i = 1;
-    while (waves_i < (uint32_t)kTransposeWaves && (uint64_t)waves_i * transpose_sub_rows(elem_size) < td.ni) waves_i *= 2;
-    td.waves_i = waves_i;
-    const uint64_t tile_i = (uint64_t)waves_i * transpose_sub_rows(elem_size);
-    const uint64_t tile_j = (uint64_t)(kTransposeWaves / waves_i) * transpose_sub_cols(elem_size);
-    td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
-    td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
-    bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * es) % 16 == 0;
-    bool vd = (td.dj * es) % 16 == 0;
-    int k = kMaxBatchDims - 1;
-    for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
-    for (int d = (int)nd - 2; d >= 0; --d) {
-      if (d == c) continue;
-      td.batch_size[k] = size[d];
-      td.batch_sstride[k] = ss[d];
-      td.batch_dstride[k] = ds[d];
-      vs = vs && (ss[d] * es) % 16 == 0;
-      vd = vd && (ds[d] * es) % 16 == 0;
-      --k;
-    }
-    td.vec_src = vs;
-    td.vec_dst = vd;
-    td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
-    for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
-    uint32_t* sum_dev = nullptr;
-    if (checksum) {
-      acquire_arena(e);
-      ensure_desc(e, 256);
-      sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
-      HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
-    }
-    HIP_OK(launch_transpose(src, dst, td, elem_size, sum_dev, stream));
-    if (checksum) {
-      HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
-      HIP_OK(hipStreamSynchronize(stream));
-      std::memcpy(checksum, e.desc_host, 4);
-      release_arena(e, stream);
-    }
+int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
+                  const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_size, int32_t cast,
+                  uint32_t* checksum, void* stream_v) {
+  return guard([&] {
+    const char* what = "mxp_copy_view";
+    check_view_args(engine, ndim, shape, elem_size, what);
+    if (cast < MXP_CAST_NONE || cast > MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_copy_view: unknown conversion code");
+    if (cast != MXP_CAST_NONE && elem_size != ((cast == MXP_CAST_BF16_F32 || cast == MXP_CAST_F16_F32) ? 4 : 2))
+      throw Error(MXP_ERR_ARG, "mxp_copy_view: elem_size is not the destination element size of the conversion");
+    std::vector<uint64_t> size;
+    for (int d = 0; d < ndim; ++d) size.push_back((uint64_t)shape[d]);
+    copy_view(*engine, src, dst, size, strides_or_row_major(src_strides, shape, ndim, what),
+              strides_or_row_major(dst_strides, shape, ndim, what), elem_size, cast, checksum,
+              static_cast<hipStream_t>(stream_v), what);
   });
 }
 

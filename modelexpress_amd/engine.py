@@ -397,6 +397,21 @@ class PlacementEngine:
                                          elem_size, C.byref(out) if checksum else None, C.c_void_p(stream)))
         return format(out.value, "08x") if checksum else None
 
+    def copy_view(self, src, dst, shape: Sequence[int], elem_size: int, *, src_strides: Sequence[int] | None = None,
+                  dst_strides: Sequence[int] | None = None, cast: int = 0, stream: int = 0,
+                  checksum: bool = True) -> str | None:
+        """``dst.as_strided(shape, dst_strides).copy_(src.as_strided(shape, src_strides))`` on the device
+        (strides in elements, ``None`` = contiguous).  ``src`` / ``dst`` address the first element of each
+        view; ``cast`` is a ``CAST_CODES`` value and ``elem_size`` then the destination element's size."""
+        n = len(shape)
+        shp = (C.c_int64 * max(1, n))(*[int(v) for v in shape])
+        ss = None if src_strides is None else (C.c_int64 * max(1, n))(*[int(v) for v in src_strides])
+        ds = None if dst_strides is None else (C.c_int64 * max(1, n))(*[int(v) for v in dst_strides])
+        out = C.c_uint32()
+        L.check(L.lib().mxp_copy_view(self._h, C.c_void_p(_addr(src)), C.c_void_p(_addr(dst)), n, shp, ss, ds,
+                                      elem_size, cast, C.byref(out) if checksum else None, C.c_void_p(stream)))
+        return format(out.value, "08x") if checksum else None
+
     def copy_batch(self, srcs: Sequence, dsts: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
                    checksums: bool = True) -> list[str] | None:
         """n contiguous device copies in one launch (optionally with destination checksums)."""

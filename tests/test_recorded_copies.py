@@ -1,0 +1,142 @@
+"""Recorded scatter copies (refit/reshard/types.py:57-71) executed on the device: the
+reference's own vectors for narrow / transpose / permute op-chains
+(tests/test_reshard_refit_slice_plan.py:54-79,155-197) and seeded random chains, against torch's
+``dest.as_strided(...).copy_(view)`` on the CPU - the operation the reference performs."""
+
+import numpy as np
+import pytest
+import torch
+
+from modelexpress_amd.reshard import RecordedCopy, UnsupportedReshard, execute_recorded_copies, replay_view
+
+
+def _apply(chain, t):
+    for op, args, kw in chain:
+        t = getattr(t, op)(*args, **dict(kw))
+    return t
+
+
+def test_replay_view_reference_vectors():
+    # test_reshard_refit_slice_plan.py:155-197 (transpose, 3-D permute, narrow + transpose)
+    assert replay_view((("transpose", (0, 1), ()),), (3, 4)) == (0, (4, 3), (1, 4))
+    assert replay_view((("permute", (2, 0, 1), ()),), (2, 3, 4)) == (0, (4, 2, 3), (1, 12, 4))
+    assert replay_view((("narrow", (0, 1, 2), ()), ("transpose", (0, 1), ())), (4, 5)) == (5, (5, 2), (1, 5))
+    # :54-65 narrow(1, 0, 4) of (4, 8): four runs at source elements 0, 8, 16, 24
+    assert replay_view((("narrow", (1, 0, 4), ()),), (4, 8)) == (0, (4, 4), (8, 1))
+    assert replay_view((("__getitem__", ((slice(1, 3), slice(None)),), ()),), (4, 6)) == (6, (2, 6), (6, 1))
+    # a copy inside the chain detaches the storage (slice_plan.py:155-159); a reshape that merges dims of a
+    # non-contiguous view copies as well
+    with pytest.raises(UnsupportedReshard, match="not a pure view"):
+        replay_view((("transpose", (0, 1), ()), ("contiguous", (), ())), (3, 4))
+    with pytest.raises(UnsupportedReshard, match="not a pure view"):
+        replay_view((("transpose", (0, 1), ()), ("reshape", (12,), ())), (3, 4))
+    with pytest.raises(UnsupportedReshard, match="non-tensor"):
+        replay_view((("size", (), ()),), (3, 4))
+
+
+CASES = [
+    # (source shape, op-chain, destination parameter shape, dest_offset, dest_stride or None = contiguous view shape)
+    ((3, 4), (("transpose", (0, 1), ()),), (4, 3), 0, None),
+    ((2, 3, 4), (("permute", (2, 0, 1), ()),), (4, 2, 3), 0, None),
+    ((4, 5), (("narrow", (0, 1, 2), ()), ("transpose", (0, 1), ())), (5, 2), 0, None),
+    ((4, 8), (("narrow", (1, 0, 4), ()),), (4, 4), 0, None),
+    ((64, 96), (("narrow", (0, 16, 32), ()),), (128, 96), 40 * 96, None),              # k rows of a fused qkv parameter
+    ((64, 96), (("narrow", (1, 48, 48), ()),), (64, 100), 3, (100, 1)),                # column block into a wider parameter
+    ((256, 192), (("transpose", (0, 1), ()),), (192, 256), 0, None),                   # whole transposed tiles
+    ((130, 70), (("transpose", (0, 1), ()),), (70, 200), 50, (200, 1)),                # transposed into a strided region
+    ((6, 40, 24), (("permute", (1, 2, 0), ()), ("narrow", (0, 8, 16), ())), (16, 24, 6), 0, None),
+    ((32, 48), (("t", (), ()),), (48, 64), 16, (1, 48)),                               # destination strided the other way: a plain row copy
+    ((20, 30), (("narrow", (0, 2, 10), ()),), (30, 10), 0, (1, 10)),                   # written transposed: the destination innermost run is the view's dim 0
+]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", range(len(CASES)))
+@pytest.mark.parametrize("dtypes", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
+                                    (torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.uint8, torch.uint8)])
+def test_recorded_copies_match_torch(gpu_engine, case, dtypes):
+    src_shape, chain, param_shape, dest_offset, dest_stride = CASES[case]
+    src_dt, dst_dt = dtypes
+    g = torch.Generator().manual_seed(100 + case)
+    if src_dt == torch.uint8:
+        src = torch.randint(0, 256, src_shape, dtype=torch.uint8, generator=g)
+    else:
+        src = (torch.randn(src_shape, generator=g) * 3).to(src_dt)
+    view = _apply(chain, src)
+    stride = dest_stride if dest_stride is not None else tuple(torch.empty(view.shape).stride())
+    want = torch.full(param_shape, 7, dtype=dst_dt)
+    want.as_strided(view.shape, stride, dest_offset).copy_(view)
+    param = torch.full(param_shape, 7, dtype=dst_dt, device="cuda")
+    copy = RecordedCopy("w", chain, "p", dest_offset, tuple(view.shape), tuple(stride), dst_dt)
+    n = execute_recorded_copies(gpu_engine, [copy], {"w": src.cuda()}, {"p": param})
+    assert n == view.numel() * param.element_size()
+    assert torch.equal(param.cpu().view(torch.uint8), want.view(torch.uint8))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", range(8))
+def test_random_chains_into_one_fused_parameter(gpu_engine, seed):
+    """Several sources scattered into disjoint row blocks of one parameter, each through a random
+    chain of narrow / transpose / permute; checked against torch on the CPU."""
+    rng = np.random.default_rng(700 + seed)
+    cols = int(rng.integers(3, 90))
+    copies, sources, row = [], {}, 0
+    blocks = []
+    for k in range(int(rng.integers(2, 6))):
+        nd = int(rng.integers(2, 4))
+        shape = tuple(int(v) for v in rng.integers(2, 40, nd))
+        src = torch.from_numpy(rng.integers(-2 ** 15, 2 ** 15, shape, dtype=np.int16)).view(torch.bfloat16)
+        chain = []
+        cur = src
+        for _ in range(int(rng.integers(1, 4))):
+            kind = int(rng.integers(0, 3))
+            if kind == 0:
+                d = int(rng.integers(0, cur.dim()))
+                if cur.shape[d] < 2:
+                    continue
+                start = int(rng.integers(0, cur.shape[d] - 1))
+                size = int(rng.integers(1, cur.shape[d] - start + 1))
+                op = ("narrow", (d, start, size), ())
+            elif kind == 1:
+                a, b = (int(v) for v in rng.choice(cur.dim(), 2, replace=False))
+                op = ("transpose", (a, b), ())
+            else:
+                op = ("permute", tuple(int(v) for v in rng.permutation(cur.dim())), ())
+            chain.append(op)
+            cur = _apply([op], cur)
+        # flatten the leading dims of the view into rows of the fused parameter; keep it when it fits
+        view = cur
+        rows = int(np.prod(view.shape[:-1]))
+        if view.shape[-1] > cols:
+            continue
+        lead = torch.empty(view.shape[:-1]).stride()
+        stride = tuple(int(s) * cols for s in lead) + (1,)
+        blocks.append((f"s{k}", tuple(chain), row * cols, tuple(view.shape), stride, view))
+        sources[f"s{k}"] = src
+        row += rows
+    if not blocks:
+        pytest.skip("no block fitted")
+    want = torch.full((row, cols), 7, dtype=torch.bfloat16)
+    for name, chain, off, shape, stride, view in blocks:
+        want.as_strided(shape, stride, off).copy_(view)
+        copies.append(RecordedCopy(name, chain, "fused", off, shape, stride, torch.bfloat16))
+    param = torch.full((row, cols), 7, dtype=torch.bfloat16, device="cuda")
+    execute_recorded_copies(gpu_engine, copies, {k: v.cuda() for k, v in sources.items()}, {"fused": param})
+    assert torch.equal(param.cpu().view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.gpu
+def test_nothing_moves_when_a_copy_cannot_be_resolved(gpu_engine):
+    src = torch.arange(12, dtype=torch.float32).reshape(3, 4).cuda()
+    param = torch.zeros(4, 3, device="cuda")
+    good = RecordedCopy("w", (("transpose", (0, 1), ()),), "p", 0, (4, 3), (3, 1))
+    bad = RecordedCopy("w", (("transpose", (0, 1), ()),), "p", 0, (3, 4), (4, 1))  # shape differs from the view
+    with pytest.raises(UnsupportedReshard, match="!= resolved view"):
+        execute_recorded_copies(gpu_engine, [good, bad], {"w": src}, {"p": param})
+    assert float(param.abs().sum()) == 0.0
+    with pytest.raises(UnsupportedReshard, match="leaves the parameter"):
+        execute_recorded_copies(gpu_engine, [RecordedCopy("w", (), "p", 4, (3, 4), (4, 1))], {"w": src}, {"p": param})
+    from modelexpress_amd._lib import MxpError
+
+    with pytest.raises(MxpError, match="overlaps itself"):
+        gpu_engine.copy_view(src, param, (3, 4), 4, dst_strides=(1, 1))
