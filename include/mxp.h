@@ -351,6 +351,25 @@ int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndi
 int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
                   const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_size,
                   int32_t cast, uint32_t* checksum, void* stream);
+/* One entry of mxp_copy_views: the arguments of mxp_copy_view. */
+typedef struct mxp_view_copy {
+  const void* src;
+  void* dst;
+  int32_t ndim;
+  int32_t elem_size;
+  int32_t cast;            /* MXP_CAST_* */
+  uint8_t contiguous_src;  /* 1: ignore src_strides, the source view is row-major contiguous */
+  uint8_t contiguous_dst;  /* 1: ignore dst_strides */
+  uint16_t reserved;
+  int64_t shape[MXP_MAX_DIMS];
+  int64_t src_strides[MXP_MAX_DIMS];
+  int64_t dst_strides[MXP_MAX_DIMS];
+} mxp_view_copy;
+/* n recorded copies at once: every view is lowered first (an error moves nothing), then all
+ * row / element boxes run in ONE launch and each transposed view in one launch of its own -
+ * in place of the reference's launch per view ("thousands of individual kernel launches",
+ * refit/reshard/receiver.py:920-923).  Destinations must not overlap one another. */
+int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, void* stream);
 /* n independent contiguous device copies in one launch, with the checksum of each
  * destination in out_checksums[k] when not NULL: the device form of the batched
  * torch._foreach_copy_ install (refit/reshard/receiver.py:939-955).  Destinations must

@@ -80,6 +80,13 @@ class Box(C.Structure):
                 ("csum_group", C.c_uint32), ("cast", C.c_uint32)]
 
 
+class ViewCopy(C.Structure):
+    _fields_ = [("src", C.c_void_p), ("dst", C.c_void_p), ("ndim", C.c_int32), ("elem_size", C.c_int32),
+                ("cast", C.c_int32), ("contiguous_src", C.c_uint8), ("contiguous_dst", C.c_uint8),
+                ("reserved", C.c_uint16), ("shape", C.c_int64 * 8), ("src_strides", C.c_int64 * 8),
+                ("dst_strides", C.c_int64 * 8)]
+
+
 class EngineOptions(C.Structure):
     _fields_ = [("device", C.c_int32), ("ring_slots", C.c_int32), ("slot_bytes", C.c_uint64),
                 ("reader_threads", C.c_int32), ("streams", C.c_int32), ("tile_bytes", C.c_uint32),
@@ -146,6 +153,7 @@ SIGNATURES = {
                                    C.POINTER(C.c_int32), C.c_int32, _U32P, _P]),
     "mxp_copy_view": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64),
                                 C.POINTER(C.c_int64), C.c_int32, C.c_int32, _U32P, _P]),
+    "mxp_copy_views": (C.c_int, [_P, C.POINTER(ViewCopy), C.c_int64, _P]),
     "mxp_copy_batch": (C.c_int, [_P, _PP, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_digest_from_scalars": (C.c_int, [_U64P, C.POINTER(C.c_uint8)]),

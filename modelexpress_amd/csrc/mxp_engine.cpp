@@ -909,20 +909,29 @@ namespace {
 //   * anything else                                 -> one element per box row (the run length
 //     the reference's paired_runs finds for such a view: slice_plan.py:259-294).
 // The checksum, when asked for, weights every written byte by its offset from `dst`.
-void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
-               std::vector<uint64_t> ds, int elem_size, int cast, uint32_t* checksum, hipStream_t stream,
-               const char* what) {
+struct TransposeJob {
+  const void* src;
+  void* dst;
+  TransposeDesc td;
+  int elem_size;
+};
+
+// Lowers one view copy: row / element boxes are appended to `boxes` (with their base pointers
+// in `srcs` / `dsts`), a transpose is returned in `tr`.  Returns false for an empty view.
+bool lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
+                std::vector<uint64_t> ds, int elem_size, int cast, uint32_t csum_slot, std::vector<BoxCopy>& boxes,
+                std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, bool& is_transpose,
+                const char* what) {
   const uint32_t op = seg_op_of_cast(cast);
   const uint64_t es = (uint64_t)elem_size;          // destination element
   const uint64_t es_s = op_src_bytes(op, es);       // source element
   auto fail = [&](int code, const std::string& msg) { throw Error(code, std::string(what) + ": " + msg); };
   uint64_t total = 1;
   for (auto n : size) total *= n;
-  if (checksum) *checksum = 0;
-  if (total == 0) return;
+  is_transpose = false;
+  if (total == 0) return false;
   if (!src || !dst) fail(MXP_ERR_ARG, "null pointer");
   if (reinterpret_cast<uintptr_t>(src) % es_s || reinterpret_cast<uintptr_t>(dst) % es) fail(MXP_ERR_ARG, "pointer is not element aligned");
-  HIP_OK(hipSetDevice(e.opt.device));
   {
     // drop unit dims, order by destination stride, refuse a self-overlapping destination, merge
     std::vector<size_t> order;
@@ -964,11 +973,14 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
     uint64_t so, d_o;
     split_ptr(src, sb, so);
     split_ptr(dst, db, d_o);
-    std::vector<BoxCopy> boxes;
     BoxCopy b;
+    b.src_buf = (uint32_t)srcs.size();
+    b.dst_buf = (uint32_t)dsts.size();
+    srcs.push_back(sb);
+    dsts.push_back(const_cast<void*>(db));
     b.row_bytes = n[m - 1] * es;
     b.op = op;
-    b.csum_slot = checksum ? 0u : 0xFFFFFFFFu;
+    b.csum_slot = csum_slot;
     b.csum_bias = (uint64_t)0 - d_o;
     if (m == 1) {
       b.src_off = so;
@@ -992,10 +1004,7 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
         for (int q = (int)m - 3; q >= 0; --q) { if (++idx[q] < n[q]) break; idx[q] = 0; }
       }
     }
-    uint32_t sum = 0;
-    run_boxes(e, boxes, {sb}, {const_cast<void*>(db)}, 1, checksum ? &sum : nullptr, stream);
-    if (checksum) *checksum = sum;
-    return;
+    return true;
   }
 
   // True transpose: i = destination innermost, j = the source's unit-stride dimension.
@@ -1030,6 +1039,12 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
   td.vec_dst = vd;
   td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
   for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
+  tr = TransposeJob{src, dst, td, elem_size};
+  is_transpose = true;
+  return true;
+}
+
+void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hipStream_t stream) {
   uint32_t* sum_dev = nullptr;
   if (checksum) {
     acquire_arena(e);
@@ -1037,13 +1052,35 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
     sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
     HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
   }
-  HIP_OK(launch_transpose(src, dst, td, elem_size, sum_dev, stream));
+  HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, sum_dev, stream));
   if (checksum) {
     HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
     std::memcpy(checksum, e.desc_host, 4);
     release_arena(e, stream);
   }
+}
+
+void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
+               std::vector<uint64_t> ds, int elem_size, int cast, uint32_t* checksum, hipStream_t stream,
+               const char* what) {
+  if (checksum) *checksum = 0;
+  std::vector<BoxCopy> boxes;
+  std::vector<const void*> srcs;
+  std::vector<void*> dsts;
+  TransposeJob tr{};
+  bool is_transpose = false;
+  if (!lower_view(src, dst, std::move(size), std::move(ss), std::move(ds), elem_size, cast, checksum ? 0u : 0xFFFFFFFFu,
+                  boxes, srcs, dsts, tr, is_transpose, what))
+    return;
+  HIP_OK(hipSetDevice(e.opt.device));
+  if (is_transpose) {
+    run_transpose(e, tr, checksum, stream);
+    return;
+  }
+  uint32_t sum = 0;
+  run_boxes(e, boxes, srcs, dsts, 1, checksum ? &sum : nullptr, stream);
+  if (checksum) *checksum = sum;
 }
 
 std::vector<uint64_t> strides_or_row_major(const int64_t* strides, const int64_t* shape, int32_t ndim, const char* what) {
@@ -1108,6 +1145,37 @@ int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, 
     copy_view(*engine, src, dst, size, strides_or_row_major(src_strides, shape, ndim, what),
               strides_or_row_major(dst_strides, shape, ndim, what), elem_size, cast, checksum,
               static_cast<hipStream_t>(stream_v), what);
+  });
+}
+
+int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, void* stream_v) {
+  return guard([&] {
+    const char* what = "mxp_copy_views";
+    if (!engine || n < 0 || (n && !views)) throw Error(MXP_ERR_ARG, "mxp_copy_views: bad argument");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    std::vector<BoxCopy> boxes;
+    std::vector<const void*> srcs;
+    std::vector<void*> dsts;
+    std::vector<TransposeJob> transposes;
+    for (int64_t k = 0; k < n; ++k) {  // everything is lowered before anything is launched
+      const mxp_view_copy& v = views[k];
+      check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
+      if (v.cast < MXP_CAST_NONE || v.cast > MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_copy_views: unknown conversion code");
+      if (v.cast != MXP_CAST_NONE && v.elem_size != ((v.cast == MXP_CAST_BF16_F32 || v.cast == MXP_CAST_F16_F32) ? 4 : 2))
+        throw Error(MXP_ERR_ARG, "mxp_copy_views: elem_size is not the destination element size of the conversion");
+      std::vector<uint64_t> size;
+      for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
+      TransposeJob tr{};
+      bool is_transpose = false;
+      if (lower_view(v.src, v.dst, size, strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what),
+                     strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what), v.elem_size,
+                     v.cast, 0xFFFFFFFFu, boxes, srcs, dsts, tr, is_transpose, what) &&
+          is_transpose)
+        transposes.push_back(tr);
+    }
+    HIP_OK(hipSetDevice(engine->opt.device));
+    if (!boxes.empty()) run_boxes(*engine, boxes, srcs, dsts, 1, nullptr, stream);
+    for (const auto& t : transposes) run_transpose(*engine, t, nullptr, stream);
   });
 }
 

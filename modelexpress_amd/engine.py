@@ -412,6 +412,22 @@ class PlacementEngine:
                                       elem_size, cast, C.byref(out) if checksum else None, C.c_void_p(stream)))
         return format(out.value, "08x") if checksum else None
 
+    def copy_views(self, views: Sequence[dict], *, stream: int = 0) -> None:
+        """Many ``copy_view`` calls in one go (keys: src, dst, shape, elem_size and optionally src_strides,
+        dst_strides, cast): all row / element boxes run in one launch, transposed views one launch each."""
+        arr = (L.ViewCopy * max(1, len(views)))()
+        for v, o in zip(views, arr):
+            shape = [int(x) for x in v["shape"]]
+            o.src, o.dst, o.ndim, o.elem_size, o.cast = _addr(v["src"]), _addr(v["dst"]), len(shape), int(v["elem_size"]), int(v.get("cast", 0))
+            for d, n in enumerate(shape):
+                o.shape[d] = n
+            for key, flag in (("src_strides", "contiguous_src"), ("dst_strides", "contiguous_dst")):
+                st = v.get(key)
+                setattr(o, flag, 1 if st is None else 0)
+                for d, x in enumerate(st or ()):
+                    getattr(o, key)[d] = int(x)
+        L.check(L.lib().mxp_copy_views(self._h, arr, len(views), C.c_void_p(stream)))
+
     def copy_batch(self, srcs: Sequence, dsts: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
                    checksums: bool = True) -> list[str] | None:
         """n contiguous device copies in one launch (optionally with destination checksums)."""

@@ -4,8 +4,8 @@ Mirrors the data model of the reference's reshard receiver: a ``RecordedCopy`` s
 ``src_name`` sliced by ``op_chain`` and write it into ``param_name`` at
 ``as_strided(dest_shape, dest_stride, dest_offset)``" (modelexpress/refit/reshard/types.py:57-71).
 The op-chain is replayed on a zero-storage tensor to a strided source view, as the reference
-does (refit/reshard/slice_plan.py:136-164, ``_replay_view``); the copy itself then runs as one
-``mxp_copy_view`` call: pitched boxes, the LDS transpose for a transposed innermost dimension,
+does (refit/reshard/slice_plan.py:136-164, ``_replay_view``); the copies then run through
+``mxp_copy_views``: pitched boxes (all of them in one launch), the LDS transpose for a transposed innermost dimension,
 or element runs - instead of the reference's per-run descriptors and per-view ``copy_``
 (slice_plan.py:259-339, receiver.py:919-960).  A dtype difference between source and
 parameter is converted on the way ("raw-copy vs convert-via-staging", types.py:62-63).
@@ -84,10 +84,12 @@ def execute_recorded_copies(engine: PlacementEngine, copies: Sequence[RecordedCo
         resolved.append((src.data_ptr() + off * src.element_size(), dst.data_ptr() + c.dest_offset * dst.element_size(),
                          shape, stride, tuple(int(s) for s in c.dest_stride), dst.element_size(), cast))
     written = 0
+    views = []
     for sp, dp, shape, ss, ds, es, cast in resolved:
-        engine.copy_view(sp, dp, shape, es, src_strides=ss, dst_strides=ds, cast=cast, stream=stream, checksum=False)
+        views.append({"src": sp, "dst": dp, "shape": shape, "elem_size": es, "src_strides": ss, "dst_strides": ds, "cast": cast})
         n = es
         for v in shape:
             n *= v
         written += n
+    engine.copy_views(views, stream=stream)  # one launch for every row / element box, one per transposed view
     return written

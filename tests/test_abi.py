@@ -41,14 +41,14 @@ def test_header_is_plain_c(tmp_path):
 
 def test_struct_layouts_match_the_header(mxp, tmp_path):
     src = tmp_path / "s.c"
-    src.write_text('#include <stdio.h>\n#include "mxp.h"\nint main(void){printf("%zu %zu %zu %zu %zu %zu\\n",'
+    src.write_text('#include <stdio.h>\n#include "mxp.h"\nint main(void){printf("%zu %zu %zu %zu %zu %zu %zu %zu\\n",'
                    "sizeof(mxp_tensor_info),sizeof(mxp_file_info),sizeof(mxp_write_info),sizeof(mxp_param_info),"
-                   "sizeof(mxp_engine_options),sizeof(mxp_exec_stats));return 0;}\n")
+                   "sizeof(mxp_engine_options),sizeof(mxp_exec_stats),sizeof(mxp_box),sizeof(mxp_view_copy));return 0;}\n")
     exe = tmp_path / "s"
     subprocess.run(["gcc", f"-I{ROOT / 'include'}", str(src), "-o", str(exe)], check=True)
     sizes = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
     assert sizes == [C.sizeof(mxp.TensorInfo), C.sizeof(mxp.FileInfo), C.sizeof(mxp.WriteInfo), C.sizeof(mxp.ParamInfo),
-                     C.sizeof(mxp.EngineOptions), C.sizeof(mxp.ExecStats)]
+                     C.sizeof(mxp.EngineOptions), C.sizeof(mxp.ExecStats), C.sizeof(mxp.Box), C.sizeof(mxp.ViewCopy)]
 
 
 def test_dtype_map_is_the_safetensors_one(mxp):
