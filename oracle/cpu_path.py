@@ -43,12 +43,14 @@ def _boxes(dst: np.ndarray, src: np.ndarray, cast: bool):
 
 
 def run(ckpt_dir: str, rank_params: list, *, tp_size=1, tp_rank=0, stacked=None, expert_mapping=None,
-        expert_local=None, allow_cast=False, nan_bits=0x7FC0, threads=1, repeats=1) -> dict:
+        expert_local=None, allow_cast=False, nan_bits=0x7FC0, threads=1, repeats=1, only_tensors=None) -> dict:
     """Parse, plan and place one rank on the CPU.  ``rank_params`` is ``[(name, dtype, shape)]``.
     Returns timings, the placed buffers and their checksums."""
     lib = cbind.load()
     t0 = time.perf_counter()
     weights = O.load_checkpoint(ckpt_dir, mmap=True)
+    if only_tensors is not None:  # a bounded sample: the checkpoint tensors that feed ``rank_params``
+        weights = [(n, t) for n, t in weights if n in only_tensors]
     t_parse = time.perf_counter() - t0
     params = {n: O.OTensor.zeros(shape, dtype) for n, dtype, shape in rank_params}
     index = {n: i for i, (n, _d, _s) in enumerate(rank_params)}
