@@ -243,29 +243,15 @@ class HipPlacementStrategy(LoadStrategy):
 
 def iter_checkpoint_tensors(model_uri: str, device: int = 0) -> Iterator[tuple[str, torch.Tensor]]:
     """Yield ``(name, device tensor)`` for every tensor of a checkpoint, one shard file at
-    a time through the pinned ring: the shape of the reference's per-file iterator
-    (gds_loader.py:84-156, ``raw.view(dtype).reshape(shape)`` at :327-328)."""
-    from .engine import Checkpoint, ParamSpec, PlacementPlan
+    a time through the pinned ring, the next file loading while the current one is consumed:
+    the reference's per-file iterator (gds_loader.py:84-156)."""
+    from .loader import MxHipLoader
 
-    eng = _engine_from_env(device)
+    loader = MxHipLoader(device=device)
     try:
-        top = Checkpoint(model_uri)
-        files = [f["path"] for f in top.files()]
-        wanted = {t.name for t in top.tensors()}
-        top.close()
-        for path in files:
-            ck = Checkpoint(path)
-            entries = [t for t in ck.tensors() if t.name in wanted]
-            params = [ParamSpec(t.name, t.dtype, t.shape) for t in entries]
-            plan = PlacementPlan(ck, params, allow_unmapped=True)
-            dst = eng.allocate(plan)
-            eng.execute(plan, dst)
-            for t, buf in zip(entries, dst):
-                yield t.name, buf.view(_TORCH_DTYPE[t.dtype]).reshape(t.shape)
-            plan.close()
-            ck.close()
+        yield from loader.load_iter(model_uri, use_tqdm=False)
     finally:
-        eng.close()
+        loader.shutdown()
 
 
 class HipStreamerStrategy(LoadStrategy):

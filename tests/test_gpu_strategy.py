@@ -227,3 +227,25 @@ def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
     assert ad.timing.emit().startswith("MX_REFIT_TIMING {")
     ad.release_staged_weight(staged)
     ad.close()
+
+
+def test_loader_class_has_the_reference_loader_interface(oracle, tmp_path, mxp):
+    # modelexpress/gds_loader.py:52-160: load() -> dict, load_iter() per file with prefetch, shutdown()
+    from modelexpress_amd.accelerators import HipAcceleratorBackend
+    from modelexpress_amd.loader import MxHipLoader
+
+    synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=3, seed=24)
+    want = oracle.load_checkpoint(str(tmp_path))
+    loader = MxHipLoader(HipAcceleratorBackend())
+    for _ in range(2):  # the engine is kept between calls
+        got = loader.load(str(tmp_path))
+        assert list(got) == [n for n, _ in want]
+        for n, t in want:
+            assert got[n].is_cuda and tuple(got[n].shape) == t.shape
+            assert got[n].contiguous().view(torch.uint8).cpu().numpy().tobytes() == t.tobytes(), n
+    first = next(iter(loader.load_iter(str(tmp_path), use_tqdm=False)))  # an abandoned iterator shuts its pool down
+    assert first[0] == want[0][0]
+    loader.shutdown()
+    loader.shutdown()
+    with pytest.raises(FileNotFoundError):
+        loader.load(str(tmp_path / "missing"))
