@@ -19,10 +19,13 @@ enum SegOp : uint32_t {
   kOpChecksumOnly = 2,  // read src, write nothing, accumulate checksum at dst_off indices
   kOpCastBf16F32 = 3,  // src is bf16, dst is fp32 (exact)
   kOpCastF16F32 = 4,   // src is fp16, dst is fp32 (exact; NaNs made quiet)
-  kOpCastF32F16 = 5    // src is fp32, dst is fp16 (round to nearest even)
+  kOpCastF32F16 = 5,   // src is fp32, dst is fp16 (round to nearest even)
+  kOpCastF8E4M3Bf16 = 6  // src is fp8 e4m3fn, dst is bf16 (exact; NaN -> 0x7FC0)
 };
 constexpr bool op_narrows(uint32_t op) { return op == kOpCastF32Bf16 || op == kOpCastF32F16; }
-constexpr bool op_widens(uint32_t op) { return op == kOpCastBf16F32 || op == kOpCastF16F32; }
+constexpr bool op_widens(uint32_t op) { return op == kOpCastBf16F32 || op == kOpCastF16F32 || op == kOpCastF8E4M3Bf16; }
+// Destination element size of a converting op (2 for a copy: only used for alignment rules).
+constexpr uint32_t op_dst_elem(uint32_t op) { return (op == kOpCastBf16F32 || op == kOpCastF16F32) ? 4u : 2u; }
 // Source bytes that produce `dst_bytes` destination bytes.
 constexpr uint64_t op_src_bytes(uint32_t op, uint64_t dst_bytes) {
   return op_narrows(op) ? dst_bytes * 2 : op_widens(op) ? dst_bytes / 2 : dst_bytes;
@@ -32,10 +35,10 @@ constexpr uint64_t op_dst_bytes(uint32_t op, uint64_t src_bytes) {
   return op_narrows(op) ? src_bytes / 2 : op_widens(op) ? src_bytes * 2 : src_bytes;
 }
 // Public conversion code of a write record (0 none, 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32,
-// 4 fp32->fp16) -> segment operation.
+// 4 fp32->fp16, 5 fp8-e4m3->bf16) -> segment operation.
 constexpr uint32_t seg_op_of_cast(int cast) {
   return cast == 1 ? kOpCastF32Bf16 : cast == 2 ? kOpCastBf16F32 : cast == 3 ? kOpCastF16F32
-       : cast == 4 ? kOpCastF32F16 : kOpCopy;
+       : cast == 4 ? kOpCastF32F16 : cast == 5 ? kOpCastF8E4M3Bf16 : kOpCopy;
 }
 
 // 80 bytes, 16-byte aligned; the index is workgroup-uniform, so the whole record

@@ -789,12 +789,12 @@ int mxp_cast(mxp_engine* engine, const void* src, void* dst, uint64_t n_elems, i
              void* stream) {
   return guard([&] {
     if (!engine || (n_elems && (!src || !dst))) throw Error(MXP_ERR_ARG, "mxp_cast: bad argument");
-    if (cast < MXP_CAST_F32_BF16 || cast > MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_cast: unknown conversion code");
+    if (cast < MXP_CAST_F32_BF16 || cast > MXP_CAST_LAST) throw Error(MXP_ERR_ARG, "mxp_cast: unknown conversion code");
     if (checksum) *checksum = 0;
     if (n_elems == 0) return;
     HIP_OK(hipSetDevice(engine->opt.device));
     const uint32_t op = seg_op_of_cast(cast);
-    const uint64_t dst_es = op_widens(op) ? 4 : 2, src_es = op_widens(op) ? 2 : 4;
+    const uint64_t dst_es = op_dst_elem(op), src_es = op_src_bytes(op, dst_es);
     if (reinterpret_cast<uintptr_t>(src) % src_es) throw Error(MXP_ERR_ARG, "mxp_cast: src must be element aligned");
     if (reinterpret_cast<uintptr_t>(dst) & 15u) throw Error(MXP_ERR_ARG, "mxp_cast: dst must be 16-byte aligned");
     const void* sb;
@@ -863,9 +863,9 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n
       if (x.rows == 0 || x.row_bytes == 0) continue;
       if (!x.src || !x.dst) throw Error(MXP_ERR_ARG, "mxp_place_boxes: null pointer");
       if (x.csum_group >= (n_groups ? n_groups : 1)) throw Error(MXP_ERR_ARG, "mxp_place_boxes: csum_group out of range");
-      if (x.cast > (uint32_t)MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_place_boxes: unknown conversion code");
+      if (x.cast > (uint32_t)MXP_CAST_LAST) throw Error(MXP_ERR_ARG, "mxp_place_boxes: unknown conversion code");
       const uint32_t op = seg_op_of_cast((int)x.cast);
-      if ((op_narrows(op) && x.row_bytes % 2) || (op_widens(op) && x.row_bytes % 4))
+      if (op != kOpCopy && x.row_bytes % op_dst_elem(op))
         throw Error(MXP_ERR_ARG, "mxp_place_boxes: row_bytes is not a whole number of elements");
       if (x.rows > 1 && (x.src_pitch < op_src_bytes(op, x.row_bytes) || x.dst_pitch < x.row_bytes))
         throw Error(MXP_ERR_ARG, "mxp_place_boxes: pitch smaller than the row");
@@ -1137,8 +1137,8 @@ int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, 
   return guard([&] {
     const char* what = "mxp_copy_view";
     check_view_args(engine, ndim, shape, elem_size, what);
-    if (cast < MXP_CAST_NONE || cast > MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_copy_view: unknown conversion code");
-    if (cast != MXP_CAST_NONE && elem_size != ((cast == MXP_CAST_BF16_F32 || cast == MXP_CAST_F16_F32) ? 4 : 2))
+    if (cast < MXP_CAST_NONE || cast > MXP_CAST_LAST) throw Error(MXP_ERR_ARG, "mxp_copy_view: unknown conversion code");
+    if (cast != MXP_CAST_NONE && elem_size != (int32_t)op_dst_elem(seg_op_of_cast(cast)))
       throw Error(MXP_ERR_ARG, "mxp_copy_view: elem_size is not the destination element size of the conversion");
     std::vector<uint64_t> size;
     for (int d = 0; d < ndim; ++d) size.push_back((uint64_t)shape[d]);
@@ -1160,8 +1160,8 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
     for (int64_t k = 0; k < n; ++k) {  // everything is lowered before anything is launched
       const mxp_view_copy& v = views[k];
       check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
-      if (v.cast < MXP_CAST_NONE || v.cast > MXP_CAST_F32_F16) throw Error(MXP_ERR_ARG, "mxp_copy_views: unknown conversion code");
-      if (v.cast != MXP_CAST_NONE && v.elem_size != ((v.cast == MXP_CAST_BF16_F32 || v.cast == MXP_CAST_F16_F32) ? 4 : 2))
+      if (v.cast < MXP_CAST_NONE || v.cast > MXP_CAST_LAST) throw Error(MXP_ERR_ARG, "mxp_copy_views: unknown conversion code");
+      if (v.cast != MXP_CAST_NONE && v.elem_size != (int32_t)op_dst_elem(seg_op_of_cast(v.cast)))
         throw Error(MXP_ERR_ARG, "mxp_copy_views: elem_size is not the destination element size of the conversion");
       std::vector<uint64_t> size;
       for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);

@@ -108,6 +108,18 @@ __device__ __forceinline__ uint32_t narrow1(uint32_t u, uint32_t nan_bits) {
   if constexpr (OP == kOpCastF32F16) return f32_to_f16_bits(u);
   else return f32_to_bf16_bits(u, nan_bits);
 }
+// fp8 e4m3fn bits -> bf16 bits, exact: bias 7 -> 127, subnormals (m * 2^-9) renormalised, the
+// two NaN codes -> 0x7FC0 (torch's image).  Reference: .to(out_dtype) at
+// engines/vllm/refit/receiver.py:258-261 when kv_b_proj is stored in fp8.
+__device__ __forceinline__ uint32_t f8e4m3_to_bf16_bits(uint32_t c) {
+  const uint32_t sign = (c & 0x80u) << 8, e = (c >> 3) & 0xFu, m = c & 7u;
+  if ((c & 0x7Fu) == 0x7Fu) return 0x7FC0u;
+  if (e != 0u) return sign | ((e + 120u) << 7) | (m << 4);
+  if (m == 0u) return sign;
+  const uint32_t top = 31u - (uint32_t)__clz((int)m);
+  return sign | ((top + 118u) << 7) | ((m << (7u - top)) & 0x7Fu);
+}
+
 template <int OP>
 __device__ __forceinline__ uint32_t widen1(uint32_t h) {
   if constexpr (OP == kOpCastF16F32) return f16_to_f32_bits(h);
@@ -122,6 +134,12 @@ __device__ __forceinline__ uint2 narrow4(const uint4& a, uint32_t nan_bits) {
 }
 template <int OP>
 __device__ __forceinline__ uint4 widen4(const uint2& a) {
+  if constexpr (OP == kOpCastF8E4M3Bf16) {  // eight one-byte elements in, eight bf16 out
+    auto two = [](uint32_t w, int sh) {
+      return f8e4m3_to_bf16_bits((w >> sh) & 0xFFu) | (f8e4m3_to_bf16_bits((w >> (sh + 8)) & 0xFFu) << 16);
+    };
+    return make_uint4(two(a.x, 0), two(a.x, 16), two(a.y, 0), two(a.y, 16));
+  } else
   return make_uint4(widen1<OP>(a.x & 0xFFFFu), widen1<OP>(a.x >> 16), widen1<OP>(a.y & 0xFFFFu), widen1<OP>(a.y >> 16));
 }
 
@@ -247,6 +265,16 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
         static_assert(UNIT == 2, "the element-wise cast path moves one element per lane");
         x = narrow1<OP>(*reinterpret_cast<const uint32_t*>(src + so), nan_bits);
         *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+      } else if constexpr (OP == kOpCastF8E4M3Bf16) {
+        if constexpr (UNIT == 4) {  // two elements per lane
+          const uint32_t w = *reinterpret_cast<const uint16_t*>(src + so);
+          x = f8e4m3_to_bf16_bits(w & 0xFFu) | (f8e4m3_to_bf16_bits(w >> 8) << 16);
+          *reinterpret_cast<uint32_t*>(dst + d_o) = x;
+        } else {
+          static_assert(UNIT == 2, "one element per lane");
+          x = f8e4m3_to_bf16_bits(src[so]);
+          *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+        }
       } else if constexpr (WIDEN) {
         static_assert(UNIT == 4, "the element-wise cast path moves one element per lane");
         x = widen1<OP>(*reinterpret_cast<const uint16_t*>(src + so));
@@ -302,6 +330,9 @@ __device__ __forceinline__ void place_body(
     case kOpCastBf16F32 * 32u + 4u: run_tile<kOpCastBf16F32, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF16F32 * 32u + 16u: run_tile<kOpCastF16F32, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF16F32 * 32u + 4u: run_tile<kOpCastF16F32, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF8E4M3Bf16 * 32u + 16u: run_tile<kOpCastF8E4M3Bf16, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF8E4M3Bf16 * 32u + 4u: run_tile<kOpCastF8E4M3Bf16, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF8E4M3Bf16 * 32u + 2u: run_tile<kOpCastF8E4M3Bf16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 4u: run_tile<kOpChecksumOnly, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 1u: run_tile<kOpChecksumOnly, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;

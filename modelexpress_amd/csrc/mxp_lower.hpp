@@ -51,6 +51,7 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
   } else if (op_widens(b.op)) {
     if (all_mult(16, 8)) unit = 16;
     else if (all_mult(4, 2)) unit = 4;
+    else if (op_dst_elem(b.op) == 2 && all_mult(2, 1)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
   } else {
     unit = all_mult(16, 16) ? 16 : all_mult(4, 4) ? 4 : 1;

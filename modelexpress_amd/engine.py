@@ -51,7 +51,7 @@ class VirtualTensor:
 
 
 # MXP_CAST_* of include/mxp.h
-CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4}
+CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4, ("F8_E4M3", "BF16"): 5}
 
 
 @dataclass(frozen=True)

@@ -201,8 +201,10 @@ def cast_tensor_f32_bf16(t: OTensor, nan_bits: int = 0x7FC0) -> OTensor:
 # The receive side of the same path converts the other way: "Cast the served bf16 staging
 # into the (fp32) receive buffer - a torch op" (refit/reshard/receiver.py:962-969), and a
 # half-precision engine takes fp32 trainer weights as fp16.  Conversion codes, shared with
-# the product's write records: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16.
-CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4}
+# the product's write records: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16,
+# 5 fp8-e4m3 -> bf16 (the ``.to(out_dtype)`` of the MLA absorbed weights when ``kv_b_proj`` is
+# stored in fp8: engines/vllm/refit/receiver.py:258-261).
+CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4, ("F8_E4M3", "BF16"): 5}
 
 
 def cast_bf16_f32_bits(u16: np.ndarray) -> np.ndarray:
@@ -250,6 +252,23 @@ def cast_f32_f16_bits(u32: np.ndarray) -> np.ndarray:
     return (sign | out).astype(np.uint16)
 
 
+_F8_TOP_BIT = np.array([0, 0, 1, 1, 2, 2, 2, 2], dtype=np.uint16)
+
+
+def cast_f8e4m3_bf16_bits(u8: np.ndarray) -> np.ndarray:
+    """Exact: e4m3fn (bias 7, no infinities, 0x7F / 0xFF = NaN) into bf16.  Subnormals
+    (m * 2^-9) are renormalised; both NaN codes become 0x7FC0, as torch's conversion does."""
+    c = u8.astype(np.uint16)
+    sign = (c & 0x80) << 8
+    e = (c >> 3) & 0xF
+    m = c & 7
+    top = _F8_TOP_BIT[m]
+    sub = np.where(m == 0, sign, sign | ((top + 118) << 7) | ((m << (7 - top)) & 0x7F))
+    normal = sign | ((e + 120) << 7) | (m << 4)
+    out = np.where(e == 0, sub, normal)
+    return np.where((e == 15) & (m == 7), np.uint16(0x7FC0), out).astype(np.uint16)
+
+
 def cast_tensor(t: OTensor, dst_dtype: str, nan_bits: int = 0x7FC0) -> OTensor:
     """dtype conversion of ``dest.copy_(src)`` for the supported pairs."""
     code = CAST_CODES.get((t.dtype, dst_dtype))
@@ -260,6 +279,8 @@ def cast_tensor(t: OTensor, dst_dtype: str, nan_bits: int = 0x7FC0) -> OTensor:
         return cast_tensor_f32_bf16(t, nan_bits)
     if code == 4:
         return OTensor.from_array(cast_f32_f16_bits(src.view("<u4").reshape(t.shape)).astype("<u2"), "F16")
+    if code == 5:
+        return OTensor.from_array(cast_f8e4m3_bf16_bits(src.view("u1").reshape(t.shape)).astype("<u2"), "BF16")
     fn = cast_bf16_f32_bits if code == 2 else cast_f16_f32_bits
     return OTensor.from_array(fn(src.view("<u2").reshape(t.shape)).astype("<u4"), "F32")
 

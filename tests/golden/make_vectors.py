@@ -8,7 +8,8 @@ digest and the cast, produced WITHOUT the oracle (oracle/) and without the produ
 * cast            torch's CPU float32 -> bfloat16 conversion (non-NaN inputs only: the NaN
                   image depends on the host's instruction set), and its float32 -> float16,
                   bfloat16 -> float32 and float16 -> float32 conversions (the widening ones on
-                  every 64th 16-bit pattern plus the special ones).
+                  every 64th 16-bit pattern plus the special ones), and float8_e4m3fn -> bfloat16
+                  on all 256 codes.
 
 Inputs come from a fixed linear congruential generator so the file is reproducible with
 nothing but the standard library and torch.  Run: python tests/golden/make_vectors.py
@@ -92,6 +93,9 @@ def main():
     g = h.view(torch.bfloat16).to(torch.float32).view(torch.int32).tolist()
     vec["cast_f16_f32"] = {"f16_bits": [halves[i] for i in not_nan16], "f32_bits": [f[i] & M32 for i in not_nan16]}
     vec["cast_bf16_f32"] = {"bf16_bits": [halves[i] for i in not_nan_bf], "f32_bits": [g[i] & M32 for i in not_nan_bf]}
+    codes = torch.arange(256, dtype=torch.uint8)
+    vec["cast_f8e4m3_bf16"] = {"f8_bits": list(range(256)),
+                               "bf16_bits": [v & 0xFFFF for v in codes.view(torch.float8_e4m3fn).to(torch.bfloat16).view(torch.int16).tolist()]}
     Path(__file__).with_name("vectors.json").write_text(json.dumps(vec, indent=0, separators=(",", ":")))
     print("wrote", Path(__file__).with_name("vectors.json"))
 

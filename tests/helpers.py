@@ -50,7 +50,8 @@ def apply_plan_numpy(ck: Checkpoint, plan: PlacementPlan, nan_bits=0x7FC0) -> di
         t = tensors[w.tensor]
         src = files[t.file_index][t.file_offset : t.file_offset + t.nbytes]
         dst = out[w.param]
-        src_row = {0: w.row_bytes, 1: w.row_bytes * 2, 4: w.row_bytes * 2, 2: w.row_bytes // 2, 3: w.row_bytes // 2}[w.cast]
+        src_row = {0: w.row_bytes, 1: w.row_bytes * 2, 4: w.row_bytes * 2, 2: w.row_bytes // 2, 3: w.row_bytes // 2,
+                   5: w.row_bytes // 2}[w.cast]
         for r in range(w.rows):
             s = src[w.src_offset + r * w.src_pitch : w.src_offset + r * w.src_pitch + src_row]
             if w.cast == 1:
@@ -60,9 +61,10 @@ def apply_plan_numpy(ck: Checkpoint, plan: PlacementPlan, nan_bits=0x7FC0) -> di
                 s = b.view(np.uint8)
             elif w.cast == 2:
                 s = (s.view("<u2").astype(np.uint32) << 16).view(np.uint8)
-            elif w.cast in (3, 4):  # torch is the library the reference converts with
+            elif w.cast in (3, 4, 5):  # torch is the library the reference converts with
                 import torch
-                src_t, dst_t = (torch.float16, torch.float32) if w.cast == 3 else (torch.float32, torch.float16)
+                src_t, dst_t = {3: (torch.float16, torch.float32), 4: (torch.float32, torch.float16),
+                                5: (torch.float8_e4m3fn, torch.bfloat16)}[w.cast]
                 s = torch.from_numpy(s.copy()).view(src_t).to(dst_t).view(torch.uint8).numpy()
             dst[w.dst_offset + r * w.dst_pitch : w.dst_offset + r * w.dst_pitch + w.row_bytes] = s
     return out

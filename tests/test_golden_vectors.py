@@ -15,8 +15,10 @@ VEC = json.loads((Path(__file__).parent / "golden" / "vectors.json").read_text()
 # (fixture key, source field, destination field, oracle function, MXP_CAST_* code, source dtype, destination dtype)
 _CASTS = [("cast_f32_f16", "f32_bits", "f16_bits", "cast_f32_f16_bits", 4),
           ("cast_f16_f32", "f16_bits", "f32_bits", "cast_f16_f32_bits", 3),
-          ("cast_bf16_f32", "bf16_bits", "f32_bits", "cast_bf16_f32_bits", 2)]
-_DTYPES = {4: ("F32", "F16"), 3: ("F16", "F32"), 2: ("BF16", "F32")}
+          ("cast_bf16_f32", "bf16_bits", "f32_bits", "cast_bf16_f32_bits", 2),
+          ("cast_f8e4m3_bf16", "f8_bits", "bf16_bits", "cast_f8e4m3_bf16_bits", 5)]
+_DTYPES = {4: ("F32", "F16"), 3: ("F16", "F32"), 2: ("BF16", "F32"), 5: ("F8_E4M3", "BF16")}
+_NP = {"f32_bits": np.uint32, "f16_bits": np.uint16, "bf16_bits": np.uint16, "f8_bits": np.uint8}
 
 
 def test_oracle_matches_golden_vectors(oracle, oracle_c):
@@ -36,8 +38,8 @@ def test_oracle_matches_golden_vectors(oracle, oracle_c):
     assert np.array_equal(oracle.cast_f32_bf16_bits(bits), want)
     assert np.array_equal(oracle_c.cast_f32_bf16(bits), want)
     for key, src_k, dst_k, fn, code in _CASTS:
-        src = np.array(VEC[key][src_k], dtype=np.uint32 if src_k == "f32_bits" else np.uint16)
-        want = np.array(VEC[key][dst_k], dtype=np.uint32 if dst_k == "f32_bits" else np.uint16)
+        src = np.array(VEC[key][src_k], dtype=_NP[src_k])
+        want = np.array(VEC[key][dst_k], dtype=_NP[dst_k])
         assert np.array_equal(getattr(oracle, fn)(src), want), key
         assert np.array_equal(oracle_c.cast(code, src), want), key
 
@@ -60,8 +62,8 @@ def test_hip_path_matches_golden_vectors(gpu_engine):
     gpu_engine.cast_f32_bf16(src, dst, bits.size)
     assert np.array_equal(dst.cpu().numpy().view(np.uint16), want)
     for key, src_k, dst_k, _fn, code in _CASTS:
-        src = np.array(VEC[key][src_k], dtype=np.uint32 if src_k == "f32_bits" else np.uint16)
-        want = np.array(VEC[key][dst_k], dtype=np.uint32 if dst_k == "f32_bits" else np.uint16)
+        src = np.array(VEC[key][src_k], dtype=_NP[src_k])
+        want = np.array(VEC[key][dst_k], dtype=_NP[dst_k])
         d_src = torch.from_numpy(src.view(np.uint8).copy()).cuda()
         d_dst = torch.zeros(want.nbytes, dtype=torch.uint8, device="cuda")
         gpu_engine.cast(d_src, d_dst, src.size, *_DTYPES[code])

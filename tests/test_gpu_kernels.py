@@ -86,7 +86,7 @@ def test_cast_f32_bf16_matches_oracle(gpu_engine, oracle, oracle_c):
         assert int(d[src.size * 2:].sum()) == 0  # nothing written past the end
 
 
-@pytest.mark.parametrize("src_dtype,dst_dtype", [("BF16", "F32"), ("F16", "F32"), ("F32", "F16")])
+@pytest.mark.parametrize("src_dtype,dst_dtype", [("BF16", "F32"), ("F16", "F32"), ("F32", "F16"), ("F8_E4M3", "BF16")])
 def test_cast_pairs_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dtype):
     """The other conversions of dest.copy_(src) (refit/reshard/receiver.py:962-969): every 16-bit
     pattern for the widening ones, every rounding class for fp32 -> fp16, odd sizes and offsets."""
@@ -98,6 +98,9 @@ def test_cast_pairs_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dt
         full = np.concatenate([(hi[:, None] | lows[None, :]).reshape(-1),
                                rng.integers(0, 1 << 32, (1 << 20) + 3, dtype=np.uint64).astype(np.uint32)])
         fn, se, de = oracle.cast_f32_f16_bits, 4, 2
+    elif src_dtype == "F8_E4M3":
+        full = np.concatenate([np.arange(256, dtype=np.uint8), rng.integers(0, 256, (1 << 20) + 5, dtype=np.uint8)])
+        fn, se, de = oracle.cast_f8e4m3_bf16_bits, 1, 2
     else:
         full = np.concatenate([np.arange(1 << 16, dtype=np.uint16), rng.integers(0, 1 << 16, (1 << 20) + 5, dtype=np.uint16)])
         fn, se, de = (oracle.cast_bf16_f32_bits if src_dtype == "BF16" else oracle.cast_f16_f32_bits), 2, 4
@@ -292,19 +295,19 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
     want = np.full(out_size, 0xEE, dtype=np.uint8)
     boxes, sums_want, cursor = [], [], 0
     for g in range(int(rng.integers(1, 9))):
-        cast = int(rng.choice([0, 0, 0, 1, 2, 3, 4]))  # MXP_CAST_* code
-        narrow, widen = cast in (1, 4), cast in (2, 3)
-        align = int(rng.choice([1, 2, 4, 8, 16])) if not cast else int(rng.choice([4, 8, 16]) if widen else rng.choice([2, 4, 8, 16]))
+        cast = int(rng.choice([0, 0, 0, 1, 2, 3, 4, 5]))  # MXP_CAST_* code
+        narrow, widen = cast in (1, 4), cast in (2, 3, 5)
+        align = int(rng.choice([1, 2, 4, 8, 16])) if not cast else int(rng.choice([4, 8, 16]) if cast in (2, 3) else rng.choice([2, 4, 8, 16]))
         rows = int(rng.choice([1, 1, 2, 7, 64, 513, 3000]))
         row_bytes = int(rng.integers(1, 40)) * align if rng.integers(0, 4) else int(rng.integers(1, 5)) * 20000 // align * align
-        row_bytes = max(align, row_bytes - row_bytes % (4 if widen else 2 if narrow else 1))
+        row_bytes = max(align, row_bytes - row_bytes % (4 if cast in (2, 3) else 2 if cast else 1))
         src_row = row_bytes * 2 if narrow else row_bytes // 2 if widen else row_bytes
         src_align = align * 2 if narrow else align // 2 if widen else align
         dst_pitch = row_bytes + int(rng.integers(0, 4)) * align
         src_pitch = src_row + int(rng.integers(0, 5)) * src_align
         if rows * max(dst_pitch, 1) > (1 << 20) or rows * src_pitch > (4 << 20):
             rows = max(1, min((1 << 20) // dst_pitch, (4 << 20) // src_pitch))
-        src_off = int(rng.integers(0, 64)) * (4 if narrow else 2 if widen else 1)
+        src_off = int(rng.integers(0, 64)) * (4 if narrow else 2 if cast in (2, 3) else 1)
         src_off -= src_off % (min(src_align, 16) if cast else min(align, 16))
         dst_off = (cursor + 15) // 16 * 16
         if rows == 1 and not cast and align < 16 and rng.integers(0, 2):
@@ -320,6 +323,8 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
                 s = oracle.cast_bf16_f32_bits(s.view(np.uint16)).view(np.uint8)
             elif cast == 3:
                 s = oracle.cast_f16_f32_bits(s.view(np.uint16)).view(np.uint8)
+            elif cast == 5:
+                s = oracle.cast_f8e4m3_bf16_bits(s).view(np.uint8)
             want[dst_off + r * dst_pitch: dst_off + r * dst_pitch + row_bytes] = s
             csum += int(oracle_c.checksum32(s, first_index=1000 + r * dst_pitch), 16)
         sums_want.append(format(csum & 0xFFFFFFFF, "08x"))

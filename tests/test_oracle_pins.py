@@ -229,6 +229,17 @@ def test_widening_casts_match_torch_on_every_pattern(oracle, oracle_c):
     assert np.array_equal(oracle.cast_f32_bf16_bits(oracle.cast_bf16_f32_bits(h))[not_nan_bf], h[not_nan_bf])
 
 
+def test_fp8_e4m3_to_bf16_matches_torch_on_every_code(oracle, oracle_c):
+    # engines/vllm/refit/receiver.py:258-261: w_uk.permute(1, 2, 0).to(out_dtype) with an fp8 kv_b_proj
+    codes = np.arange(256, dtype=np.uint8)
+    ref = torch.from_numpy(codes.copy()).view(torch.float8_e4m3fn).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(oracle.cast_f8e4m3_bf16_bits(codes), ref)
+    assert np.array_equal(oracle_c.cast(5, codes), ref)
+    # hand values: 1.0 (0x38), -448 (largest), 2^-9 (smallest subnormal), 2^-6 (smallest normal), NaN of either sign
+    hv = np.array([0x38, 0xFE, 0x01, 0x08, 0x7F, 0xFF], dtype=np.uint8)
+    assert oracle.cast_f8e4m3_bf16_bits(hv).tolist() == [0x3F80, 0xC3E0, 0x3B00, 0x3C80, 0x7FC0, 0x7FC0]
+
+
 def test_f32_to_f16_matches_torch_and_numpy(oracle, oracle_c):
     hi = np.arange(1 << 16, dtype=np.uint32) << 16
     lows = np.array([0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF, 0x2000, 0x2FFF, 0x3000, 0x7FFF, 0x8000, 0x8001, 0xFFFF],

@@ -285,5 +285,12 @@ def test_widening_and_half_conversions_are_planned(mxp, oracle, tmp_path):
     assert (a.cast, a.rows, a.row_bytes, a.src_offset, a.src_pitch, a.dst_pitch) == (2, 4, 16, 8, 16, 16)
     assert (b.cast, b.rows, b.row_bytes, b.src_offset, b.src_pitch, b.dst_pitch) == (3, 4, 16, 8, 16, 16)
     assert (c.cast, c.rows, c.row_bytes, c.src_offset, c.src_pitch, c.dst_pitch) == (4, 4, 8, 16, 32, 8)
+    # fp8-e4m3 into bf16 (receiver.py:258-261): one byte in, two out
+    save_file({"d.weight": w.to(torch.float8_e4m3fn)}, str(tmp_path / "model.safetensors"))
+    plan8 = PlacementPlan(Checkpoint(str(tmp_path)), [ParamSpec("d.weight", "BF16", (4, 4))], tp_size=2, tp_rank=1, allow_cast=True)
+    d = plan8.writes()[0]
+    assert (d.cast, d.rows, d.row_bytes, d.src_offset, d.src_pitch, d.dst_pitch) == (5, 4, 8, 4, 8, 8)
+    assert apply_plan_numpy(Checkpoint(str(tmp_path)), plan8)["d.weight"].tobytes() == \
+        w[:, 4:].to(torch.float8_e4m3fn).to(torch.bfloat16).contiguous().view(torch.uint8).numpy().tobytes()
     with pytest.raises(MxpError, match="no conversion"):  # pairs outside the table stay refused
         PlacementPlan(ck, [ParamSpec("a.weight", "F16", (4, 8))], allow_cast=True, allow_uncovered=True, allow_unmapped=True)
