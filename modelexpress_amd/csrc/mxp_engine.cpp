@@ -110,6 +110,7 @@ struct mxp_engine {
   uint8_t* desc_host = nullptr;  // pinned
   size_t desc_host_cap = 0;
   DevBuf<uint8_t> desc_dev;
+  DevBuf<uint8_t> view_tmp;  // scratch of converting transposes
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
   hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
   bool arena_recorded = false;
@@ -916,20 +917,26 @@ struct TransposeJob {
   int elem_size;
 };
 
-// Lowers one view copy: row / element boxes are appended to `boxes` (with their base pointers
-// in `srcs` / `dsts`), a transpose is returned in `tr`.  Returns false for an empty view.
-bool lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
-                std::vector<uint64_t> ds, int elem_size, int cast, uint32_t csum_slot, std::vector<BoxCopy>& boxes,
-                std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, bool& is_transpose,
-                const char* what) {
+enum ViewKind {
+  kViewEmpty,          // nothing to move
+  kViewBoxes,          // row / element boxes appended to `boxes`
+  kViewTranspose,      // `tr` holds the whole copy
+  kViewNeedsScratch,   // a converting transpose: call again with `scratch` of total * source-element bytes
+  kViewTransposeBoxes  // `tr` transposes into `scratch` at the source dtype, then `boxes` convert rows out of it
+};
+
+// Lowers one view copy.  Boxes are appended to `boxes` with their base pointers in `srcs` / `dsts`.
+ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
+                    std::vector<uint64_t> ds, int elem_size, int cast, uint32_t csum_slot, std::vector<BoxCopy>& boxes,
+                    std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, void* scratch,
+                    const char* what) {
   const uint32_t op = seg_op_of_cast(cast);
   const uint64_t es = (uint64_t)elem_size;          // destination element
   const uint64_t es_s = op_src_bytes(op, es);       // source element
   auto fail = [&](int code, const std::string& msg) { throw Error(code, std::string(what) + ": " + msg); };
   uint64_t total = 1;
   for (auto n : size) total *= n;
-  is_transpose = false;
-  if (total == 0) return false;
+  if (total == 0) return kViewEmpty;
   if (!src || !dst) fail(MXP_ERR_ARG, "null pointer");
   if (reinterpret_cast<uintptr_t>(src) % es_s || reinterpret_cast<uintptr_t>(dst) % es) fail(MXP_ERR_ARG, "pointer is not element aligned");
   {
@@ -960,18 +967,19 @@ bool lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vec
   for (size_t d = 0; d + 1 < nd; ++d)
     if (ss[d] == 1) c = (int)d;
   const bool dst_inner = ds[nd - 1] == 1 || total == 1;
-  const bool transpose = op == kOpCopy && dst_inner && ss[nd - 1] != 1 && total != 1 && c >= 0 && nd - 2 <= (size_t)kMaxBatchDims;
+  const bool transposed = dst_inner && ss[nd - 1] != 1 && total != 1 && c >= 0 && nd - 2 <= (size_t)kMaxBatchDims;
 
-  if (!transpose) {
-    // Row boxes: whole innermost rows when both sides are contiguous there, else one element per row.
-    const bool rows_ok = dst_inner && (ss[nd - 1] == 1 || total == 1);
-    std::vector<uint64_t> n = size, s = ss, d = ds;
+  // Row boxes from a source laid out with strides `s` at `sp`: whole innermost rows when both
+  // sides are contiguous there, else one element per row.
+  auto emit_boxes = [&](const void* sp, const std::vector<uint64_t>& s_in) {
+    const bool rows_ok = dst_inner && (s_in[nd - 1] == 1 || total == 1);
+    std::vector<uint64_t> n = size, s = s_in, d = ds;
     if (!rows_ok) { n.push_back(1); s.push_back(1); d.push_back(1); }  // a virtual innermost dimension of one element
     const size_t m = n.size();
     const void* sb;
     const void* db;
     uint64_t so, d_o;
-    split_ptr(src, sb, so);
+    split_ptr(sp, sb, so);
     split_ptr(dst, db, d_o);
     BoxCopy b;
     b.src_buf = (uint32_t)srcs.size();
@@ -986,62 +994,79 @@ bool lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vec
       b.src_off = so;
       b.dst_off = d_o;
       boxes.push_back(b);
-    } else {
-      b.rows = n[m - 2];
-      b.src_pitch = s[m - 2] * es_s;
-      b.dst_pitch = d[m - 2] * es;
-      uint64_t outer = 1;
-      for (size_t q = 0; q + 2 < m; ++q) outer *= n[q];
-      if (outer > (1u << 20)) fail(MXP_ERR_UNSUPPORTED, "too many row bands");
-      std::vector<uint64_t> idx(m, 0);
-      for (uint64_t o = 0; o < outer; ++o) {
-        uint64_t s_el = 0, d_el = 0;
-        for (size_t q = 0; q + 2 < m; ++q) { s_el += idx[q] * s[q]; d_el += idx[q] * d[q]; }
-        BoxCopy x = b;
-        x.src_off = so + s_el * es_s;
-        x.dst_off = d_o + d_el * es;
-        boxes.push_back(x);
-        for (int q = (int)m - 3; q >= 0; --q) { if (++idx[q] < n[q]) break; idx[q] = 0; }
-      }
+      return;
     }
-    return true;
-  }
+    b.rows = n[m - 2];
+    b.src_pitch = s[m - 2] * es_s;
+    b.dst_pitch = d[m - 2] * es;
+    uint64_t outer = 1;
+    for (size_t q = 0; q + 2 < m; ++q) outer *= n[q];
+    if (outer > (1u << 20)) fail(MXP_ERR_UNSUPPORTED, "too many row bands");
+    std::vector<uint64_t> idx(m, 0);
+    for (uint64_t o = 0; o < outer; ++o) {
+      uint64_t s_el = 0, d_el = 0;
+      for (size_t q = 0; q + 2 < m; ++q) { s_el += idx[q] * s[q]; d_el += idx[q] * d[q]; }
+      BoxCopy x = b;
+      x.src_off = so + s_el * es_s;
+      x.dst_off = d_o + d_el * es;
+      boxes.push_back(x);
+      for (int q = (int)m - 3; q >= 0; --q) { if (++idx[q] < n[q]) break; idx[q] = 0; }
+    }
+  };
 
-  // True transpose: i = destination innermost, j = the source's unit-stride dimension.
-  TransposeDesc td{};
-  td.ni = size[nd - 1];
-  td.si = ss[nd - 1];
-  td.nj = size[c];
-  td.dj = ds[c];
-  // Workgroup shape: as many wavefronts along i (long destination runs) as the extent can
-  // use, the rest along j.
-  uint32_t waves_i = 1;
-  while (waves_i < (uint32_t)kTransposeWaves && (uint64_t)waves_i * transpose_sub_rows(elem_size) < td.ni) waves_i *= 2;
-  td.waves_i = waves_i;
-  const uint64_t tile_i = (uint64_t)waves_i * transpose_sub_rows(elem_size);
-  const uint64_t tile_j = (uint64_t)(kTransposeWaves / waves_i) * transpose_sub_cols(elem_size);
-  td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
-  td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
-  bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * es) % 16 == 0;
-  bool vd = (reinterpret_cast<uintptr_t>(dst) % 16 == 0) && (td.dj * es) % 16 == 0;
-  int k = kMaxBatchDims - 1;
-  for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
-  for (int d = (int)nd - 2; d >= 0; --d) {
-    if (d == c) continue;
-    td.batch_size[k] = size[d];
-    td.batch_sstride[k] = ss[d];
-    td.batch_dstride[k] = ds[d];
-    vs = vs && (ss[d] * es) % 16 == 0;
-    vd = vd && (ds[d] * es) % 16 == 0;
-    --k;
+  // Transpose of `eb`-byte elements into `dp` laid out with strides `d_in` (innermost 1):
+  // i = destination innermost, j = the source's unit-stride dimension.
+  auto make_transpose = [&](void* dp, const std::vector<uint64_t>& d_in, uint64_t eb) {
+    TransposeDesc td{};
+    td.ni = size[nd - 1];
+    td.si = ss[nd - 1];
+    td.nj = size[c];
+    td.dj = d_in[c];
+    // Workgroup shape: as many wavefronts along i (long destination runs) as the extent can
+    // use, the rest along j.
+    uint32_t waves_i = 1;
+    while (waves_i < (uint32_t)kTransposeWaves && (uint64_t)waves_i * transpose_sub_rows((int)eb) < td.ni) waves_i *= 2;
+    td.waves_i = waves_i;
+    const uint64_t tile_i = (uint64_t)waves_i * transpose_sub_rows((int)eb);
+    const uint64_t tile_j = (uint64_t)(kTransposeWaves / waves_i) * transpose_sub_cols((int)eb);
+    td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
+    td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
+    bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * eb) % 16 == 0;
+    bool vd = (reinterpret_cast<uintptr_t>(dp) % 16 == 0) && (td.dj * eb) % 16 == 0;
+    int k = kMaxBatchDims - 1;
+    for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
+    for (int d = (int)nd - 2; d >= 0; --d) {
+      if (d == c) continue;
+      td.batch_size[k] = size[d];
+      td.batch_sstride[k] = ss[d];
+      td.batch_dstride[k] = d_in[d];
+      vs = vs && (ss[d] * eb) % 16 == 0;
+      vd = vd && (d_in[d] * eb) % 16 == 0;
+      --k;
+    }
+    td.vec_src = vs;
+    td.vec_dst = vd;
+    td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
+    for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
+    tr = TransposeJob{src, dp, td, (int)eb};
+  };
+
+  if (!transposed) {
+    emit_boxes(src, ss);
+    return kViewBoxes;
   }
-  td.vec_src = vs;
-  td.vec_dst = vd;
-  td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
-  for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
-  tr = TransposeJob{src, dst, td, elem_size};
-  is_transpose = true;
-  return true;
+  if (op == kOpCopy) {
+    make_transpose(dst, ds, es);
+    return kViewTranspose;
+  }
+  // A converting transpose: transpose at the source dtype into contiguous scratch (dimensions in
+  // destination order), then convert whole rows out of it.
+  if (!scratch) return kViewNeedsScratch;
+  std::vector<uint64_t> ts(nd, 1);
+  for (int d = (int)nd - 2; d >= 0; --d) ts[d] = ts[d + 1] * size[d + 1];
+  make_transpose(scratch, ts, es_s);
+  emit_boxes(scratch, ts);
+  return kViewTransposeBoxes;
 }
 
 void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hipStream_t stream) {
@@ -1061,6 +1086,20 @@ void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hip
   }
 }
 
+// Scratch for converting transposes; grown on demand, kept by the engine.  Users hold the
+// arena (acquire_arena / release_arena) from before the first kernel that writes it until
+// after the last one that reads it has been enqueued.
+void* view_scratch(mxp_engine& e, uint64_t bytes) {
+  e.view_tmp.reserve(align_up(bytes, 1 << 20));
+  return e.view_tmp.p;
+}
+
+uint64_t view_source_bytes(const std::vector<uint64_t>& size, int elem_size, int cast) {
+  uint64_t total = op_src_bytes(seg_op_of_cast(cast), (uint64_t)elem_size);
+  for (auto n : size) total *= n;
+  return total;
+}
+
 void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
                std::vector<uint64_t> ds, int elem_size, int cast, uint32_t* checksum, hipStream_t stream,
                const char* what) {
@@ -1069,15 +1108,20 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
   std::vector<const void*> srcs;
   std::vector<void*> dsts;
   TransposeJob tr{};
-  bool is_transpose = false;
-  if (!lower_view(src, dst, std::move(size), std::move(ss), std::move(ds), elem_size, cast, checksum ? 0u : 0xFFFFFFFFu,
-                  boxes, srcs, dsts, tr, is_transpose, what))
-    return;
+  const uint32_t slot = checksum ? 0u : 0xFFFFFFFFu;
+  ViewKind kind = lower_view(src, dst, size, ss, ds, elem_size, cast, slot, boxes, srcs, dsts, tr, nullptr, what);
+  if (kind == kViewEmpty) return;
   HIP_OK(hipSetDevice(e.opt.device));
-  if (is_transpose) {
+  if (kind == kViewNeedsScratch) {
+    acquire_arena(e);
+    void* tmp = view_scratch(e, view_source_bytes(size, elem_size, cast));
+    kind = lower_view(src, dst, size, ss, ds, elem_size, cast, slot, boxes, srcs, dsts, tr, tmp, what);
+  }
+  if (kind == kViewTranspose) {
     run_transpose(e, tr, checksum, stream);
     return;
   }
+  if (kind == kViewTransposeBoxes) run_transpose(e, tr, nullptr, stream);
   uint32_t sum = 0;
   run_boxes(e, boxes, srcs, dsts, 1, checksum ? &sum : nullptr, stream);
   if (checksum) *checksum = sum;
@@ -1157,6 +1201,7 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
     std::vector<const void*> srcs;
     std::vector<void*> dsts;
     std::vector<TransposeJob> transposes;
+    std::vector<int64_t> two_step;  // converting transposes: run one by one through the scratch buffer
     for (int64_t k = 0; k < n; ++k) {  // everything is lowered before anything is launched
       const mxp_view_copy& v = views[k];
       check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
@@ -1166,16 +1211,24 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
       std::vector<uint64_t> size;
       for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
       TransposeJob tr{};
-      bool is_transpose = false;
-      if (lower_view(v.src, v.dst, size, strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what),
-                     strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what), v.elem_size,
-                     v.cast, 0xFFFFFFFFu, boxes, srcs, dsts, tr, is_transpose, what) &&
-          is_transpose)
-        transposes.push_back(tr);
+      const auto s_st = strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what);
+      const auto d_st = strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what);
+      const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts,
+                                       tr, nullptr, what);
+      if (kind == kViewTranspose) transposes.push_back(tr);
+      else if (kind == kViewNeedsScratch) two_step.push_back(k);
     }
     HIP_OK(hipSetDevice(engine->opt.device));
     if (!boxes.empty()) run_boxes(*engine, boxes, srcs, dsts, 1, nullptr, stream);
     for (const auto& t : transposes) run_transpose(*engine, t, nullptr, stream);
+    for (int64_t k : two_step) {
+      const mxp_view_copy& v = views[k];
+      std::vector<uint64_t> size;
+      for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
+      copy_view(*engine, v.src, v.dst, size, strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what),
+                strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what), v.elem_size, v.cast,
+                nullptr, stream, what);
+    }
   });
 }
 

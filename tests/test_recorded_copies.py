@@ -141,3 +141,33 @@ def test_nothing_moves_when_a_copy_cannot_be_resolved(gpu_engine):
 
     with pytest.raises(MxpError, match="overlaps itself"):
         gpu_engine.copy_view(src, param, (3, 4), 4, dst_strides=(1, 1))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("src_dt", [torch.bfloat16, torch.float8_e4m3fn])
+def test_mla_absorbed_weights_as_recorded_copies(gpu_engine, src_dt):
+    """engines/vllm/refit/receiver.py:244-261 as two recorded copies out of kv_b_proj:
+    W_UV = w_uv.transpose(0, 1).to(out_dtype) and W_UK_T = w_uk.permute(1, 2, 0).to(out_dtype),
+    with kv_b_proj in bf16 or in fp8 (then the permute goes through the scratch transpose)."""
+    H, P, V, L = 16, 128, 128, 512
+    g = torch.Generator().manual_seed(5)
+    kv_b = (torch.randn(H * (P + V), L, generator=g) * 0.5).to(src_dt)
+    view = kv_b.view(H, P + V, L)
+    w_uk, w_uv = view.split([P, V], dim=1)
+    want_uv = w_uv.transpose(0, 1).to(torch.bfloat16).contiguous()
+    want_ukt = w_uk.permute(1, 2, 0).to(torch.bfloat16).contiguous()
+    head = ("view", (H, P + V, L), ())
+    copies = [
+        RecordedCopy("kv_b", (head, ("narrow", (1, P, V), ()), ("transpose", (0, 1), ())), "W_UV", 0, (V, H, L),
+                     tuple(want_uv.stride()), torch.bfloat16),
+        RecordedCopy("kv_b", (head, ("narrow", (1, 0, P), ()), ("permute", (1, 2, 0), ())), "W_UK_T", 0, (P, L, H),
+                     tuple(want_ukt.stride()), torch.bfloat16),
+    ]
+    params = {"W_UV": torch.zeros(V, H, L, dtype=torch.bfloat16, device="cuda"),
+              "W_UK_T": torch.zeros(P, L, H, dtype=torch.bfloat16, device="cuda")}
+    ptrs = {k: v.data_ptr() for k, v in params.items()}
+    for _ in range(2):  # a second cycle reuses the engine's scratch
+        execute_recorded_copies(gpu_engine, copies, {"kv_b": kv_b.cuda()}, params)
+    assert torch.equal(params["W_UV"].cpu().view(torch.int16), want_uv.view(torch.int16))
+    assert torch.equal(params["W_UK_T"].cpu().view(torch.int16), want_ukt.view(torch.int16))
+    assert {k: v.data_ptr() for k, v in params.items()} == ptrs  # written in place: graph-bound addresses are kept
