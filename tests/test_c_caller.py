@@ -25,8 +25,14 @@ def _setup(tmp_path, name, tp_rank):
 
 
 def _need_driver():
-    if not DRIVER.exists():
-        pytest.fail(f"{DRIVER} is not built: run `python -m modelexpress_amd.build --abi-driver`")
+    if DRIVER.exists():
+        return
+    try:  # normally prebuilt by `python -m modelexpress_amd.build --abi-driver`; one gcc call otherwise
+        from modelexpress_amd.build import build_abi_driver
+
+        build_abi_driver()
+    except Exception as e:  # noqa: BLE001
+        pytest.fail(f"{DRIVER} is not built and could not be built here: {e}")
 
 
 def test_c_caller_reports_a_missing_device_as_an_error(tmp_path):
