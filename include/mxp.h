@@ -229,7 +229,7 @@ typedef struct mxp_engine_options {
   int32_t device;          /* HIP device ordinal */
   int32_t ring_slots;      /* pinned host slots (each with a device bounce slot); 0 = default 32 */
   uint64_t slot_bytes;     /* bytes per slot; 0 = default 16 MiB */
-  int32_t reader_threads;  /* pread workers; 0 = default 8 */
+  int32_t reader_threads;  /* pread workers; 0 = min(16, host cores) */
   int32_t streams;         /* HIP streams for H2D + kernels; 0 = default 4 */
   uint32_t tile_bytes;     /* source bytes per workgroup, 1 KiB .. 128 KiB; 0 = 128 KiB */
   uint16_t nan_bits;       /* bf16 image of every NaN in the cast; 0 = default 0x7FC0 */
