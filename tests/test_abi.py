@@ -32,6 +32,36 @@ def test_library_exports_every_declared_symbol(mxp):
     assert mxp.lib().mxp_abi_version() == 1
 
 
+def test_rust_sys_generator_covers_the_header():
+    """include/gen_rust_sys.py (no Rust toolchain here, so the output is checked for coverage and
+    shape, not compiled): one ``pub fn`` per declared function with the same parameter count,
+    one ``#[repr(C)]`` struct per typedef with the same field count, every MXP_* constant."""
+    import importlib.util
+    import re
+
+    spec = importlib.util.spec_from_file_location("gen_rust_sys", ROOT / "include" / "gen_rust_sys.py")
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    header = (ROOT / "include" / "mxp.h").read_text()
+    out = gen.generate(header)
+    consts, opaque, structs, funcs = gen.parse(header)
+    assert sorted(name for _r, name, _p in funcs) == _declared()
+    for ret, name, params in funcs:
+        m = re.search(rf"pub fn {name}\((.*?)\)( -> [^;]+)?;", out)
+        assert m, name
+        assert (m.group(1).count(":") == len(params)) and (bool(m.group(2)) == (ret != "void")), name
+    for sname, fields in structs.items():
+        body = re.search(rf"pub struct {sname} \{{(.*?)\n\}}", out, flags=re.S).group(1)
+        assert body.count("pub ") == len(fields), sname
+    for o in opaque:
+        assert f"pub struct {o} {{ _private: [u8; 0] }}" in out
+    for name, _v in consts:
+        assert f"pub const {name}:" in out
+    assert "pub fn mxp_execute(engine: *mut mxp_engine, plan: *mut mxp_plan, dst_ptrs: *const *mut c_void, " \
+           "stats: *mut mxp_exec_stats) -> c_int;" in out
+    assert "pub shape: [i64; MXP_MAX_DIMS as usize]," in out and "pub const MXP_ERR_IO: i32 = -1;" in out
+
+
 def test_header_is_plain_c(tmp_path):
     src = tmp_path / "t.c"
     src.write_text('#include "mxp.h"\nint main(void){ mxp_engine_options o; (void)o; return MXP_OK; }\n')
