@@ -114,6 +114,8 @@ struct TransposeDesc {
   uint32_t vec_src, vec_dst;  // 16-byte accesses are aligned on that side
   uint32_t csum_bias;
   uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides kTransposeWaves)
+  uint32_t group_j;           // tiles along j that consecutive workgroups visit before stepping along i (>= 1)
+  uint32_t pad;
 };
 // Per-device set-up of the placement kernels (idempotent; also done lazily by launch_place).
 hipError_t configure_place_kernels();

@@ -32,8 +32,12 @@
 // picks waves_i from the extent of i.  The workgroup only exists to share an LDS allocation
 // and one checksum atomic.  Measured on 2-byte elements: 16384 x 16384 5.4 TB/s, sixteen
 // 4096 x 4096 matrices 6.2 TB/s (a plain copy of the same bytes through place_kernel: 5.7);
-// the rate falls as the destination pitch grows (65536 x 4096: 4.6-5.0 TB/s).  Visiting
-// tiles in compact super-tiles or in bands along j measured no better than plain order.
+// the rate depends on the two pitches.  When the destination pitch is the larger one, the host
+// asks for two wavefronts along i and bands of eight tiles along j (65536 x 4096: 5.3 against
+// 4.6 TB/s in plain order; 32768 x 8192: 5.5 against 4.8); otherwise eight wavefronts along i
+// and plain order are best (4096 x 65536: 5.8 TB/s).  Padding a power-of-two source pitch by
+// 384 bytes lifts 16384 x 16384 to 6.0 TB/s: the loss is in how the strided source lines fall
+// on the memory channels, which a caller controls and this kernel does not.
 #include "mxp_device.h"
 
 namespace mxp {
@@ -241,11 +245,16 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   Csum cs;
   // Linear tile index -> (batch, tile_j, tile_i), tile_i fastest.  Workgroup-uniform.
-  uint64_t b = blockIdx.x;
-  const uint32_t ti = (uint32_t)(b % d.tiles_i);
-  b /= d.tiles_i;
-  const uint32_t tj = (uint32_t)(b % d.tiles_j);
-  b /= d.tiles_j;
+  const uint64_t per_batch = (uint64_t)d.tiles_i * d.tiles_j;
+  uint64_t b = blockIdx.x / per_batch;
+  const uint32_t within = (uint32_t)(blockIdx.x % per_batch);
+  // Inside a batch, tiles are visited in bands of group_j tiles along j: with group_j > 1,
+  // consecutive workgroups read neighbouring lines of the same source rows.
+  const uint32_t gj = d.group_j;
+  const uint32_t band = within / (gj * d.tiles_i), in_band = within % (gj * d.tiles_i);
+  const uint32_t band_w = min(gj, d.tiles_j - band * gj);
+  const uint32_t tj = band * gj + in_band % band_w;
+  const uint32_t ti = in_band / band_w;
   uint64_t s_off = 0, d_off = 0;  // element offsets of the batch
 #pragma unroll
   for (int k = kMaxBatchDims - 1; k >= 0; --k) {
@@ -291,7 +300,9 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
                             uint32_t* sum_out, hipStream_t stream) {
   if (d.n_tiles == 0) return hipSuccess;
-  if (d.n_tiles > 0x7FFFFFFFull || d.waves_i == 0 || kWaves % d.waves_i) return hipErrorInvalidValue;
+  if (d.n_tiles > 0x7FFFFFFFull || d.waves_i == 0 || kWaves % d.waves_i || d.group_j == 0 ||
+      (uint64_t)d.tiles_i * d.tiles_j > 0x7FFFFFFFull || (uint64_t)d.tiles_i * d.group_j > 0x7FFFFFFFull)
+    return hipErrorInvalidValue;
   const dim3 grid((uint32_t)d.n_tiles), block(kThreads);
   const uint8_t* s = static_cast<const uint8_t*>(src);
   uint8_t* t = static_cast<uint8_t*>(dst);
