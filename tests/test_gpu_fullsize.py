@@ -81,3 +81,27 @@ def test_llama3_8b_rank_slice_full_size(oracle, oracle_c, tmp_path, mxp):
     assert eng.checksums(plan) == fused
     assert all(torch.equal(a, b) for a, b in zip(before, dst[:8]))
     eng.close()
+
+
+def test_buffer_beyond_4_gib_wraps_positions_like_the_reference(oracle_c, gpu_engine):
+    """A single buffer of 2^32 + 12,345 bytes: checksum positions wrap mod 2^32 exactly as the
+    reference's masked int64 weights do (tensor_utils.py:39-42), in the stand-alone checksum,
+    in the checksum fused into a copy, and in a digest (which carries no position)."""
+    n = (1 << 32) + 12345
+    dev = torch.empty(n, dtype=torch.uint8, device="cuda")
+    chunk = 1 << 28
+    host = np.empty(n, dtype=np.uint8)
+    for lo in range(0, n, chunk):  # bytes = (i * 131 + 7) mod 251, built piecewise on both sides
+        hi = min(n, lo + chunk)
+        idx = torch.arange(lo, hi, dtype=torch.int64, device="cuda")
+        dev[lo:hi] = ((idx * 131 + 7) % 251).to(torch.uint8)
+        del idx
+        host[lo:hi] = ((np.arange(lo, hi, dtype=np.int64) * 131 + 7) % 251).astype(np.uint8)
+    want = oracle_c.checksum32(host)
+    # the tail beyond 2^32 re-uses positions 0 .. 12,344: the total differs from a non-wrapping sum
+    assert want == format((int(oracle_c.checksum32(host[: 1 << 32]), 16) + int(oracle_c.checksum32(host[1 << 32:]), 16)) & 0xFFFFFFFF, "08x")
+    assert gpu_engine.checksum32([dev]) == [want]
+    out = torch.empty(n, dtype=torch.uint8, device="cuda")
+    assert gpu_engine.copy_batch([dev], [out], [n]) == [want]
+    assert torch.equal(out[-(1 << 20):], dev[-(1 << 20):]) and torch.equal(out[: 1 << 20], dev[: 1 << 20])
+    assert gpu_engine.digest([out]) == gpu_engine.digest([dev])
