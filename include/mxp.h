@@ -170,7 +170,9 @@ int mxp_plan_build(mxp_plan* plan);
 #define MXP_CAST_F16_F32 3
 #define MXP_CAST_F32_F16 4
 #define MXP_CAST_F8E4M3_BF16 5 /* exact; the .to(out_dtype) of engines/vllm/refit/receiver.py:258-261 */
-#define MXP_CAST_LAST MXP_CAST_F8E4M3_BF16
+#define MXP_CAST_F16_BF16 6 /* through fp32, as copy_ converts; NaN -> nan_bits */
+#define MXP_CAST_BF16_F16 7
+#define MXP_CAST_LAST MXP_CAST_BF16_F16
 
 #define MXP_WRITE_DIRECT 0
 #define MXP_WRITE_FUSED 1

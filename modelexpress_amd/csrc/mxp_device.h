@@ -20,8 +20,12 @@ enum SegOp : uint32_t {
   kOpCastBf16F32 = 3,  // src is bf16, dst is fp32 (exact)
   kOpCastF16F32 = 4,   // src is fp16, dst is fp32 (exact; NaNs made quiet)
   kOpCastF32F16 = 5,   // src is fp32, dst is fp16 (round to nearest even)
-  kOpCastF8E4M3Bf16 = 6  // src is fp8 e4m3fn, dst is bf16 (exact; NaN -> 0x7FC0)
+  kOpCastF8E4M3Bf16 = 6,  // src is fp8 e4m3fn, dst is bf16 (exact; NaN -> 0x7FC0)
+  kOpCastF16Bf16 = 7,  // src is fp16, dst is bf16 (through fp32, round to nearest even)
+  kOpCastBf16F16 = 8   // src is bf16, dst is fp16 (through fp32, round to nearest even)
 };
+// Conversions between two 16-bit formats: same size on both sides, values change.
+constexpr bool op_recodes16(uint32_t op) { return op == kOpCastF16Bf16 || op == kOpCastBf16F16; }
 constexpr bool op_narrows(uint32_t op) { return op == kOpCastF32Bf16 || op == kOpCastF32F16; }
 constexpr bool op_widens(uint32_t op) { return op == kOpCastBf16F32 || op == kOpCastF16F32 || op == kOpCastF8E4M3Bf16; }
 // Destination element size of a converting op (2 for a copy: only used for alignment rules).
@@ -35,10 +39,11 @@ constexpr uint64_t op_dst_bytes(uint32_t op, uint64_t src_bytes) {
   return op_narrows(op) ? src_bytes / 2 : op_widens(op) ? src_bytes * 2 : src_bytes;
 }
 // Public conversion code of a write record (0 none, 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32,
-// 4 fp32->fp16, 5 fp8-e4m3->bf16) -> segment operation.
+// 4 fp32->fp16, 5 fp8-e4m3->bf16, 6 fp16->bf16, 7 bf16->fp16) -> segment operation.
 constexpr uint32_t seg_op_of_cast(int cast) {
   return cast == 1 ? kOpCastF32Bf16 : cast == 2 ? kOpCastBf16F32 : cast == 3 ? kOpCastF16F32
-       : cast == 4 ? kOpCastF32F16 : cast == 5 ? kOpCastF8E4M3Bf16 : kOpCopy;
+       : cast == 4 ? kOpCastF32F16 : cast == 5 ? kOpCastF8E4M3Bf16 : cast == 6 ? kOpCastF16Bf16
+       : cast == 7 ? kOpCastBf16F16 : kOpCopy;
 }
 
 // 80 bytes, 16-byte aligned; the index is workgroup-uniform, so the whole record

@@ -103,6 +103,18 @@ __device__ __forceinline__ uint32_t f16_to_f32_bits(uint32_t h) {
   return ((h & 0x7C00u) == 0x7C00u && m) ? (((h & 0x8000u) << 16) | 0x7FC00000u | (m << 13)) : f;
 }
 
+// One 16-bit element of a conversion between the two 16-bit formats, through fp32 as torch's
+// copy_ does: fp16 -> bf16 (NaN -> nan_bits) or bf16 -> fp16.
+template <int OP>
+__device__ __forceinline__ uint32_t recode1(uint32_t h, uint32_t nan_bits) {
+  if constexpr (OP == kOpCastF16Bf16) return f32_to_bf16_bits(f16_to_f32_bits(h), nan_bits);
+  else return f32_to_f16_bits(h << 16);
+}
+template <int OP>
+__device__ __forceinline__ uint32_t recode2(uint32_t w, uint32_t nan_bits) {
+  return recode1<OP>(w & 0xFFFFu, nan_bits) | (recode1<OP>(w >> 16, nan_bits) << 16);
+}
+
 template <int OP>
 __device__ __forceinline__ uint32_t narrow1(uint32_t u, uint32_t nan_bits) {
   if constexpr (OP == kOpCastF32F16) return f32_to_f16_bits(u);
@@ -207,6 +219,9 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
     auto convert = [&](const In& a) -> Out {
       if constexpr (NARROW) return narrow4<OP>(a, nan_bits);
       else if constexpr (WIDEN) return widen4<OP>(a);
+      else if constexpr (op_recodes16(OP))
+        return make_uint4(recode2<OP>(a.x, nan_bits), recode2<OP>(a.y, nan_bits), recode2<OP>(a.z, nan_bits),
+                          recode2<OP>(a.w, nan_bits));
       else return a;
     };
     auto store = [&](uint32_t off, const Out& x) {
@@ -265,6 +280,15 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
         static_assert(UNIT == 2, "the element-wise cast path moves one element per lane");
         x = narrow1<OP>(*reinterpret_cast<const uint32_t*>(src + so), nan_bits);
         *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+      } else if constexpr (op_recodes16(OP)) {
+        if constexpr (UNIT == 4) {  // two elements per lane
+          x = recode2<OP>(*reinterpret_cast<const uint32_t*>(src + so), nan_bits);
+          *reinterpret_cast<uint32_t*>(dst + d_o) = x;
+        } else {
+          static_assert(UNIT == 2, "one element per lane");
+          x = recode1<OP>(*reinterpret_cast<const uint16_t*>(src + so), nan_bits);
+          *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+        }
       } else if constexpr (OP == kOpCastF8E4M3Bf16) {
         if constexpr (UNIT == 4) {  // two elements per lane
           const uint32_t w = *reinterpret_cast<const uint16_t*>(src + so);
@@ -333,6 +357,12 @@ __device__ __forceinline__ void place_body(
     case kOpCastF8E4M3Bf16 * 32u + 16u: run_tile<kOpCastF8E4M3Bf16, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF8E4M3Bf16 * 32u + 4u: run_tile<kOpCastF8E4M3Bf16, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF8E4M3Bf16 * 32u + 2u: run_tile<kOpCastF8E4M3Bf16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF16Bf16 * 32u + 16u: run_tile<kOpCastF16Bf16, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF16Bf16 * 32u + 4u: run_tile<kOpCastF16Bf16, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastF16Bf16 * 32u + 2u: run_tile<kOpCastF16Bf16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastBf16F16 * 32u + 16u: run_tile<kOpCastBf16F16, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastBf16F16 * 32u + 4u: run_tile<kOpCastBf16F16, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCastBf16F16 * 32u + 2u: run_tile<kOpCastBf16F16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 4u: run_tile<kOpChecksumOnly, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 1u: run_tile<kOpChecksumOnly, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;

@@ -53,6 +53,11 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
     else if (all_mult(4, 2)) unit = 4;
     else if (op_dst_elem(b.op) == 2 && all_mult(2, 1)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
+  } else if (op_recodes16(b.op)) {
+    if (all_mult(16, 16)) unit = 16;
+    else if (all_mult(4, 4)) unit = 4;
+    else if (all_mult(2, 2)) unit = 2;
+    else throw std::invalid_argument("cast box is not element aligned");
   } else {
     unit = all_mult(16, 16) ? 16 : all_mult(4, 4) ? 4 : 1;
   }
@@ -98,7 +103,7 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
                       std::vector<WorkItem>& work) {
   if (in.rows == 0 || in.row_bytes == 0) return;
   const uint32_t op = in.op;
-  const bool is_cast = op_narrows(op) || op_widens(op);
+  const bool is_cast = op_narrows(op) || op_widens(op) || op_recodes16(op);
   BoxCopy b = in;
   // Rows that abut in both layouts are one contiguous run.
   if (b.rows > 1 && b.src_pitch == op_src_bytes(op, b.row_bytes) && b.dst_pitch == b.row_bytes) {

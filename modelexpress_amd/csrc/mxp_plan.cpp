@@ -289,6 +289,8 @@ struct Planner {
         else if (t.dtype == MXP_DTYPE_F16 && p.dtype == MXP_DTYPE_F32) cast = MXP_CAST_F16_F32;
         else if (t.dtype == MXP_DTYPE_F32 && p.dtype == MXP_DTYPE_F16) cast = MXP_CAST_F32_F16;
         else if (t.dtype == MXP_DTYPE_F8_E4M3 && p.dtype == MXP_DTYPE_BF16) cast = MXP_CAST_F8E4M3_BF16;
+        else if (t.dtype == MXP_DTYPE_F16 && p.dtype == MXP_DTYPE_BF16) cast = MXP_CAST_F16_BF16;
+        else if (t.dtype == MXP_DTYPE_BF16 && p.dtype == MXP_DTYPE_F16) cast = MXP_CAST_BF16_F16;
       }
       if (!cast)
         throw Error(MXP_ERR_UNSUPPORTED, "tensor '" + t.name + "' is " + mxp_dtype_name(t.dtype) +

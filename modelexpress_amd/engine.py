@@ -51,7 +51,8 @@ class VirtualTensor:
 
 
 # MXP_CAST_* of include/mxp.h
-CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4, ("F8_E4M3", "BF16"): 5}
+CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4, ("F8_E4M3", "BF16"): 5,
+              ("F16", "BF16"): 6, ("BF16", "F16"): 7}
 
 
 @dataclass(frozen=True)

@@ -62,7 +62,8 @@ class OracleC:
     def cast(self, code: int, bits: np.ndarray, nan_bits: int = 0x7FC0) -> np.ndarray:
         """Conversion ``code`` (1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16, 5 fp8-e4m3->bf16) on bit patterns."""
         src_t, dst_t = {1: (np.uint32, np.uint16), 2: (np.uint16, np.uint32), 3: (np.uint16, np.uint32),
-                        4: (np.uint32, np.uint16), 5: (np.uint8, np.uint16)}[code]
+                        4: (np.uint32, np.uint16), 5: (np.uint8, np.uint16), 6: (np.uint16, np.uint16),
+                        7: (np.uint16, np.uint16)}[code]
         src = np.ascontiguousarray(bits, dtype=src_t)
         dst = np.empty(src.shape, dtype=dst_t)
         self.h.orc_cast(code, src.ctypes.data, dst.ctypes.data, src.size, nan_bits)

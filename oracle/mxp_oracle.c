@@ -70,7 +70,8 @@ void orc_cast_f32_bf16(const uint32_t* src, uint16_t* dst, uint64_t n, uint16_t 
 }
 
 /* The other conversions of the same copy_ (receive side: refit/reshard/receiver.py:962-969).
- * Codes: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16, 5 fp8-e4m3 -> bf16. */
+ * Codes: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16, 5 fp8-e4m3 -> bf16,
+ * 6 fp16->bf16 and 7 bf16->fp16 (both through fp32). */
 static inline uint16_t f8e4m3_to_bf16_bits(uint8_t c) {
   const uint16_t sign = (uint16_t)((c & 0x80u) << 8), e = (c >> 3) & 0xFu, m = c & 7u;
   if (e == 15u && m == 7u) return 0x7FC0u;
@@ -115,6 +116,8 @@ void orc_cast(uint32_t code, const void* src, void* dst, uint64_t n, uint16_t na
     case 3: for (i = 0; i < n; ++i) ((uint32_t*)dst)[i] = f16_to_f32_bits(((const uint16_t*)src)[i]); break;
     case 4: for (i = 0; i < n; ++i) ((uint16_t*)dst)[i] = f32_to_f16_bits(((const uint32_t*)src)[i]); break;
     case 5: for (i = 0; i < n; ++i) ((uint16_t*)dst)[i] = f8e4m3_to_bf16_bits(((const uint8_t*)src)[i]); break;
+    case 6: for (i = 0; i < n; ++i) ((uint16_t*)dst)[i] = bf16_bits(f16_to_f32_bits(((const uint16_t*)src)[i]), nan_bits); break;
+    case 7: for (i = 0; i < n; ++i) ((uint16_t*)dst)[i] = f32_to_f16_bits((uint32_t)((const uint16_t*)src)[i] << 16); break;
     default: break;
   }
 }

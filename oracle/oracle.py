@@ -204,7 +204,9 @@ def cast_tensor_f32_bf16(t: OTensor, nan_bits: int = 0x7FC0) -> OTensor:
 # the product's write records: 1 fp32->bf16, 2 bf16->fp32, 3 fp16->fp32, 4 fp32->fp16,
 # 5 fp8-e4m3 -> bf16 (the ``.to(out_dtype)`` of the MLA absorbed weights when ``kv_b_proj`` is
 # stored in fp8: engines/vllm/refit/receiver.py:258-261).
-CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4, ("F8_E4M3", "BF16"): 5}
+# 6 fp16 -> bf16 and 7 bf16 -> fp16 go through fp32, as torch's copy_ does between the two 16-bit formats.
+CAST_CODES = {("F32", "BF16"): 1, ("BF16", "F32"): 2, ("F16", "F32"): 3, ("F32", "F16"): 4, ("F8_E4M3", "BF16"): 5,
+              ("F16", "BF16"): 6, ("BF16", "F16"): 7}
 
 
 def cast_bf16_f32_bits(u16: np.ndarray) -> np.ndarray:
@@ -281,6 +283,12 @@ def cast_tensor(t: OTensor, dst_dtype: str, nan_bits: int = 0x7FC0) -> OTensor:
         return OTensor.from_array(cast_f32_f16_bits(src.view("<u4").reshape(t.shape)).astype("<u2"), "F16")
     if code == 5:
         return OTensor.from_array(cast_f8e4m3_bf16_bits(src.view("u1").reshape(t.shape)).astype("<u2"), "BF16")
+    if code == 6:
+        u = cast_f32_bf16_bits(cast_f16_f32_bits(src.view("<u2").reshape(t.shape)), nan_bits)
+        return OTensor.from_array(u.astype("<u2"), "BF16")
+    if code == 7:
+        u = cast_f32_f16_bits(cast_bf16_f32_bits(src.view("<u2").reshape(t.shape)))
+        return OTensor.from_array(u.astype("<u2"), "F16")
     fn = cast_bf16_f32_bits if code == 2 else cast_f16_f32_bits
     return OTensor.from_array(fn(src.view("<u2").reshape(t.shape)).astype("<u4"), "F32")
 

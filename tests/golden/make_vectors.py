@@ -93,6 +93,10 @@ def main():
     g = h.view(torch.bfloat16).to(torch.float32).view(torch.int32).tolist()
     vec["cast_f16_f32"] = {"f16_bits": [halves[i] for i in not_nan16], "f32_bits": [f[i] & M32 for i in not_nan16]}
     vec["cast_bf16_f32"] = {"bf16_bits": [halves[i] for i in not_nan_bf], "f32_bits": [g[i] & M32 for i in not_nan_bf]}
+    vec["cast_f16_bf16"] = {"f16_bits": [halves[i] for i in not_nan16],
+                            "bf16_bits": [h.view(torch.float16).to(torch.bfloat16).view(torch.int16).tolist()[i] & 0xFFFF for i in not_nan16]}
+    vec["cast_bf16_f16"] = {"bf16_bits": [halves[i] for i in not_nan_bf],
+                            "f16_bits": [h.view(torch.bfloat16).to(torch.float16).view(torch.int16).tolist()[i] & 0xFFFF for i in not_nan_bf]}
     codes = torch.arange(256, dtype=torch.uint8)
     vec["cast_f8e4m3_bf16"] = {"f8_bits": list(range(256)),
                                "bf16_bits": [v & 0xFFFF for v in codes.view(torch.float8_e4m3fn).to(torch.bfloat16).view(torch.int16).tolist()]}

@@ -51,7 +51,7 @@ def apply_plan_numpy(ck: Checkpoint, plan: PlacementPlan, nan_bits=0x7FC0) -> di
         src = files[t.file_index][t.file_offset : t.file_offset + t.nbytes]
         dst = out[w.param]
         src_row = {0: w.row_bytes, 1: w.row_bytes * 2, 4: w.row_bytes * 2, 2: w.row_bytes // 2, 3: w.row_bytes // 2,
-                   5: w.row_bytes // 2}[w.cast]
+                   5: w.row_bytes // 2, 6: w.row_bytes, 7: w.row_bytes}[w.cast]
         for r in range(w.rows):
             s = src[w.src_offset + r * w.src_pitch : w.src_offset + r * w.src_pitch + src_row]
             if w.cast == 1:
@@ -61,10 +61,11 @@ def apply_plan_numpy(ck: Checkpoint, plan: PlacementPlan, nan_bits=0x7FC0) -> di
                 s = b.view(np.uint8)
             elif w.cast == 2:
                 s = (s.view("<u2").astype(np.uint32) << 16).view(np.uint8)
-            elif w.cast in (3, 4, 5):  # torch is the library the reference converts with
+            elif w.cast in (3, 4, 5, 6, 7):  # torch is the library the reference converts with
                 import torch
                 src_t, dst_t = {3: (torch.float16, torch.float32), 4: (torch.float32, torch.float16),
-                                5: (torch.float8_e4m3fn, torch.bfloat16)}[w.cast]
+                                5: (torch.float8_e4m3fn, torch.bfloat16), 6: (torch.float16, torch.bfloat16),
+                                7: (torch.bfloat16, torch.float16)}[w.cast]
                 s = torch.from_numpy(s.copy()).view(src_t).to(dst_t).view(torch.uint8).numpy()
             dst[w.dst_offset + r * w.dst_pitch : w.dst_offset + r * w.dst_pitch + w.row_bytes] = s
     return out
@@ -90,6 +91,8 @@ def tiny_layouts():
                                 4, 1, 2, {"dtype": "BF16", "edge_cases": models.NORMAL_EDGE_DENSE, "param_dtype": "F32"}),
         "llama_f16_into_f32": (models.Llama(layers=1, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
                                2, 1, 1, {"dtype": "F16", "edge_cases": models.NORMAL_EDGE_DENSE, "param_dtype": "F32"}),
+        "llama_f16_into_bf16": (models.Llama(layers=1, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
+                                2, 1, 2, {"dtype": "F16", "param_dtype": "BF16"}),
         "llama_f32_into_f16": (models.Llama(layers=1, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_dim=8, vocab=256),
                                2, 1, 2, {"dtype": "F32", "edge_cases": models.NORMAL_EDGE_DENSE, "param_dtype": "F16"}),
         "gpt2": (models.Gpt2(layers=2, hidden=32, ffn=64, vocab=97, positions=16), 1, 1, 1, {}),

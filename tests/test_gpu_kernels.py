@@ -86,7 +86,8 @@ def test_cast_f32_bf16_matches_oracle(gpu_engine, oracle, oracle_c):
         assert int(d[src.size * 2:].sum()) == 0  # nothing written past the end
 
 
-@pytest.mark.parametrize("src_dtype,dst_dtype", [("BF16", "F32"), ("F16", "F32"), ("F32", "F16"), ("F8_E4M3", "BF16")])
+@pytest.mark.parametrize("src_dtype,dst_dtype", [("BF16", "F32"), ("F16", "F32"), ("F32", "F16"), ("F8_E4M3", "BF16"),
+                                                 ("F16", "BF16"), ("BF16", "F16")])
 def test_cast_pairs_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dtype):
     """The other conversions of dest.copy_(src) (refit/reshard/receiver.py:962-969): every 16-bit
     pattern for the widening ones, every rounding class for fp32 -> fp16, odd sizes and offsets."""
@@ -101,6 +102,13 @@ def test_cast_pairs_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dt
     elif src_dtype == "F8_E4M3":
         full = np.concatenate([np.arange(256, dtype=np.uint8), rng.integers(0, 256, (1 << 20) + 5, dtype=np.uint8)])
         fn, se, de = oracle.cast_f8e4m3_bf16_bits, 1, 2
+    elif dst_dtype != "F32":  # between the two 16-bit formats, through fp32
+        full = np.concatenate([np.arange(1 << 16, dtype=np.uint16), rng.integers(0, 1 << 16, (1 << 20) + 5, dtype=np.uint16)])
+        if src_dtype == "F16":
+            fn = lambda u: oracle.cast_f32_bf16_bits(oracle.cast_f16_f32_bits(u))  # noqa: E731
+        else:
+            fn = lambda u: oracle.cast_f32_f16_bits(oracle.cast_bf16_f32_bits(u))  # noqa: E731
+        se, de = 2, 2
     else:
         full = np.concatenate([np.arange(1 << 16, dtype=np.uint16), rng.integers(0, 1 << 16, (1 << 20) + 5, dtype=np.uint16)])
         fn, se, de = (oracle.cast_bf16_f32_bits if src_dtype == "BF16" else oracle.cast_f16_f32_bits), 2, 4
@@ -116,7 +124,7 @@ def test_cast_pairs_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dt
         assert csum == oracle_c.checksum32(want.view(np.uint8))
         assert int(d[n * de:].sum()) == 0  # nothing written past the end
     with pytest.raises(ValueError):
-        gpu_engine.cast(dev, dev, 1, "BF16", "F16")
+        gpu_engine.cast(dev, dev, 1, "BF16", "I32")
 
 
 def test_cast_nan_image_is_a_parameter(mxp, oracle):
@@ -295,7 +303,7 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
     want = np.full(out_size, 0xEE, dtype=np.uint8)
     boxes, sums_want, cursor = [], [], 0
     for g in range(int(rng.integers(1, 9))):
-        cast = int(rng.choice([0, 0, 0, 1, 2, 3, 4, 5]))  # MXP_CAST_* code
+        cast = int(rng.choice([0, 0, 0, 1, 2, 3, 4, 5, 6, 7]))  # MXP_CAST_* code
         narrow, widen = cast in (1, 4), cast in (2, 3, 5)
         align = int(rng.choice([1, 2, 4, 8, 16])) if not cast else int(rng.choice([4, 8, 16]) if cast in (2, 3) else rng.choice([2, 4, 8, 16]))
         rows = int(rng.choice([1, 1, 2, 7, 64, 513, 3000]))
@@ -307,7 +315,7 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
         src_pitch = src_row + int(rng.integers(0, 5)) * src_align
         if rows * max(dst_pitch, 1) > (1 << 20) or rows * src_pitch > (4 << 20):
             rows = max(1, min((1 << 20) // dst_pitch, (4 << 20) // src_pitch))
-        src_off = int(rng.integers(0, 64)) * (4 if narrow else 2 if cast in (2, 3) else 1)
+        src_off = int(rng.integers(0, 64)) * (4 if narrow else 2 if cast in (2, 3, 6, 7) else 1)
         src_off -= src_off % (min(src_align, 16) if cast else min(align, 16))
         dst_off = (cursor + 15) // 16 * 16
         if rows == 1 and not cast and align < 16 and rng.integers(0, 2):
@@ -325,6 +333,10 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
                 s = oracle.cast_f16_f32_bits(s.view(np.uint16)).view(np.uint8)
             elif cast == 5:
                 s = oracle.cast_f8e4m3_bf16_bits(s).view(np.uint8)
+            elif cast == 6:
+                s = oracle.cast_f32_bf16_bits(oracle.cast_f16_f32_bits(s.view(np.uint16))).view(np.uint8)
+            elif cast == 7:
+                s = oracle.cast_f32_f16_bits(oracle.cast_bf16_f32_bits(s.view(np.uint16))).view(np.uint8)
             want[dst_off + r * dst_pitch: dst_off + r * dst_pitch + row_bytes] = s
             csum += int(oracle_c.checksum32(s, first_index=1000 + r * dst_pitch), 16)
         sums_want.append(format(csum & 0xFFFFFFFF, "08x"))

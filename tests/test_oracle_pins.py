@@ -240,6 +240,20 @@ def test_fp8_e4m3_to_bf16_matches_torch_on_every_code(oracle, oracle_c):
     assert oracle.cast_f8e4m3_bf16_bits(hv).tolist() == [0x3F80, 0xC3E0, 0x3B00, 0x3C80, 0x7FC0, 0x7FC0]
 
 
+def test_fp16_bf16_recoding_matches_torch_on_every_pattern(oracle, oracle_c):
+    # destination.copy_(source) between the two 16-bit formats (installer.py:419-424) goes through fp32
+    h = np.arange(1 << 16, dtype=np.uint16)
+    OT = oracle.OTensor
+    a = oracle.cast_tensor(OT.from_array(h, "F16"), "BF16").data.reshape(-1).view("<u2")
+    b = oracle.cast_tensor(OT.from_array(h, "BF16"), "F16").data.reshape(-1).view("<u2")
+    assert np.array_equal(a, _torch_convert(h, "F16", "BF16"))  # torch's NaN image here is 0x7FC0, the default
+    assert np.array_equal(b, _torch_convert(h, "BF16", "F16"))
+    assert np.array_equal(oracle_c.cast(6, h), a) and np.array_equal(oracle_c.cast(7, h), b)
+    # hand values: fp16 1.0 -> bf16 1.0; fp16 65504 -> bf16 0x4780 (rounds up to 65536); bf16 1e5 -> fp16 inf
+    assert oracle.cast_tensor(OT.from_array(np.array([0x3C00, 0x7BFF], dtype=np.uint16), "F16"), "BF16").data.reshape(-1).view("<u2").tolist() == [0x3F80, 0x4780]
+    assert oracle.cast_tensor(OT.from_array(np.array([0x47C3], dtype=np.uint16), "BF16"), "F16").data.reshape(-1).view("<u2").tolist() == [0x7C00]
+
+
 def test_f32_to_f16_matches_torch_and_numpy(oracle, oracle_c):
     hi = np.arange(1 << 16, dtype=np.uint32) << 16
     lows = np.array([0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF, 0x2000, 0x2FFF, 0x3000, 0x7FFF, 0x8000, 0x8001, 0xFFFF],

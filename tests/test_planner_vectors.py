@@ -293,4 +293,8 @@ def test_widening_and_half_conversions_are_planned(mxp, oracle, tmp_path):
     assert apply_plan_numpy(Checkpoint(str(tmp_path)), plan8)["d.weight"].tobytes() == \
         w[:, 4:].to(torch.float8_e4m3fn).to(torch.bfloat16).contiguous().view(torch.uint8).numpy().tobytes()
     with pytest.raises(MxpError, match="no conversion"):  # pairs outside the table stay refused
-        PlacementPlan(ck, [ParamSpec("a.weight", "F16", (4, 8))], allow_cast=True, allow_uncovered=True, allow_unmapped=True)
+        PlacementPlan(ck, [ParamSpec("a.weight", "F8_E4M3", (4, 8))], allow_cast=True, allow_uncovered=True, allow_unmapped=True)
+    # the two 16-bit formats convert into each other through fp32 (copy_ semantics)
+    p16 = PlacementPlan(ck, [ParamSpec("a.weight", "F16", (4, 8)), ParamSpec("b.weight", "BF16", (4, 8))], allow_cast=True,
+                        allow_unmapped=True)
+    assert {x.tensor: (x.cast, x.row_bytes, x.src_pitch) for x in p16.writes()} == {"a.weight": (7, 64, 64), "b.weight": (6, 64, 64)}

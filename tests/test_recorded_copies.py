@@ -54,7 +54,7 @@ CASES = [
 @pytest.mark.parametrize("case", range(len(CASES)))
 @pytest.mark.parametrize("dtypes", [(torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32),
                                     (torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.uint8, torch.uint8),
-                                    (torch.float8_e4m3fn, torch.bfloat16)])
+                                    (torch.float8_e4m3fn, torch.bfloat16), (torch.float16, torch.bfloat16)])
 def test_recorded_copies_match_torch(gpu_engine, case, dtypes):
     src_shape, chain, param_shape, dest_offset, dest_stride = CASES[case]
     src_dt, dst_dt = dtypes
