@@ -81,3 +81,20 @@ def test_env_registry_reads_live(monkeypatch):
         pass
     else:
         raise AssertionError("unknown variables must raise")
+
+
+def test_product_never_imports_the_oracle_or_scratch_files():
+    """The oracle is test infrastructure: nothing under modelexpress_amd/ or include/ may import,
+    load or name it, and no committed file may reach into the scratch directory."""
+    import re
+    from pathlib import Path
+
+    root = Path(__file__).resolve().parent.parent
+    for path in list((root / "modelexpress_amd").rglob("*.py")) + list((root / "modelexpress_amd" / "csrc").iterdir()) + \
+            list((root / "include").iterdir()):
+        if path.is_file() and path.suffix in (".py", ".cpp", ".hpp", ".h", ".hip"):
+            text = path.read_text()
+            assert not re.search(r"\boracle\b", text), f"{path} mentions the oracle"
+            assert "_work/" not in text, f"{path} names the scratch directory"
+    for path in [root / "bench.py", root / "__graft_entry__.py"] + list((root / "tests").rglob("*.py")) + list((root / "oracle").glob("*.py")):
+        assert "_work/" not in path.read_text() or path.name == "test_configs.py", f"{path} names the scratch directory"
