@@ -95,7 +95,7 @@ def main() -> int:
         print("bench.py: no GPU visible; the placement path has no CPU fallback", file=sys.stderr)
         return 1
     from modelexpress_amd import _lib, models, synth
-    from modelexpress_amd.engine import Checkpoint, PlacementEngine, PlacementPlan
+    from modelexpress_amd.engine import CAST_CODES, Checkpoint, PlacementEngine, PlacementPlan
 
     _lib.lib()  # fail loudly if the HIP library is missing
     layout, tp, ep, n_shards, ck_dtype, ck_kind = models.baseline_config(args.config)
@@ -278,6 +278,35 @@ def main() -> int:
                 ops[f"cast_{src_dt.lower()}_{dst_dt.lower()}"] = {
                     "elements": n_el, "ms": round(ms, 4), "gbps_algorithmic": round(6 * n_el / ms / 1e6, 1),
                     "frac_of_hbm_peak": round(6 * n_el / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                del a, b
+            # transposes that convert on the way: an fp32 master weight written transposed as bf16, a bf16
+            # weight widened, and the MLA W_UK_T shape out of an fp8 kv_b_proj
+            for label, src_dt, dst_dt, shape, perm in (
+                    ("transpose_f32_bf16_16384x16384", "F32", "BF16", (16384, 16384), (1, 0)),
+                    ("transpose_bf16_f32_16384x16384", "BF16", "F32", (16384, 16384), (1, 0)),
+                    ("mla_w_uk_t_f8_bf16_128x128x512", "F8_E4M3", "BF16", (128, 128, 512), (1, 2, 0))):
+                se = {"F32": 4, "BF16": 2, "F8_E4M3": 1}[src_dt]
+                de = {"F32": 4, "BF16": 2}[dst_dt]
+                n_el = 1
+                for v in shape:
+                    n_el *= v
+                st = [1] * len(shape)
+                for d in range(len(shape) - 2, -1, -1):
+                    st[d] = st[d + 1] * shape[d + 1]
+                v_shape, v_strides = [shape[q] for q in perm], [st[q] for q in perm]
+                a = torch.empty(n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256)
+                b = torch.empty(n_el * de, dtype=torch.uint8, device="cuda")
+                code = CAST_CODES[(src_dt, dst_dt)]
+                eng.copy_view(a, b, v_shape, de, src_strides=v_strides, cast=code, checksum=False)
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ev0.record()
+                for _ in range(10):
+                    eng.copy_view(a, b, v_shape, de, src_strides=v_strides, cast=code, checksum=False)
+                ev1.record()
+                torch.cuda.synchronize()
+                ms = ev0.elapsed_time(ev1) / 10
+                ops[label] = {"elements": n_el, "ms": round(ms, 4), "gbps_algorithmic": round((se + de) * n_el / ms / 1e6, 1),
+                              "frac_of_hbm_peak": round((se + de) * n_el / ms / 1e6 / HBM_PEAK_GBPS, 4)}
                 del a, b
             out["ops"] = ops
 

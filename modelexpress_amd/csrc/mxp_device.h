@@ -101,12 +101,13 @@ hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_
 // Batched 2-D transpose (mxp_permute.hip).  "i" = the destination's innermost dimension,
 // "j" = the source's innermost dimension; strides are in elements.
 constexpr int kMaxBatchDims = 6;
-// Transpose tiling.  One wavefront owns a sub-tile of 64 (128 for 1-byte elements) source rows
-// (i) x 128 source bytes (j); a workgroup is kTransposeWaves wavefronts arranged
-// waves_i x (kTransposeWaves / waves_i), chosen per call from the extents.
+// Transpose tiling.  One wavefront owns a sub-tile of 64 (128 for 1-byte destination elements)
+// source rows (i) x 128 source bytes (j); a workgroup is `waves` <= kTransposeWaves wavefronts
+// arranged waves_i x (waves / waves_i), chosen per call from the extents.
 constexpr int kTransposeWaves = 8;
-constexpr int transpose_sub_rows(int elem_size) { return elem_size == 1 ? 128 : 64; }
-constexpr int transpose_sub_cols(int elem_size) { return 128 / elem_size; }
+constexpr int kChipCus = 256;  // compute units of the one chip this library is written for
+constexpr int transpose_sub_rows(int dst_elem_size) { return dst_elem_size == 1 ? 128 : 64; }
+constexpr int transpose_sub_cols(int src_elem_size) { return 128 / src_elem_size; }
 struct TransposeDesc {
   uint64_t ni, nj;   // extents
   uint64_t si;       // source stride of i (source stride of j is 1)
@@ -118,14 +119,16 @@ struct TransposeDesc {
   uint64_t batch_dstride[kMaxBatchDims];
   uint32_t vec_src, vec_dst;  // 16-byte accesses are aligned on that side
   uint32_t csum_bias;
-  uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides kTransposeWaves)
+  uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides waves)
   uint32_t group_j;           // tiles along j that consecutive workgroups visit before stepping along i (>= 1)
-  uint32_t pad;
+  uint32_t waves;             // wavefronts of a workgroup (1, 2, 4 or 8)
 };
 // Per-device set-up of the placement kernels (idempotent; also done lazily by launch_place).
 hipError_t configure_place_kernels();
-hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
-                            uint32_t* sum_out, hipStream_t stream);
+// `elem_size` is the source element; `op` is kOpCopy or a conversion whose source element it is
+// (dj, batch_dstride and the checksum positions then count destination elements / bytes).
+hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size, uint32_t op,
+                            uint32_t nan_bits, uint32_t* sum_out, hipStream_t stream);
 
 // Synthetic-checkpoint generator (mxp_synth.hip), same arithmetic on host and device.
 enum SynthKind : uint32_t {

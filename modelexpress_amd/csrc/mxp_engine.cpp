@@ -110,7 +110,6 @@ struct mxp_engine {
   uint8_t* desc_host = nullptr;  // pinned
   size_t desc_host_cap = 0;
   DevBuf<uint8_t> desc_dev;
-  DevBuf<uint8_t> view_tmp;  // scratch of converting transposes
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
   hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
   bool arena_recorded = false;
@@ -917,22 +916,20 @@ struct TransposeJob {
   const void* src;
   void* dst;
   TransposeDesc td;
-  int elem_size;
+  int elem_size;  // source element
+  uint32_t op;    // kOpCopy, or the conversion applied on the way
 };
 
 enum ViewKind {
-  kViewEmpty,          // nothing to move
-  kViewBoxes,          // row / element boxes appended to `boxes`
-  kViewTranspose,      // `tr` holds the whole copy
-  kViewNeedsScratch,   // a converting transpose: call again with `scratch` of total * source-element bytes
-  kViewTransposeBoxes  // `tr` transposes into `scratch` at the source dtype, then `boxes` convert rows out of it
+  kViewEmpty,     // nothing to move
+  kViewBoxes,     // row boxes appended to `boxes`
+  kViewTranspose  // `tr` filled in: one launch of the transpose kernel, converting on the way if asked
 };
 
 // Lowers one view copy.  Boxes are appended to `boxes` with their base pointers in `srcs` / `dsts`.
 ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
                     std::vector<uint64_t> ds, int elem_size, int cast, uint32_t csum_slot, std::vector<BoxCopy>& boxes,
-                    std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, void* scratch,
-                    const char* what) {
+                    std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, const char* what) {
   const uint32_t op = seg_op_of_cast(cast);
   const uint64_t es = (uint64_t)elem_size;          // destination element
   const uint64_t es_s = op_src_bytes(op, es);       // source element
@@ -972,11 +969,11 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
   const bool dst_inner = ds[nd - 1] == 1 || total == 1;
   const bool transposed = dst_inner && ss[nd - 1] != 1 && total != 1 && c >= 0 && nd - 2 <= (size_t)kMaxBatchDims;
 
-  // Row boxes from a source laid out with strides `s` at `sp`: whole innermost rows when both
-  // sides are contiguous there, else one element per row.
-  auto emit_boxes = [&](const void* sp, const std::vector<uint64_t>& s_in) {
-    const bool rows_ok = dst_inner && (s_in[nd - 1] == 1 || total == 1);
-    std::vector<uint64_t> n = size, s = s_in, d = ds;
+  // Row boxes: whole innermost rows when both sides are contiguous there, else one element per row.
+  auto emit_boxes = [&] {
+    const void* sp = src;
+    const bool rows_ok = dst_inner && (ss[nd - 1] == 1 || total == 1);
+    std::vector<uint64_t> n = size, s = ss, d = ds;
     if (!rows_ok) { n.push_back(1); s.push_back(1); d.push_back(1); }  // a virtual innermost dimension of one element
     const size_t m = n.size();
     const void* sb;
@@ -1017,32 +1014,43 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
     }
   };
 
-  // Transpose of `eb`-byte elements into `dp` laid out with strides `d_in` (innermost 1):
-  // i = destination innermost, j = the source's unit-stride dimension.
-  auto make_transpose = [&](void* dp, const std::vector<uint64_t>& d_in, uint64_t eb) {
+  // Transpose: i = destination innermost, j = the source's unit-stride dimension.  The tile
+  // shape follows the source element (`eb`); destination alignment follows its own (`es`).
+  auto make_transpose = [&] {
+    void* dp = dst;
+    const std::vector<uint64_t>& d_in = ds;
+    const uint64_t eb = es_s;
     TransposeDesc td{};
     td.ni = size[nd - 1];
     td.si = ss[nd - 1];
     td.nj = size[c];
     td.dj = d_in[c];
+    uint64_t batches = 1;
+    for (int d = (int)nd - 2; d >= 0; --d)
+      if (d != c) batches *= size[d];
     // Workgroup shape: as many wavefronts along i (long destination runs) as the extent can
-    // use, the rest along j.
-    uint32_t waves_i = 1;
-    while (waves_i < (uint32_t)kTransposeWaves && (uint64_t)waves_i * transpose_sub_rows((int)eb) < td.ni) waves_i *= 2;
-    // Larger destination pitch than source pitch: short, wide workgroups visited in bands along j
-    // (measured +15% on 65536 x 4096 and 32768 x 8192); otherwise long destination runs, plain order.
-    td.group_j = 1;
-    if (td.dj > td.si) {
-      waves_i = std::min(waves_i, 2u);
-      td.group_j = 8;
+    // use, the rest along j; fewer wavefronts per workgroup while the launch would leave
+    // compute units without one.
+    const uint64_t sub_i = transpose_sub_rows((int)es), sub_j = transpose_sub_cols((int)eb);
+    for (uint32_t waves = (uint32_t)kTransposeWaves;; waves /= 2) {
+      uint32_t waves_i = 1;
+      while (waves_i < waves && (uint64_t)waves_i * sub_i < td.ni) waves_i *= 2;
+      // Larger destination pitch than source pitch: short, wide workgroups visited in bands along j
+      // (measured +15% on 65536 x 4096 and 32768 x 8192); otherwise long destination runs, plain order.
+      td.group_j = 1;
+      if (td.dj > td.si) {
+        waves_i = std::min(waves_i, 2u);
+        td.group_j = 8;
+      }
+      td.waves = waves;
+      td.waves_i = waves_i;
+      const uint64_t tile_i = waves_i * sub_i, tile_j = (waves / waves_i) * sub_j;
+      td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
+      td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
+      if (waves == 1 || batches * td.tiles_i * td.tiles_j >= 2ull * kChipCus) break;
     }
-    td.waves_i = waves_i;
-    const uint64_t tile_i = (uint64_t)waves_i * transpose_sub_rows((int)eb);
-    const uint64_t tile_j = (uint64_t)(kTransposeWaves / waves_i) * transpose_sub_cols((int)eb);
-    td.tiles_i = (uint32_t)((td.ni + tile_i - 1) / tile_i);
-    td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
     bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * eb) % 16 == 0;
-    bool vd = (reinterpret_cast<uintptr_t>(dp) % 16 == 0) && (td.dj * eb) % 16 == 0;
+    bool vd = (reinterpret_cast<uintptr_t>(dp) % 16 == 0) && (td.dj * es) % 16 == 0;
     int k = kMaxBatchDims - 1;
     for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
     for (int d = (int)nd - 2; d >= 0; --d) {
@@ -1051,32 +1059,22 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
       td.batch_sstride[k] = ss[d];
       td.batch_dstride[k] = d_in[d];
       vs = vs && (ss[d] * eb) % 16 == 0;
-      vd = vd && (d_in[d] * eb) % 16 == 0;
+      vd = vd && (d_in[d] * es) % 16 == 0;
       --k;
     }
     td.vec_src = vs;
     td.vec_dst = vd;
     td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
     for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
-    tr = TransposeJob{src, dp, td, (int)eb};
+    tr = TransposeJob{src, dp, td, (int)eb, op};
   };
 
   if (!transposed) {
-    emit_boxes(src, ss);
+    emit_boxes();
     return kViewBoxes;
   }
-  if (op == kOpCopy) {
-    make_transpose(dst, ds, es);
-    return kViewTranspose;
-  }
-  // A converting transpose: transpose at the source dtype into contiguous scratch (dimensions in
-  // destination order), then convert whole rows out of it.
-  if (!scratch) return kViewNeedsScratch;
-  std::vector<uint64_t> ts(nd, 1);
-  for (int d = (int)nd - 2; d >= 0; --d) ts[d] = ts[d + 1] * size[d + 1];
-  make_transpose(scratch, ts, es_s);
-  emit_boxes(scratch, ts);
-  return kViewTransposeBoxes;
+  make_transpose();
+  return kViewTranspose;
 }
 
 void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hipStream_t stream) {
@@ -1087,27 +1085,13 @@ void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hip
     sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
     HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
   }
-  HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, sum_dev, stream));
+  HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, e.opt.nan_bits, sum_dev, stream));
   if (checksum) {
     HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
     std::memcpy(checksum, e.desc_host, 4);
     release_arena(e, stream);
   }
-}
-
-// Scratch for converting transposes; grown on demand, kept by the engine.  Users hold the
-// arena (acquire_arena / release_arena) from before the first kernel that writes it until
-// after the last one that reads it has been enqueued.
-void* view_scratch(mxp_engine& e, uint64_t bytes) {
-  e.view_tmp.reserve(align_up(bytes, 1 << 20));
-  return e.view_tmp.p;
-}
-
-uint64_t view_source_bytes(const std::vector<uint64_t>& size, int elem_size, int cast) {
-  uint64_t total = op_src_bytes(seg_op_of_cast(cast), (uint64_t)elem_size);
-  for (auto n : size) total *= n;
-  return total;
 }
 
 void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
@@ -1119,19 +1103,13 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
   std::vector<void*> dsts;
   TransposeJob tr{};
   const uint32_t slot = checksum ? 0u : 0xFFFFFFFFu;
-  ViewKind kind = lower_view(src, dst, size, ss, ds, elem_size, cast, slot, boxes, srcs, dsts, tr, nullptr, what);
+  const ViewKind kind = lower_view(src, dst, size, ss, ds, elem_size, cast, slot, boxes, srcs, dsts, tr, what);
   if (kind == kViewEmpty) return;
   HIP_OK(hipSetDevice(e.opt.device));
-  if (kind == kViewNeedsScratch) {
-    acquire_arena(e);
-    void* tmp = view_scratch(e, view_source_bytes(size, elem_size, cast));
-    kind = lower_view(src, dst, size, ss, ds, elem_size, cast, slot, boxes, srcs, dsts, tr, tmp, what);
-  }
   if (kind == kViewTranspose) {
     run_transpose(e, tr, checksum, stream);
     return;
   }
-  if (kind == kViewTransposeBoxes) run_transpose(e, tr, nullptr, stream);
   uint32_t sum = 0;
   run_boxes(e, boxes, srcs, dsts, 1, checksum ? &sum : nullptr, stream);
   if (checksum) *checksum = sum;
@@ -1211,7 +1189,6 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
     std::vector<const void*> srcs;
     std::vector<void*> dsts;
     std::vector<TransposeJob> transposes;
-    std::vector<int64_t> two_step;  // converting transposes: run one by one through the scratch buffer
     for (int64_t k = 0; k < n; ++k) {  // everything is lowered before anything is launched
       const mxp_view_copy& v = views[k];
       check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
@@ -1224,21 +1201,12 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
       const auto s_st = strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what);
       const auto d_st = strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what);
       const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts,
-                                       tr, nullptr, what);
+                                       tr, what);
       if (kind == kViewTranspose) transposes.push_back(tr);
-      else if (kind == kViewNeedsScratch) two_step.push_back(k);
     }
     HIP_OK(hipSetDevice(engine->opt.device));
     if (!boxes.empty()) run_boxes(*engine, boxes, srcs, dsts, 1, nullptr, stream);
     for (const auto& t : transposes) run_transpose(*engine, t, nullptr, stream);
-    for (int64_t k : two_step) {
-      const mxp_view_copy& v = views[k];
-      std::vector<uint64_t> size;
-      for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
-      copy_view(*engine, v.src, v.dst, size, strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what),
-                strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what), v.elem_size, v.cast,
-                nullptr, stream, what);
-    }
   });
 }
 

@@ -12,6 +12,7 @@
 //  digest_kernel  int32-word row sums for the blake2b-hashed tensor digest
 //                 (reads each byte once)
 #include "mxp_device.h"
+#include "mxp_convert.h"
 #include <atomic>
 #include <type_traits>
 
@@ -69,90 +70,6 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
   return v;
-}
-
-// fp32 bits -> bf16 bits, round to nearest even; every NaN becomes `nan_bits`.
-// Reference arithmetic: torch `copy_` at modelexpress_rl/train/engines/fsdp/adapter.py:203-206
-// and refit/reshard/receiver.py:964-971.
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(uint32_t u, uint32_t nan_bits) {
-  const uint32_t r = (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-  return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? nan_bits : r;
-}
-
-// fp32 bits -> fp16 bits, round to nearest even (the wavefront's default rounding mode, with
-// fp16 denormals enabled): overflow -> infinity, subnormal results rounded like any other.
-// The hardware converter does the arithmetic in one instruction; the bit arithmetic it
-// replaces kept this path VALU-bound (4.4 TB/s against 6.0 for fp32 -> bf16).  NaNs are set
-// explicitly so the image does not depend on the converter: the top ten payload bits are kept
-// and the NaN is made quiet (the rule of torch's CPU copy_).
-__device__ __forceinline__ uint32_t f32_to_f16_bits(uint32_t u) {
-  const uint32_t a = u & 0x7FFFFFFFu;
-  const _Float16 h = (_Float16)__uint_as_float(u);
-  uint16_t hb;
-  __builtin_memcpy(&hb, &h, 2);
-  return (a > 0x7F800000u) ? (((u >> 16) & 0x8000u) | 0x7E00u | ((a >> 13) & 0x3FFu)) : (uint32_t)hb;
-}
-
-// fp16 bits -> fp32 bits, exact (subnormals renormalised by the converter); NaNs made quiet.
-__device__ __forceinline__ uint32_t f16_to_f32_bits(uint32_t h) {
-  const uint16_t hb = (uint16_t)h;
-  _Float16 x;
-  __builtin_memcpy(&x, &hb, 2);
-  const uint32_t f = __float_as_uint((float)x);
-  const uint32_t m = h & 0x3FFu;
-  return ((h & 0x7C00u) == 0x7C00u && m) ? (((h & 0x8000u) << 16) | 0x7FC00000u | (m << 13)) : f;
-}
-
-// One 16-bit element of a conversion between the two 16-bit formats, through fp32 as torch's
-// copy_ does: fp16 -> bf16 (NaN -> nan_bits) or bf16 -> fp16.
-template <int OP>
-__device__ __forceinline__ uint32_t recode1(uint32_t h, uint32_t nan_bits) {
-  if constexpr (OP == kOpCastF16Bf16) return f32_to_bf16_bits(f16_to_f32_bits(h), nan_bits);
-  else return f32_to_f16_bits(h << 16);
-}
-template <int OP>
-__device__ __forceinline__ uint32_t recode2(uint32_t w, uint32_t nan_bits) {
-  return recode1<OP>(w & 0xFFFFu, nan_bits) | (recode1<OP>(w >> 16, nan_bits) << 16);
-}
-
-template <int OP>
-__device__ __forceinline__ uint32_t narrow1(uint32_t u, uint32_t nan_bits) {
-  if constexpr (OP == kOpCastF32F16) return f32_to_f16_bits(u);
-  else return f32_to_bf16_bits(u, nan_bits);
-}
-// fp8 e4m3fn bits -> bf16 bits, exact: bias 7 -> 127, subnormals (m * 2^-9) renormalised, the
-// two NaN codes -> 0x7FC0 (torch's image).  Reference: .to(out_dtype) at
-// engines/vllm/refit/receiver.py:258-261 when kv_b_proj is stored in fp8.
-__device__ __forceinline__ uint32_t f8e4m3_to_bf16_bits(uint32_t c) {
-  const uint32_t sign = (c & 0x80u) << 8, e = (c >> 3) & 0xFu, m = c & 7u;
-  if ((c & 0x7Fu) == 0x7Fu) return 0x7FC0u;
-  if (e != 0u) return sign | ((e + 120u) << 7) | (m << 4);
-  if (m == 0u) return sign;
-  const uint32_t top = 31u - (uint32_t)__clz((int)m);
-  return sign | ((top + 118u) << 7) | ((m << (7u - top)) & 0x7Fu);
-}
-
-template <int OP>
-__device__ __forceinline__ uint32_t widen1(uint32_t h) {
-  if constexpr (OP == kOpCastF16F32) return f16_to_f32_bits(h);
-  else return h << 16;
-}
-template <int OP>
-__device__ __forceinline__ uint2 narrow4(const uint4& a, uint32_t nan_bits) {
-  uint2 o;
-  o.x = narrow1<OP>(a.x, nan_bits) | (narrow1<OP>(a.y, nan_bits) << 16);
-  o.y = narrow1<OP>(a.z, nan_bits) | (narrow1<OP>(a.w, nan_bits) << 16);
-  return o;
-}
-template <int OP>
-__device__ __forceinline__ uint4 widen4(const uint2& a) {
-  if constexpr (OP == kOpCastF8E4M3Bf16) {  // eight one-byte elements in, eight bf16 out
-    auto two = [](uint32_t w, int sh) {
-      return f8e4m3_to_bf16_bits((w >> sh) & 0xFFu) | (f8e4m3_to_bf16_bits((w >> (sh + 8)) & 0xFFu) << 16);
-    };
-    return make_uint4(two(a.x, 0), two(a.x, 16), two(a.y, 0), two(a.y, 16));
-  } else
-  return make_uint4(widen1<OP>(a.x & 0xFFFFu), widen1<OP>(a.x >> 16), widen1<OP>(a.y & 0xFFFFu), widen1<OP>(a.y >> 16));
 }
 
 // 128-bit non-temporal accesses: every byte is touched exactly once, so nothing is worth

@@ -39,6 +39,7 @@
 // 384 bytes lifts 16384 x 16384 to 6.0 TB/s: the loss is in how the strided source lines fall
 // on the memory channels, which a caller controls and this kernel does not.
 #include "mxp_device.h"
+#include "mxp_convert.h"
 
 namespace mxp {
 
@@ -86,12 +87,17 @@ struct Csum {
 constexpr int kWaves = kTransposeWaves;
 constexpr int kThreads = kWaves * 64;
 
-template <int ES>
+// Output element size of a transpose that converts on the way (OP = kOpCopy: none).
+constexpr int out_elem(int es, int op) { return op == kOpCopy ? es : (int)op_dst_elem((uint32_t)op); }
+
+template <int ES, int OP>
 struct Sub {
-  static constexpr int kLoads = transpose_sub_rows(ES) / 8;  // 16-byte loads per lane
-  static constexpr int RI = transpose_sub_rows(ES);          // rows (i) of a wavefront's sub-tile
+  static constexpr int EO = out_elem(ES, OP);                 // destination element size
+  static constexpr int RI = transpose_sub_rows(EO);          // rows (i) of a wavefront's sub-tile
+  static constexpr int kLoads = RI / 8;                      // 16-byte loads per lane
   static constexpr int TJ = 128 / ES;                        // columns (j): 128 source bytes per row
-  static constexpr int V = 16 / ES;                          // rows gathered into one 16-byte destination chunk
+  static constexpr int VJ = 16 / ES;                         // source elements in one 16-byte chunk of a row
+  static constexpr int V = 16 / EO;                          // rows gathered into one 16-byte destination chunk
   static constexpr int G = ES == 8 ? 8 : 4;                  // bytes per LDS read
   static constexpr int DPC = 16 / G;                         // LDS reads across one 16-byte source chunk
   static constexpr int CPR = G / ES;                         // destination rows fed by one LDS column
@@ -118,32 +124,53 @@ __device__ __forceinline__ void or_byte(uint4& v, uint32_t e, uint32_t byte) {
   v.w |= (e >= 12u) ? s : 0u;
 }
 
-// Destination chunk p (0 <= p < CPR) out of the NW gathered dwords: element p of every row.
-template <int ES, int P>
-__device__ __forceinline__ uint4 regroup(const uint32_t (&w)[Sub<ES>::NW]) {
-  if constexpr (ES >= 4) {
+// Destination chunk p (0 <= p < CPR) out of the NW gathered dwords: element p of every row,
+// converted where the transpose converts.  Sixteen destination bytes hold V rows; the gathered
+// source bytes for them are 16 (same size), 8 (widening) or 32 (narrowing).
+template <int ES, int OP, int P>
+__device__ __forceinline__ uint4 make_chunk(const uint32_t (&w)[Sub<ES, OP>::NW], uint32_t nan_bits) {
+  constexpr uint32_t kHalf = P == 0 ? 0x05040100u : 0x07060302u;                     // halfword P of two dwords
+  constexpr uint32_t kByte = (uint32_t)P | ((uint32_t)(4 + P) << 8) | 0x0c0c0000u;   // byte P of two dwords, low half
+  if constexpr (OP == kOpCopy && ES >= 4) {
     return make_uint4(w[0], w[1], w[2], w[3]);
-  } else if constexpr (ES == 2) {
-    constexpr uint32_t sel = P == 0 ? 0x05040100u : 0x07060302u;
-    return make_uint4(__builtin_amdgcn_perm(w[1], w[0], sel), __builtin_amdgcn_perm(w[3], w[2], sel),
-                      __builtin_amdgcn_perm(w[5], w[4], sel), __builtin_amdgcn_perm(w[7], w[6], sel));
-  } else {
-    constexpr uint32_t sel = (uint32_t)P | ((uint32_t)(4 + P) << 8) | 0x0c0c0000u;  // byte P of both operands, low half
+  } else if constexpr ((OP == kOpCopy || op_recodes16(OP)) && ES == 2) {
+    const uint4 g = make_uint4(__builtin_amdgcn_perm(w[1], w[0], kHalf), __builtin_amdgcn_perm(w[3], w[2], kHalf),
+                               __builtin_amdgcn_perm(w[5], w[4], kHalf), __builtin_amdgcn_perm(w[7], w[6], kHalf));
+    if constexpr (OP == kOpCopy) return g;
+    else return recode8<OP>(g, nan_bits);
+  } else if constexpr (OP == kOpCopy && ES == 1) {
     uint32_t o[4];
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      const uint32_t a = __builtin_amdgcn_perm(w[4 * d + 1], w[4 * d], sel);
-      const uint32_t b = __builtin_amdgcn_perm(w[4 * d + 3], w[4 * d + 2], sel);
+      const uint32_t a = __builtin_amdgcn_perm(w[4 * d + 1], w[4 * d], kByte);
+      const uint32_t b = __builtin_amdgcn_perm(w[4 * d + 3], w[4 * d + 2], kByte);
       o[d] = a | (b << 16);
     }
     return make_uint4(o[0], o[1], o[2], o[3]);
+  } else if constexpr (op_narrows(OP)) {  // eight fp32 rows -> eight 16-bit elements
+    static_assert(ES == 4, "narrowing transposes read 4-byte elements");
+    const uint2 lo = narrow4<OP>(make_uint4(w[0], w[1], w[2], w[3]), nan_bits);
+    const uint2 hi = narrow4<OP>(make_uint4(w[4], w[5], w[6], w[7]), nan_bits);
+    return make_uint4(lo.x, lo.y, hi.x, hi.y);
+  } else if constexpr (OP == kOpCastF8E4M3Bf16) {  // eight fp8 rows -> eight bf16
+    static_assert(ES == 1, "fp8 source");
+    uint2 g;
+    g.x = __builtin_amdgcn_perm(w[1], w[0], kByte) | (__builtin_amdgcn_perm(w[3], w[2], kByte) << 16);
+    g.y = __builtin_amdgcn_perm(w[5], w[4], kByte) | (__builtin_amdgcn_perm(w[7], w[6], kByte) << 16);
+    return widen4<OP>(g);
+  } else {  // four 16-bit rows -> four fp32
+    static_assert(op_widens(OP) && ES == 2, "widening transposes read 2-byte elements");
+    uint2 g;
+    g.x = __builtin_amdgcn_perm(w[1], w[0], kHalf);
+    g.y = __builtin_amdgcn_perm(w[3], w[2], kHalf);
+    return widen4<OP>(g);
   }
 }
 
-template <int ES, bool FULL>
+template <int ES, int OP, bool FULL>
 __device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_t ci, uint8_t* __restrict__ dp, uint32_t ni,
                                             uint32_t nj, uint64_t dj_bytes, uint32_t csum_base, bool vec_dst, Csum& cs) {
-  using S = Sub<ES>;
+  using S = Sub<ES, OP>;
   const uint64_t off = (uint64_t)jj * dj_bytes + ci * 16u;
   const uint32_t pos = csum_base + (uint32_t)off;
   if constexpr (FULL) {
@@ -156,7 +183,7 @@ __device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_
         st16_nt(dp + off, v);
         cs.add16(v, pos);
       } else {
-        for (uint32_t e = 0; e < n * ES; ++e) {
+        for (uint32_t e = 0; e < n * S::EO; ++e) {
           const uint32_t byte = get_byte(v, e);
           dp[off + e] = (uint8_t)byte;
           cs.add_byte(byte, pos + e);
@@ -169,11 +196,11 @@ __device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_
 // Moves one sub-tile.  FULL: the sub-tile is complete and both sides allow 16-byte accesses,
 // so nothing is predicated.  Otherwise rows / columns beyond (ni, nj) are skipped and chunks
 // that cannot use a 16-byte access are moved byte-wise.
-template <int ES, bool FULL>
+template <int ES, int OP, bool FULL>
 __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uint8_t* __restrict__ dp, uint32_t ni,
                                              uint32_t nj, uint64_t si_bytes, uint64_t dj_bytes, uint32_t csum_base,
-                                             bool vec_src, bool vec_dst, uint8_t* lds, Csum& cs) {
-  using S = Sub<ES>;
+                                             bool vec_src, bool vec_dst, uint32_t nan_bits, uint8_t* lds, Csum& cs) {
+  using S = Sub<ES, OP>;
   const uint32_t lane = threadIdx.x & 63u;
   {
     const uint32_t lrow = lane >> 3, c = lane & 7u;
@@ -186,11 +213,11 @@ __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uin
         x[k] = ld16_nt(g);
       } else {
         x[k] = make_uint4(0, 0, 0, 0);
-        if (row < ni && c * S::V < nj) {
-          if (vec_src && c * S::V + S::V <= nj) {
+        if (row < ni && c * S::VJ < nj) {
+          if (vec_src && c * S::VJ + S::VJ <= nj) {
             x[k] = ld16_nt(g);
           } else {
-            const uint32_t n = min((uint32_t)S::V, nj - c * S::V) * ES;
+            const uint32_t n = min((uint32_t)S::VJ, nj - c * S::VJ) * ES;
             for (uint32_t e = 0; e < n; ++e) or_byte(x[k], e, g[e]);
           }
         }
@@ -225,22 +252,23 @@ __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uin
         w[k] = *reinterpret_cast<const uint32_t*>(l + k * 128);
       }
     }
-    const uint32_t jj0 = a * (16u / ES) + dlo * S::CPR;
-    store_chunk<ES, FULL>(regroup<ES, 0>(w), jj0, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
-    if constexpr (S::CPR >= 2) store_chunk<ES, FULL>(regroup<ES, 1>(w), jj0 + 1, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+    const uint32_t jj0 = a * (uint32_t)S::VJ + dlo * S::CPR;
+    store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 0>(w, nan_bits), jj0, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+    if constexpr (S::CPR >= 2)
+      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 1>(w, nan_bits), jj0 + 1, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
     if constexpr (S::CPR == 4) {
-      store_chunk<ES, FULL>(regroup<ES, 2>(w), jj0 + 2, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
-      store_chunk<ES, FULL>(regroup<ES, 3>(w), jj0 + 3, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 2>(w, nan_bits), jj0 + 2, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 3>(w, nan_bits), jj0 + 3, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
     }
   }
 }
 
-template <int ES>
+template <int ES, int OP>
 __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
                                                               uint8_t* __restrict__ dst,
-                                                              const TransposeDesc d,
+                                                              const TransposeDesc d, uint32_t nan_bits,
                                                               uint32_t* __restrict__ sum_out) {
-  using S = Sub<ES>;
+  using S = Sub<ES, OP>;
   __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   Csum cs;
@@ -264,20 +292,21 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
     s_off += idx * d.batch_sstride[k];
     d_off += idx * d.batch_dstride[k];
   }
-  const uint32_t waves_j = (uint32_t)kWaves / d.waves_i;
+  const uint32_t waves_j = d.waves / d.waves_i;
   const uint64_t i0 = ((uint64_t)ti * d.waves_i + wave % d.waves_i) * S::RI;
   const uint64_t j0 = ((uint64_t)tj * waves_j + wave / d.waves_i) * S::TJ;
   if (i0 < d.ni && j0 < d.nj) {
     const uint32_t ni = (uint32_t)min((uint64_t)S::RI, d.ni - i0), nj = (uint32_t)min((uint64_t)S::TJ, d.nj - j0);
     const uint64_t d_el = d_off + j0 * d.dj + i0;
     const uint8_t* sp = src + (s_off + i0 * d.si + j0) * ES;
-    uint8_t* dp = dst + d_el * ES;
-    const uint32_t csum_base = (uint32_t)(d_el * ES) + d.csum_bias;
+    uint8_t* dp = dst + d_el * S::EO;
+    const uint32_t csum_base = (uint32_t)(d_el * S::EO) + d.csum_bias;
     uint8_t* my_lds = lds + wave * S::kLdsBytes;
     if (d.vec_src && d.vec_dst && ni == (uint32_t)S::RI && nj == (uint32_t)S::TJ)
-      move_subtile<ES, true>(sp, dp, ni, nj, d.si * ES, d.dj * ES, csum_base, true, true, my_lds, cs);
+      move_subtile<ES, OP, true>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, true, true, nan_bits, my_lds, cs);
     else
-      move_subtile<ES, false>(sp, dp, ni, nj, d.si * ES, d.dj * ES, csum_base, d.vec_src != 0, d.vec_dst != 0, my_lds, cs);
+      move_subtile<ES, OP, false>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, d.vec_src != 0, d.vec_dst != 0,
+                                  nan_bits, my_lds, cs);
   }
 
   if (sum_out) {
@@ -289,7 +318,8 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
     if (threadIdx.x == 0) {
       uint32_t t = 0;
 #pragma unroll
-      for (int k = 0; k < kWaves; ++k) t += *reinterpret_cast<const uint32_t*>(lds + k * S::kLdsBytes);
+      for (int k = 0; k < kWaves; ++k)
+        if ((uint32_t)k < d.waves) t += *reinterpret_cast<const uint32_t*>(lds + k * S::kLdsBytes);
       atomicAdd(sum_out, t);
     }
   }
@@ -297,22 +327,39 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
 
 }  // namespace
 
-hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size,
-                            uint32_t* sum_out, hipStream_t stream) {
+hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size, uint32_t op,
+                            uint32_t nan_bits, uint32_t* sum_out, hipStream_t stream) {
   if (d.n_tiles == 0) return hipSuccess;
-  if (d.n_tiles > 0x7FFFFFFFull || d.waves_i == 0 || kWaves % d.waves_i || d.group_j == 0 ||
+  if (d.n_tiles > 0x7FFFFFFFull || d.waves == 0 || d.waves > (uint32_t)kWaves || (d.waves & (d.waves - 1)) ||
+      d.waves_i == 0 || d.waves % d.waves_i || d.group_j == 0 ||
       (uint64_t)d.tiles_i * d.tiles_j > 0x7FFFFFFFull || (uint64_t)d.tiles_i * d.group_j > 0x7FFFFFFFull)
     return hipErrorInvalidValue;
-  const dim3 grid((uint32_t)d.n_tiles), block(kThreads);
+  if (op != kOpCopy && (int)op_src_bytes(op, op_dst_elem(op)) != elem_size) return hipErrorInvalidValue;
+  const dim3 grid((uint32_t)d.n_tiles), block(d.waves * 64u);
   const uint8_t* s = static_cast<const uint8_t*>(src);
   uint8_t* t = static_cast<uint8_t*>(dst);
-  switch (elem_size) {
-    case 1: hipLaunchKernelGGL(transpose_kernel<1>, grid, block, 0, stream, s, t, d, sum_out); break;
-    case 2: hipLaunchKernelGGL(transpose_kernel<2>, grid, block, 0, stream, s, t, d, sum_out); break;
-    case 4: hipLaunchKernelGGL(transpose_kernel<4>, grid, block, 0, stream, s, t, d, sum_out); break;
-    case 8: hipLaunchKernelGGL(transpose_kernel<8>, grid, block, 0, stream, s, t, d, sum_out); break;
+#define MXP_TRANSPOSE(ES, OP) \
+  hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, 0, stream, s, t, d, nan_bits, sum_out)
+  switch (op) {
+    case kOpCopy:
+      switch (elem_size) {
+        case 1: MXP_TRANSPOSE(1, kOpCopy); break;
+        case 2: MXP_TRANSPOSE(2, kOpCopy); break;
+        case 4: MXP_TRANSPOSE(4, kOpCopy); break;
+        case 8: MXP_TRANSPOSE(8, kOpCopy); break;
+        default: return hipErrorInvalidValue;
+      }
+      break;
+    case kOpCastF32Bf16: MXP_TRANSPOSE(4, kOpCastF32Bf16); break;
+    case kOpCastF32F16: MXP_TRANSPOSE(4, kOpCastF32F16); break;
+    case kOpCastBf16F32: MXP_TRANSPOSE(2, kOpCastBf16F32); break;
+    case kOpCastF16F32: MXP_TRANSPOSE(2, kOpCastF16F32); break;
+    case kOpCastF8E4M3Bf16: MXP_TRANSPOSE(1, kOpCastF8E4M3Bf16); break;
+    case kOpCastF16Bf16: MXP_TRANSPOSE(2, kOpCastF16Bf16); break;
+    case kOpCastBf16F16: MXP_TRANSPOSE(2, kOpCastBf16F16); break;
     default: return hipErrorInvalidValue;
   }
+#undef MXP_TRANSPOSE
   return hipGetLastError();
 }
 

@@ -273,6 +273,65 @@ def test_permute_copy_random(gpu_engine, oracle, oracle_c, seed):
     assert csum == oracle_c.checksum32(np.frombuffer(want.tobytes(), dtype=np.uint8))
 
 
+_SRC_WORD = {"F32": np.uint32, "BF16": np.uint16, "F16": np.uint16, "F8_E4M3": np.uint8}
+_DST_WORD = {"F32": np.uint32, "BF16": np.uint16, "F16": np.uint16}
+
+
+@pytest.mark.parametrize("src_dtype,dst_dtype", [("F32", "BF16"), ("BF16", "F32"), ("F16", "F32"), ("F32", "F16"),
+                                                 ("F8_E4M3", "BF16"), ("F16", "BF16"), ("BF16", "F16")])
+def test_converting_transposes_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dtype):
+    """``dest.copy_(src.t())`` across dtypes (refit/reshard/receiver.py:962-969 on a transposed view;
+    engines/vllm/refit/receiver.py:258-261): one pass, bit-exact against convert-then-transpose on the
+    host, over every 16-bit pattern (every rounding class for fp32 sources), ragged edges, strided and
+    unaligned sides, batches, with the checksum of the destination bytes."""
+    rng = np.random.default_rng(77)
+    code = oracle.CAST_CODES[(src_dtype, dst_dtype)]
+    sw, dw = _SRC_WORD[src_dtype], _DST_WORD[dst_dtype]
+    se, de = np.dtype(sw).itemsize, np.dtype(dw).itemsize
+
+    def patterns(n):
+        if src_dtype == "F32":
+            hi = rng.integers(0, 1 << 16, n, dtype=np.uint32) << 16
+            lows = np.array([0, 1, 0x0FFF, 0x1000, 0x1001, 0x1FFF, 0x2000, 0x3000, 0x7FFF, 0x8000, 0x8001, 0xFFFF], dtype=np.uint32)
+            out = hi | lows[rng.integers(0, lows.size, n)]
+            out[: min(n, 1 << 16)] = (np.arange(min(n, 1 << 16), dtype=np.uint32) << 16) | lows[np.arange(min(n, 1 << 16)) % lows.size]
+            return out
+        out = rng.integers(0, 1 << (8 * se), n, dtype=np.uint64).astype(sw)
+        k = min(n, 1 << (8 * se))
+        out[:k] = np.arange(k, dtype=sw)
+        return out
+
+    # (batch, rows, cols, source row pitch, destination row pitch, source offset, destination offset), in elements:
+    # dst[b, c, r] = convert(src[b, r, c])
+    cases = [(1, 512, 512, 512, 512, 0, 0),      # whole tiles, every pattern
+             (1, 130, 70, 70, 130, 0, 0),        # ragged both ways
+             (1, 130, 70, 75, 131, 3, 5),        # odd pitches and offsets: no 16-byte access is aligned
+             (3, 65, 257, 264, 72, 8, 8),        # batch, aligned pitches, ragged extents
+             (1, 1, 300, 300, 1, 0, 0),          # degenerate: a single source row
+             (2, 7, 5, 5, 7, 1, 0)]
+    for (nb, r, c, sp, dp, so, do) in cases:
+        raw = patterns(so + nb * r * sp + 16)
+        src = raw[so: so + nb * r * sp].reshape(nb, r, sp)[:, :, :c]
+        conv = oracle_c.cast(code, np.ascontiguousarray(src).reshape(-1)).reshape(nb, r, c)
+        dst_elems = do + nb * c * dp + 16
+        want = np.full(dst_elems, 0xEEEE if de == 2 else 0xEEEEEEEE, dtype=dw)
+        want[do: do + nb * c * dp].reshape(nb, c, dp)[:, :, :r] = conv.transpose(0, 2, 1)
+        d = torch.from_numpy(np.full(dst_elems * de, 0xEE, dtype=np.uint8)).cuda()
+        dev = _dev(raw.view(np.uint8))
+        csum = gpu_engine.copy_view(dev[so * se:], d[do * de:], (nb, c, r), de, src_strides=(r * sp, 1, sp),
+                                    dst_strides=(c * dp, dp, 1), cast=code)
+        got = d.cpu().numpy().view(dw)
+        assert np.array_equal(got, want), (src_dtype, dst_dtype, nb, r, c, sp, dp, so, do)
+        # the checksum is over the destination view's bytes, positions counted from its first element
+        region = want[do: do + nb * c * dp].copy()
+        mask = np.zeros(nb * c * dp, dtype=bool)
+        mask.reshape(nb, c, dp)[:, :, :r] = True
+        pos = np.flatnonzero(np.repeat(mask, de))
+        b = region.view(np.uint8)[pos].astype(np.uint64)
+        ref = int((b * ((pos.astype(np.uint64) * np.uint64(2654435761) + np.uint64(1)) & np.uint64(0xFFFFFFFF))).sum() & np.uint64(0xFFFFFFFF))
+        assert int(csum, 16) == ref, (src_dtype, dst_dtype, nb, r, c)
+
+
 def test_mla_absorbed_weights_on_device(gpu_engine, oracle, oracle_c):
     # engines/vllm/refit/receiver.py:244-261 on a strided view of kv_b_proj (no intermediate copy)
     H, nope, v, L, es = 16, 128, 128, 512, 2
