@@ -308,6 +308,27 @@ def main() -> int:
                 ops[label] = {"elements": n_el, "ms": round(ms, 4), "gbps_algorithmic": round((se + de) * n_el / ms / 1e6, 1),
                               "frac_of_hbm_peak": round((se + de) * n_el / ms / 1e6 / HBM_PEAK_GBPS, 4)}
                 del a, b
+            # the W_UK_T of every layer of a DeepSeek-V3-shaped model in one call (61 transposes, one launch)
+            H, nope, lat, layers = 128, 128, 512, 61
+            for label, src_dt, se in (("mla_w_uk_t_61_layers_bf16", "BF16", 2), ("mla_w_uk_t_61_layers_f8_bf16", "F8_E4M3", 1)):
+                n_el = H * nope * lat
+                a = torch.empty(layers * n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256)
+                b = torch.empty(layers * n_el * 2, dtype=torch.uint8, device="cuda")
+                code = 0 if src_dt == "BF16" else CAST_CODES[(src_dt, "BF16")]
+                views = [{"src": a[k * n_el * se:], "dst": b[k * n_el * 2:], "shape": (nope, lat, H), "elem_size": 2,
+                          "src_strides": (lat, 1, nope * lat), "cast": code} for k in range(layers)]
+                eng.copy_views(views)
+                ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                ev0.record()
+                for _ in range(10):
+                    eng.copy_views(views)
+                ev1.record()
+                torch.cuda.synchronize()
+                ms = ev0.elapsed_time(ev1) / 10
+                ops[label] = {"elements": layers * n_el, "ms": round(ms, 4),
+                              "gbps_algorithmic": round((se + 2) * layers * n_el / ms / 1e6, 1),
+                              "frac_of_hbm_peak": round((se + 2) * layers * n_el / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                del a, b, views
             out["ops"] = ops
 
         # ---- end-to-end ingest from files through the pinned ring ----

@@ -123,12 +123,31 @@ struct TransposeDesc {
   uint32_t group_j;           // tiles along j that consecutive workgroups visit before stepping along i (>= 1)
   uint32_t waves;             // wavefronts of a workgroup (1, 2, 4 or 8)
 };
+// What the kernels assume of a descriptor (index arithmetic in 32 bits, workgroup shape).
+inline bool transpose_desc_ok(const TransposeDesc& d) {
+  return d.n_tiles <= 0x7FFFFFFFull && d.waves != 0 && d.waves <= (uint32_t)kTransposeWaves && (d.waves & (d.waves - 1)) == 0 &&
+         d.waves_i != 0 && d.waves % d.waves_i == 0 && d.group_j != 0 && (uint64_t)d.tiles_i * d.tiles_j <= 0x7FFFFFFFull &&
+         (uint64_t)d.tiles_i * d.group_j <= 0x7FFFFFFFull;
+}
+// One transpose of a batched launch: `first_tile` is the number of workgroups of the items
+// before it (items sorted by it; every item has d.n_tiles >= 1 and the same d.waves).
+struct alignas(16) TransposeItem {
+  const uint8_t* src;
+  uint8_t* dst;
+  uint64_t first_tile;
+  uint64_t pad;
+  TransposeDesc d;
+};
 // Per-device set-up of the placement kernels (idempotent; also done lazily by launch_place).
 hipError_t configure_place_kernels();
 // `elem_size` is the source element; `op` is kOpCopy or a conversion whose source element it is
 // (dj, batch_dstride and the checksum positions then count destination elements / bytes).
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size, uint32_t op,
                             uint32_t nan_bits, uint32_t* sum_out, hipStream_t stream);
+// `n_items` transposes of one (elem_size, op, waves) in a launch of `total_tiles` workgroups; the
+// host checks each descriptor as launch_transpose would (transpose_desc_ok).
+hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_items, uint64_t total_tiles, uint32_t waves,
+                                  int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream);
 
 // Synthetic-checkpoint generator (mxp_synth.hip), same arithmetic on host and device.
 enum SynthKind : uint32_t {

@@ -113,9 +113,17 @@ struct mxp_engine {
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
   hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
   bool arena_recorded = false;
+  // descriptor table of batched transposes: same protocol as the arena, its own event
+  TransposeItem* items_host = nullptr;  // pinned
+  size_t items_cap = 0;
+  DevBuf<TransposeItem> items_dev;
+  hipEvent_t items_busy = nullptr;
+  bool items_recorded = false;
 
   ~mxp_engine() {
     if (arena_busy) (void)hipEventDestroy(arena_busy);
+    if (items_busy) (void)hipEventDestroy(items_busy);
+    if (items_host) (void)hipHostFree(items_host);
     for (auto s : streams) (void)hipStreamDestroy(s);
     for (auto& s : slots)
       if (s->done) (void)hipEventDestroy(s->done);
@@ -504,6 +512,7 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     HIP_OK(hipEventCreate(&e->ev_a));
     HIP_OK(hipEventCreate(&e->ev_b));
     HIP_OK(hipEventCreateWithFlags(&e->arena_busy, hipEventDisableTiming));
+    HIP_OK(hipEventCreateWithFlags(&e->items_busy, hipEventDisableTiming));
     *out = e.release();
   });
 }
@@ -1066,6 +1075,7 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
     td.vec_dst = vd;
     td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
     for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
+    if (!transpose_desc_ok(td)) fail(MXP_ERR_UNSUPPORTED, "the transposed view needs more workgroups than one launch holds");
     tr = TransposeJob{src, dp, td, (int)eb, op};
   };
 
@@ -1113,6 +1123,58 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
   uint32_t sum = 0;
   run_boxes(e, boxes, srcs, dsts, 1, checksum ? &sum : nullptr, stream);
   if (checksum) *checksum = sum;
+}
+
+// Runs transposes that report no checksum: those that share a kernel instance and workgroup
+// size go out as one launch, the rest one by one.
+void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStream_t stream) {
+  std::vector<size_t> order;
+  for (size_t k = 0; k < jobs.size(); ++k) {
+    if (jobs[k].td.n_tiles) order.push_back(k);  // descriptors were checked when the views were lowered
+  }
+  auto key = [&](size_t k) { return ((uint64_t)jobs[k].op << 16) | ((uint64_t)jobs[k].elem_size << 8) | jobs[k].td.waves; };
+  std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return key(a) < key(b); });
+  std::vector<TransposeItem> items;
+  struct Group { size_t first, count; uint64_t tiles; size_t job; };  // job: any member, for the shared op / element / waves
+  std::vector<Group> groups;
+  for (size_t q = 0; q < order.size();) {
+    size_t r = q;
+    uint64_t tiles = 0;
+    while (r < order.size() && key(order[r]) == key(order[q]) && tiles + jobs[order[r]].td.n_tiles <= 0x7FFFFFFFull)
+      tiles += jobs[order[r++]].td.n_tiles;
+    if (r - q == 1) {
+      run_transpose(e, jobs[order[q]], nullptr, stream);
+    } else {
+      groups.push_back(Group{items.size(), r - q, tiles, order[q]});
+      uint64_t first = 0;
+      for (size_t k = q; k < r; ++k) {
+        const TransposeJob& j = jobs[order[k]];
+        items.push_back(TransposeItem{static_cast<const uint8_t*>(j.src), static_cast<uint8_t*>(j.dst), first, 0, j.td});
+        first += j.td.n_tiles;
+      }
+    }
+    q = r;
+  }
+  if (groups.empty()) return;
+  if (e.items_recorded) HIP_OK(hipEventSynchronize(e.items_busy));
+  if (items.size() > e.items_cap) {
+    if (e.items_host) (void)hipHostFree(e.items_host);
+    e.items_host = nullptr;
+    e.items_cap = 0;
+    const size_t cap = std::max<size_t>(64, items.size() * 2);
+    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e.items_host), cap * sizeof(TransposeItem), hipHostMallocDefault));
+    e.items_cap = cap;
+  }
+  e.items_dev.reserve(e.items_cap);
+  std::memcpy(e.items_host, items.data(), items.size() * sizeof(TransposeItem));
+  HIP_OK(hipMemcpyAsync(e.items_dev.p, e.items_host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
+  for (const Group& g : groups) {
+    const TransposeJob& j = jobs[g.job];
+    HIP_OK(launch_transpose_batch(e.items_dev.p + g.first, (uint32_t)g.count, g.tiles, j.td.waves, j.elem_size, j.op,
+                                  e.opt.nan_bits, stream));
+  }
+  HIP_OK(hipEventRecord(e.items_busy, stream));
+  e.items_recorded = true;
 }
 
 std::vector<uint64_t> strides_or_row_major(const int64_t* strides, const int64_t* shape, int32_t ndim, const char* what) {
@@ -1206,7 +1268,7 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
     }
     HIP_OK(hipSetDevice(engine->opt.device));
     if (!boxes.empty()) run_boxes(*engine, boxes, srcs, dsts, 1, nullptr, stream);
-    for (const auto& t : transposes) run_transpose(*engine, t, nullptr, stream);
+    run_transposes(*engine, transposes, stream);
   });
 }
 

@@ -11,26 +11,32 @@
 // source's innermost dimension (strided in the destination); every other dimension is a
 // batch index.
 //
+// The element type may change on the way (OP: one of the conversions of mxp_convert.h), as in
+// dest.copy_(src.t()) across dtypes (modelexpress/refit/reshard/receiver.py:962-969) or W_UK_T
+// taken from an fp8 kv_b_proj: the conversion happens in registers between steps 3 and 4, so
+// a converting transpose reads every source byte once and writes every destination byte once.
+//
 // Every wavefront moves its own sub-tile and never waits for another one (no workgroup
-// barrier on the data path): 64 or 128 source rows (i) x 128 source bytes (j).
-//   1. global -> registers: lane = (row mod 8, 16-byte chunk); 8 (16 for 1-byte elements)
-//      128-bit loads per lane, all issued before anything else; a wavefront load covers eight
-//      whole 128-byte lines.
+// barrier on the data path): 64 source rows (i; 128 for 1-byte destination elements) x 128
+// source bytes (j).
+//   1. global -> registers: lane = (row mod 8, 16-byte chunk); 8 (or 16) 128-bit loads per
+//      lane, all issued before anything else; a wavefront load covers eight whole 128-byte lines.
 //   2. registers -> LDS, row major, with the chunk index XOR-swizzled by the row group, one
 //      ds_write_b128 per load, conflict free.
 //   3. LDS -> registers: a lane owns a dword column (two bf16 / four fp8 columns) and reads it
-//      down the V = 16 / elem_size rows that make one 16-byte destination chunk; the swizzle
-//      makes the 32 lanes of an LDS cycle hit 32 different banks.  Bytes are regrouped with
-//      v_perm_b32.
+//      down the V = 16 / (destination element size) rows that make one 16-byte destination
+//      chunk; the swizzle makes the 32 lanes of an LDS cycle hit 32 different banks.  Bytes are
+//      regrouped with v_perm_b32 and converted.
 //   4. registers -> global: eight consecutive lanes write one whole 128-byte destination
 //      line, so a wavefront store is eight full lines.  The checksum is taken from the
 //      registers being stored.
 // HBM traffic: every element read once and written once, in whole lines.
 //
-// A workgroup is eight such wavefronts, waves_i of them side by side along i (so the
+// A workgroup is up to eight such wavefronts, waves_i of them side by side along i (so the
 // workgroup writes runs of up to 1 KiB per destination row) and the rest along j; the host
-// picks waves_i from the extent of i.  The workgroup only exists to share an LDS allocation
-// and one checksum atomic.  Measured on 2-byte elements: 16384 x 16384 5.4 TB/s, sixteen
+// picks both numbers from the extents (fewer wavefronts per workgroup when the launch is small).
+// The workgroup only exists to share an LDS allocation and one checksum atomic.  Many
+// transposes of one element type run as one launch (transpose_batch_kernel).  Measured on 2-byte elements: 16384 x 16384 5.4 TB/s, sixteen
 // 4096 x 4096 matrices 6.2 TB/s (a plain copy of the same bytes through place_kernel: 5.7);
 // the rate depends on the two pitches.  When the destination pitch is the larger one, the host
 // asks for two wavefronts along i and bands of eight tiles along j (65536 x 4096: 5.3 against
@@ -263,19 +269,16 @@ __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uin
   }
 }
 
+// One workgroup's share of transpose `d`: tile number `tile` of its n_tiles.
 template <int ES, int OP>
-__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
-                                                              uint8_t* __restrict__ dst,
-                                                              const TransposeDesc d, uint32_t nan_bits,
-                                                              uint32_t* __restrict__ sum_out) {
+__device__ __forceinline__ void transpose_tile(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                               const TransposeDesc& d, uint64_t tile, uint32_t nan_bits, uint8_t* lds,
+                                               uint32_t wave, Csum& cs) {
   using S = Sub<ES, OP>;
-  __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
-  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  Csum cs;
   // Linear tile index -> (batch, tile_j, tile_i), tile_i fastest.  Workgroup-uniform.
   const uint64_t per_batch = (uint64_t)d.tiles_i * d.tiles_j;
-  uint64_t b = blockIdx.x / per_batch;
-  const uint32_t within = (uint32_t)(blockIdx.x % per_batch);
+  uint64_t b = tile / per_batch;
+  const uint32_t within = (uint32_t)(tile % per_batch);
   // Inside a batch, tiles are visited in bands of group_j tiles along j: with group_j > 1,
   // consecutive workgroups read neighbouring lines of the same source rows.
   const uint32_t gj = d.group_j;
@@ -308,6 +311,18 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
       move_subtile<ES, OP, false>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, d.vec_src != 0, d.vec_dst != 0,
                                   nan_bits, my_lds, cs);
   }
+}
+
+template <int ES, int OP>
+__global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
+                                                              uint8_t* __restrict__ dst,
+                                                              const TransposeDesc d, uint32_t nan_bits,
+                                                              uint32_t* __restrict__ sum_out) {
+  using S = Sub<ES, OP>;
+  __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  Csum cs;
+  transpose_tile<ES, OP>(src, dst, d, blockIdx.x, nan_bits, lds, wave, cs);
 
   if (sum_out) {
     // Each wavefront leaves its partial sum in the first dword of its own LDS region (its
@@ -325,41 +340,96 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
   }
 }
 
+// Many transposes of one element type in one launch: `items` is sorted by first_tile, and a
+// workgroup finds its transpose by bisection (workgroup-uniform, scalar loads).
+template <int ES, int OP>
+__global__ __launch_bounds__(kThreads) void transpose_batch_kernel(const TransposeItem* __restrict__ items,
+                                                                    uint32_t n_items, uint32_t nan_bits) {
+  using S = Sub<ES, OP>;
+  __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
+  const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  uint32_t lo = 0, hi = n_items;  // the last item with first_tile <= blockIdx.x
+  while (hi - lo > 1) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (items[mid].first_tile <= (uint64_t)blockIdx.x) lo = mid;
+    else hi = mid;
+  }
+  const TransposeItem& it = items[lo];
+  Csum cs;
+  transpose_tile<ES, OP>(it.src, it.dst, it.d, (uint64_t)blockIdx.x - it.first_tile, nan_bits, lds, wave, cs);
+}
+
+}  // namespace
+
+namespace {
+
+// Calls f.template operator()<ES, OP>() for the kernel instance of (elem_size, op); false if there is none.
+template <typename F>
+bool with_instance(int elem_size, uint32_t op, F&& f) {
+  if (op != kOpCopy && (int)op_src_bytes(op, op_dst_elem(op)) != elem_size) return false;
+  switch (op) {
+    case kOpCopy:
+      switch (elem_size) {
+        case 1: f.template operator()<1, kOpCopy>(); return true;
+        case 2: f.template operator()<2, kOpCopy>(); return true;
+        case 4: f.template operator()<4, kOpCopy>(); return true;
+        case 8: f.template operator()<8, kOpCopy>(); return true;
+        default: return false;
+      }
+    case kOpCastF32Bf16: f.template operator()<4, kOpCastF32Bf16>(); return true;
+    case kOpCastF32F16: f.template operator()<4, kOpCastF32F16>(); return true;
+    case kOpCastBf16F32: f.template operator()<2, kOpCastBf16F32>(); return true;
+    case kOpCastF16F32: f.template operator()<2, kOpCastF16F32>(); return true;
+    case kOpCastF8E4M3Bf16: f.template operator()<1, kOpCastF8E4M3Bf16>(); return true;
+    case kOpCastF16Bf16: f.template operator()<2, kOpCastF16Bf16>(); return true;
+    case kOpCastBf16F16: f.template operator()<2, kOpCastBf16F16>(); return true;
+    default: return false;
+  }
+}
+
+struct LaunchOne {
+  dim3 grid, block;
+  hipStream_t stream;
+  const uint8_t* s;
+  uint8_t* t;
+  const TransposeDesc& d;
+  uint32_t nan_bits;
+  uint32_t* sum_out;
+  template <int ES, int OP>
+  void operator()() const {
+    hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, 0, stream, s, t, d, nan_bits, sum_out);
+  }
+};
+
+struct LaunchBatch {
+  dim3 grid, block;
+  hipStream_t stream;
+  const TransposeItem* items;
+  uint32_t n_items, nan_bits;
+  template <int ES, int OP>
+  void operator()() const {
+    hipLaunchKernelGGL((transpose_batch_kernel<ES, OP>), grid, block, 0, stream, items, n_items, nan_bits);
+  }
+};
+
 }  // namespace
 
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size, uint32_t op,
                             uint32_t nan_bits, uint32_t* sum_out, hipStream_t stream) {
   if (d.n_tiles == 0) return hipSuccess;
-  if (d.n_tiles > 0x7FFFFFFFull || d.waves == 0 || d.waves > (uint32_t)kWaves || (d.waves & (d.waves - 1)) ||
-      d.waves_i == 0 || d.waves % d.waves_i || d.group_j == 0 ||
-      (uint64_t)d.tiles_i * d.tiles_j > 0x7FFFFFFFull || (uint64_t)d.tiles_i * d.group_j > 0x7FFFFFFFull)
-    return hipErrorInvalidValue;
-  if (op != kOpCopy && (int)op_src_bytes(op, op_dst_elem(op)) != elem_size) return hipErrorInvalidValue;
-  const dim3 grid((uint32_t)d.n_tiles), block(d.waves * 64u);
-  const uint8_t* s = static_cast<const uint8_t*>(src);
-  uint8_t* t = static_cast<uint8_t*>(dst);
-#define MXP_TRANSPOSE(ES, OP) \
-  hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, 0, stream, s, t, d, nan_bits, sum_out)
-  switch (op) {
-    case kOpCopy:
-      switch (elem_size) {
-        case 1: MXP_TRANSPOSE(1, kOpCopy); break;
-        case 2: MXP_TRANSPOSE(2, kOpCopy); break;
-        case 4: MXP_TRANSPOSE(4, kOpCopy); break;
-        case 8: MXP_TRANSPOSE(8, kOpCopy); break;
-        default: return hipErrorInvalidValue;
-      }
-      break;
-    case kOpCastF32Bf16: MXP_TRANSPOSE(4, kOpCastF32Bf16); break;
-    case kOpCastF32F16: MXP_TRANSPOSE(4, kOpCastF32F16); break;
-    case kOpCastBf16F32: MXP_TRANSPOSE(2, kOpCastBf16F32); break;
-    case kOpCastF16F32: MXP_TRANSPOSE(2, kOpCastF16F32); break;
-    case kOpCastF8E4M3Bf16: MXP_TRANSPOSE(1, kOpCastF8E4M3Bf16); break;
-    case kOpCastF16Bf16: MXP_TRANSPOSE(2, kOpCastF16Bf16); break;
-    case kOpCastBf16F16: MXP_TRANSPOSE(2, kOpCastBf16F16); break;
-    default: return hipErrorInvalidValue;
-  }
-#undef MXP_TRANSPOSE
+  if (!transpose_desc_ok(d)) return hipErrorInvalidValue;
+  const LaunchOne one{dim3((uint32_t)d.n_tiles), dim3(d.waves * 64u), stream, static_cast<const uint8_t*>(src),
+                      static_cast<uint8_t*>(dst), d, nan_bits, sum_out};
+  if (!with_instance(elem_size, op, one)) return hipErrorInvalidValue;
+  return hipGetLastError();
+}
+
+hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_items, uint64_t total_tiles, uint32_t waves,
+                                  int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream) {
+  if (n_items == 0 || total_tiles == 0) return hipSuccess;
+  if (total_tiles > 0x7FFFFFFFull || waves == 0 || waves > (uint32_t)kWaves || (waves & (waves - 1))) return hipErrorInvalidValue;
+  const LaunchBatch many{dim3((uint32_t)total_tiles), dim3(waves * 64u), stream, items_dev, n_items, nan_bits};
+  if (!with_instance(elem_size, op, many)) return hipErrorInvalidValue;
   return hipGetLastError();
 }
 

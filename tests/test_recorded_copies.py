@@ -171,3 +171,43 @@ def test_mla_absorbed_weights_as_recorded_copies(gpu_engine, src_dt):
     assert torch.equal(params["W_UV"].cpu().view(torch.int16), want_uv.view(torch.int16))
     assert torch.equal(params["W_UK_T"].cpu().view(torch.int16), want_ukt.view(torch.int16))
     assert {k: v.data_ptr() for k, v in params.items()} == ptrs  # written in place: graph-bound addresses are kept
+
+
+@pytest.mark.gpu
+def test_many_transposed_copies_share_launches(gpu_engine):
+    """A refit's worth of transposed copies (one W_UK_T per layer, engines/vllm/refit/receiver.py:252-261,
+    plus transposed weights of other dtypes) handed over in one call: transposes of one element type run
+    as one launch, and every destination matches torch's ``as_strided().copy_()``."""
+    g = torch.Generator().manual_seed(5)
+    specs = []
+    for layer in range(6):  # same shape, same dtype: one group
+        specs.append(((8, 24, 40), (("permute", (1, 2, 0), ()),), torch.bfloat16, torch.bfloat16))
+    specs += [
+        ((130, 70), (("transpose", (0, 1), ()),), torch.bfloat16, torch.bfloat16),      # ragged member of the same group
+        ((256, 192), (("transpose", (0, 1), ()),), torch.float32, torch.bfloat16),
+        ((65, 33), (("transpose", (0, 1), ()),), torch.float32, torch.bfloat16),
+        ((4, 64, 128), (("permute", (1, 2, 0), ()),), torch.float8_e4m3fn, torch.bfloat16),
+        ((4, 64, 128), (("permute", (0, 2, 1), ()),), torch.float8_e4m3fn, torch.bfloat16),
+        ((96, 48), (("transpose", (0, 1), ()),), torch.bfloat16, torch.float32),
+        ((2048, 1024), (("transpose", (0, 1), ()),), torch.bfloat16, torch.bfloat16),   # eight waves per workgroup: its own group
+        ((2048, 1024), (("transpose", (0, 1), ()),), torch.bfloat16, torch.bfloat16),
+        ((64, 96), (("narrow", (0, 16, 32), ()),), torch.bfloat16, torch.bfloat16),     # a row copy in the same call
+        ((7, 9), (("transpose", (0, 1), ()),), torch.float32, torch.float32),           # alone in its group
+    ]
+    sources, params, wants, copies = {}, {}, {}, []
+    for k, (shape, chain, src_dt, dst_dt) in enumerate(specs):
+        src = (torch.randn(shape, generator=g) * 3).to(src_dt)
+        view = _apply(chain, src)
+        stride = tuple(torch.empty(view.shape).stride())
+        want = torch.full(tuple(view.shape), 7, dtype=dst_dt)
+        want.copy_(view)
+        sources[f"w{k}"], wants[f"p{k}"] = src.cuda(), want
+        params[f"p{k}"] = torch.full(tuple(view.shape), 7, dtype=dst_dt, device="cuda")
+        copies.append(RecordedCopy(f"w{k}", chain, f"p{k}", 0, tuple(view.shape), stride, dst_dt))
+    for _ in range(2):  # the descriptor table is reused by the second call
+        n = execute_recorded_copies(gpu_engine, copies, sources, params)
+        assert n == sum(w.numel() * w.element_size() for w in wants.values())
+        for name, want in wants.items():
+            assert torch.equal(params[name].cpu().view(torch.uint8), want.view(torch.uint8)), name
+        for p in params.values():
+            p.fill_(7)
