@@ -241,6 +241,21 @@ def main() -> int:
                                 "gbps_wall": round(placed / dt / 1e9, 1),
                                 "note": "one batched launch; wall time includes descriptor upload, result copy and sync"}
             ops["checksum32"]["matches_fused"] = eng.checksum32(dst, sizes) == resident_sums
+            # context only: the platform's own device copy of as many bytes as one step places
+            a = torch.empty(placed, dtype=torch.uint8, device="cuda").random_(0, 256)
+            b = torch.empty_like(a)
+            b.copy_(a)
+            ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            ev0.record()
+            for _ in range(10):
+                b.copy_(a)
+            ev1.record()
+            torch.cuda.synchronize()
+            ms = ev0.elapsed_time(ev1) / 10
+            ops["torch_copy_same_bytes"] = {"bytes": placed, "ms": round(ms, 4), "gbps_algorithmic": round(2 * placed / ms / 1e6, 1),
+                                            "frac_of_hbm_peak": round(2 * placed / ms / 1e6 / HBM_PEAK_GBPS, 4),
+                                            "note": "torch.Tensor.copy_ between two contiguous device buffers; not part of the path"}
+            del a, b
             # LDS transpose (permuted copies): a square bf16 matrix, a batch of smaller ones and the MLA W_UK_T shape
             for label, shape, perm in (("transpose_bf16_16384x16384", (16384, 16384), (1, 0)),
                                        ("transpose_bf16_16x4096x4096", (16, 4096, 4096), (0, 2, 1)),
