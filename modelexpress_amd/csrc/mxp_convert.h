@@ -14,6 +14,23 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(uint32_t u, uint32_t nan_bi
   return ((u & 0x7FFFFFFFu) > 0x7F800000u) ? nan_bits : r;
 }
 
+// Two fp32 -> two bf16 (a in the low half), same result as f32_to_bf16_bits on each: the
+// hardware's packed converter rounds to nearest even, and since rounding a finite value never
+// gives a NaN, a NaN half of its result marks a NaN input; those halves become `nan_bits`.
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2(uint32_t a, uint32_t b, uint32_t nan_bits) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  f32x2 f;
+  f.x = __uint_as_float(a);
+  f.y = __uint_as_float(b);
+  const bf16x2 h = __builtin_convertvector(f, bf16x2);
+  uint32_t p;
+  __builtin_memcpy(&p, &h, 4);
+  const uint32_t nan = (((p & 0x7FFF7FFFu) + 0x007F007Fu) & 0x80008000u) >> 15;  // bit 0 / bit 16 per NaN half
+  const uint32_t mask = nan * 0xFFFFu;
+  return (p & ~mask) | ((nan_bits * 0x00010001u) & mask);
+}
+
 // fp32 bits -> fp16 bits, round to nearest even (the wavefront's default rounding mode, with
 // fp16 denormals enabled): overflow -> infinity, subnormal results rounded like any other.
 // The hardware converter does the arithmetic in one instruction; the bit arithmetic it
@@ -47,7 +64,15 @@ __device__ __forceinline__ uint32_t recode1(uint32_t h, uint32_t nan_bits) {
 }
 template <int OP>
 __device__ __forceinline__ uint32_t recode2(uint32_t w, uint32_t nan_bits) {
-  return recode1<OP>(w & 0xFFFFu, nan_bits) | (recode1<OP>(w >> 16, nan_bits) << 16);
+  if constexpr (OP == kOpCastF16Bf16) {
+    // exact widening by the converter (a NaN stays a NaN, whatever its payload), then the packed rounding
+    typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+    f16x2 h;
+    __builtin_memcpy(&h, &w, 4);
+    return f32x2_to_bf16x2(__float_as_uint((float)h.x), __float_as_uint((float)h.y), nan_bits);
+  } else {
+    return recode1<OP>(w & 0xFFFFu, nan_bits) | (recode1<OP>(w >> 16, nan_bits) << 16);
+  }
 }
 
 template <int OP>
@@ -90,8 +115,13 @@ __device__ __forceinline__ uint32_t widen1(uint32_t h) {
 template <int OP>
 __device__ __forceinline__ uint2 narrow4(const uint4& a, uint32_t nan_bits) {
   uint2 o;
-  o.x = narrow1<OP>(a.x, nan_bits) | (narrow1<OP>(a.y, nan_bits) << 16);
-  o.y = narrow1<OP>(a.z, nan_bits) | (narrow1<OP>(a.w, nan_bits) << 16);
+  if constexpr (OP == kOpCastF32Bf16) {
+    o.x = f32x2_to_bf16x2(a.x, a.y, nan_bits);
+    o.y = f32x2_to_bf16x2(a.z, a.w, nan_bits);
+  } else {
+    o.x = narrow1<OP>(a.x, nan_bits) | (narrow1<OP>(a.y, nan_bits) << 16);
+    o.y = narrow1<OP>(a.z, nan_bits) | (narrow1<OP>(a.w, nan_bits) << 16);
+  }
   return o;
 }
 template <int OP>
