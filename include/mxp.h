@@ -349,9 +349,9 @@ int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndi
  * source.as_strided(shape, src_strides)).  Rows contiguous on both sides run as pitched boxes,
  * a transposed innermost dimension through the LDS transpose, anything else element by
  * element (the run length paired_runs would find).  A destination view that overlaps itself
- * is refused.  `cast` is an MXP_CAST_* code (then `elem_size` is the destination element's and the
- * transpose route is not taken).  *checksum, when not NULL, receives the position-weighted checksum of the
- * written bytes, positions counted from `dst`. */
+ * is refused.  `cast` is an MXP_CAST_* code (then `elem_size` is the destination element's; a
+ * transposed view converts inside the transpose, in one pass).  *checksum, when not NULL, receives
+ * the position-weighted checksum of the written bytes, positions counted from `dst`. */
 int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
                   const int64_t* src_strides, const int64_t* dst_strides, int32_t elem_size,
                   int32_t cast, uint32_t* checksum, void* stream);
@@ -370,9 +370,10 @@ typedef struct mxp_view_copy {
   int64_t dst_strides[MXP_MAX_DIMS];
 } mxp_view_copy;
 /* n recorded copies at once: every view is lowered first (an error moves nothing), then all
- * row / element boxes run in ONE launch and each transposed view in one launch of its own -
- * in place of the reference's launch per view ("thousands of individual kernel launches",
- * refit/reshard/receiver.py:920-923).  Destinations must not overlap one another. */
+ * row / element boxes run in ONE launch and the transposed views in one launch per element
+ * type and conversion - in place of the reference's launch per view ("thousands of
+ * individual kernel launches", refit/reshard/receiver.py:920-923).  Destinations must not
+ * overlap one another: the launches give no order between views. */
 int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, void* stream);
 /* n independent contiguous device copies in one launch, with the checksum of each
  * destination in out_checksums[k] when not NULL: the device form of the batched

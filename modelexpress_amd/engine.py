@@ -415,7 +415,7 @@ class PlacementEngine:
 
     def copy_views(self, views: Sequence[dict], *, stream: int = 0) -> None:
         """Many ``copy_view`` calls in one go (keys: src, dst, shape, elem_size and optionally src_strides,
-        dst_strides, cast): all row / element boxes run in one launch, transposed views one launch each."""
+        dst_strides, cast): all row / element boxes run in one launch, transposed views in one launch per element type and conversion."""
         arr = (L.ViewCopy * max(1, len(views)))()
         for v, o in zip(views, arr):
             shape = [int(x) for x in v["shape"]]
