@@ -105,3 +105,29 @@ def test_buffer_beyond_4_gib_wraps_positions_like_the_reference(oracle_c, gpu_en
     assert gpu_engine.copy_batch([dev], [out], [n]) == [want]
     assert torch.equal(out[-(1 << 20):], dev[-(1 << 20):]) and torch.equal(out[: 1 << 20], dev[: 1 << 20])
     assert gpu_engine.digest([out]) == gpu_engine.digest([dev])
+
+
+def test_transposes_beyond_4_gib(gpu_engine, oracle_c):
+    """A transposed copy larger than 4 GiB on each side (offsets and tile indices beyond 32 bits):
+    transposing twice gives the source back, a strip pulled to the host equals the host transpose,
+    and the fused checksum equals the stand-alone checksum of the result."""
+    rows, cols = 70_000, 33_000  # 4.62 GB of bf16 per side; neither extent is a tile multiple
+    src = torch.empty(rows * cols * 2, dtype=torch.uint8, device="cuda").random_(0, 256)
+    mid = torch.empty_like(src)
+    c_mid = gpu_engine.permute_copy(src, mid, (rows, cols), (1, 0), 2)
+    assert c_mid == gpu_engine.checksum32([mid], [mid.numel()])[0]
+    s2 = src.view(torch.int16).view(rows, cols)
+    m2 = mid.view(torch.int16).view(cols, rows)
+    for r0, c0 in ((0, 0), (rows - 300, cols - 500), (33_333, 17_001)):  # strips around both ends and past 4 GiB
+        want = s2[r0:r0 + 300, c0:c0 + 500].cpu().numpy().T
+        assert np.array_equal(m2[c0:c0 + 500, r0:r0 + 300].cpu().numpy(), want), (r0, c0)
+    back = torch.empty_like(src)
+    gpu_engine.permute_copy(mid, back, (cols, rows), (1, 0), 2, checksum=False)
+    assert torch.equal(back, src)
+    del back, mid
+    # the same extents converting fp32 -> bf16 on the way (source 9.2 GB), against torch's device conversion
+    f = torch.randn(rows, cols, device="cuda")
+    out = torch.empty(cols, rows, dtype=torch.bfloat16, device="cuda")
+    gpu_engine.copy_view(f, out, (cols, rows), 2, src_strides=(1, cols), cast=1, checksum=False)
+    for c0 in (0, cols - 1000, 20_000):
+        assert torch.equal(out[c0:c0 + 1000].view(torch.int16), f[:, c0:c0 + 1000].t().to(torch.bfloat16).contiguous().view(torch.int16)), c0
