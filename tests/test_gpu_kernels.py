@@ -332,6 +332,50 @@ def test_converting_transposes_match_oracle(gpu_engine, oracle, oracle_c, src_dt
         assert int(csum, 16) == ref, (src_dtype, dst_dtype, nb, r, c)
 
 
+def _random_layout(rng, shape):
+    """Strides (in elements) of a view of `shape` inside a padded buffer whose dimensions are stored in a random order."""
+    order = list(rng.permutation(len(shape)))  # storage order, outermost first
+    strides = [0] * len(shape)
+    run = 1
+    for d in reversed(order):
+        strides[d] = run
+        run *= shape[d] + int(rng.integers(0, 3)) * int(rng.integers(0, 2))  # sometimes padded
+    return strides, run
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_copy_view_random_layouts_and_conversions(gpu_engine, oracle, oracle_c, seed):
+    """``dst.as_strided(shape, ds).copy_(src.as_strided(shape, ss))`` for random shapes, storage orders,
+    paddings, offsets and conversions (refit/reshard/types.py:57-71 executed on the device): whichever
+    route a view takes - row boxes, the transpose, element runs - the bytes equal numpy's strided copy
+    of the host-converted source, and nothing outside the view is written."""
+    rng = np.random.default_rng(4000 + seed)
+    pairs = [None] + list(oracle.CAST_CODES)
+    pair = pairs[seed % len(pairs)]
+    if pair is None:
+        es = int(rng.choice([1, 2, 4, 8]))
+        sw = dw = {1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[es]
+        code = 0
+    else:
+        sw, dw, code = _SRC_WORD[pair[0]], _DST_WORD[pair[1]], oracle.CAST_CODES[pair]
+    se, de = np.dtype(sw).itemsize, np.dtype(dw).itemsize
+    nd = int(rng.integers(1, 5))
+    shape = [int(x) for x in rng.integers(1, {1: 5000, 2: 300, 3: 60, 4: 20}[nd], nd)]
+    ss, s_span = _random_layout(rng, shape)
+    ds, d_span = _random_layout(rng, shape)
+    so, do = int(rng.integers(0, 9)), int(rng.integers(0, 9))
+    raw = rng.integers(0, 1 << 63, so + s_span + 8, dtype=np.uint64).astype(sw)
+    view = np.lib.stride_tricks.as_strided(raw[so:], shape, [x * se for x in ss])
+    conv = view.copy() if code == 0 else oracle_c.cast(code, np.ascontiguousarray(view).reshape(-1)).reshape(shape)
+    fill = np.array(0xEEEEEEEEEEEEEEEE, dtype=np.uint64).astype(dw)
+    want = np.full(do + d_span + 8, fill, dtype=dw)
+    np.lib.stride_tricks.as_strided(want[do:], shape, [x * de for x in ds])[...] = conv
+    d = torch.from_numpy(np.full(want.size * de, 0xEE, dtype=np.uint8)).cuda()
+    dev = _dev(raw.view(np.uint8))
+    gpu_engine.copy_view(dev[so * se:], d[do * de:], shape, de, src_strides=ss, dst_strides=ds, cast=code, checksum=False)
+    assert np.array_equal(d.cpu().numpy().view(dw), want), (pair, shape, ss, ds, so, do)
+
+
 def test_mla_absorbed_weights_on_device(gpu_engine, oracle, oracle_c):
     # engines/vllm/refit/receiver.py:244-261 on a strided view of kv_b_proj (no intermediate copy)
     H, nope, v, L, es = 16, 128, 128, 512, 2
