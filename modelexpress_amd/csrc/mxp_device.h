@@ -117,7 +117,7 @@ struct TransposeDesc {
   uint64_t batch_size[kMaxBatchDims];     // unused entries are 1
   uint64_t batch_sstride[kMaxBatchDims];
   uint64_t batch_dstride[kMaxBatchDims];
-  uint32_t vec_src, vec_dst;  // 16-byte accesses are aligned on that side
+  uint32_t align_src, align_dst;  // power of two <= 16 that divides every address a chunk access can have on that side
   uint32_t csum_bias;
   uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides waves)
   uint32_t group_j;           // tiles along j that consecutive workgroups visit before stepping along i (>= 1)

@@ -1058,8 +1058,10 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
       td.tiles_j = (uint32_t)((td.nj + tile_j - 1) / tile_j);
       if (waves == 1 || batches * td.tiles_i * td.tiles_j >= 2ull * kChipCus) break;
     }
-    bool vs = (reinterpret_cast<uintptr_t>(src) % 16 == 0) && (td.si * eb) % 16 == 0;
-    bool vd = (reinterpret_cast<uintptr_t>(dp) % 16 == 0) && (td.dj * es) % 16 == 0;
+    // Alignment of each side: the largest power of two (at most 16) dividing the base address and every byte stride.
+    auto pow2 = [](uint64_t v) { return (v | 16u) & (~(v | 16u) + 1u); };
+    uint64_t vs = pow2(reinterpret_cast<uintptr_t>(src) | (td.si * eb));
+    uint64_t vd = pow2(reinterpret_cast<uintptr_t>(dp) | (td.dj * es));
     int k = kMaxBatchDims - 1;
     for (int q = 0; q < kMaxBatchDims; ++q) { td.batch_size[q] = 1; td.batch_sstride[q] = 0; td.batch_dstride[q] = 0; }
     for (int d = (int)nd - 2; d >= 0; --d) {
@@ -1067,12 +1069,14 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
       td.batch_size[k] = size[d];
       td.batch_sstride[k] = ss[d];
       td.batch_dstride[k] = d_in[d];
-      vs = vs && (ss[d] * eb) % 16 == 0;
-      vd = vd && (d_in[d] * es) % 16 == 0;
+      if (size[d] > 1) {
+        vs = std::min(vs, pow2(ss[d] * eb));
+        vd = std::min(vd, pow2(d_in[d] * es));
+      }
       --k;
     }
-    td.vec_src = vs;
-    td.vec_dst = vd;
+    td.align_src = (uint32_t)vs;
+    td.align_dst = (uint32_t)vd;
     td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
     for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
     if (!transpose_desc_ok(td)) fail(MXP_ERR_UNSUPPORTED, "the transposed view needs more workgroups than one launch holds");

@@ -175,7 +175,7 @@ __device__ __forceinline__ uint4 make_chunk(const uint32_t (&w)[Sub<ES, OP>::NW]
 
 template <int ES, int OP, bool FULL>
 __device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_t ci, uint8_t* __restrict__ dp, uint32_t ni,
-                                            uint32_t nj, uint64_t dj_bytes, uint32_t csum_base, bool vec_dst, Csum& cs) {
+                                            uint32_t nj, uint64_t dj_bytes, uint32_t csum_base, uint32_t align_dst, Csum& cs) {
   using S = Sub<ES, OP>;
   const uint64_t off = (uint64_t)jj * dj_bytes + ci * 16u;
   const uint32_t pos = csum_base + (uint32_t)off;
@@ -185,8 +185,24 @@ __device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_
   } else {
     if (jj < nj && ci * S::V < ni) {
       const uint32_t n = min((uint32_t)S::V, ni - ci * S::V);
-      if (vec_dst && n == (uint32_t)S::V) {
-        st16_nt(dp + off, v);
+      if (n == (uint32_t)S::V && align_dst >= 2u) {
+        // a whole chunk: the widest stores the destination's alignment allows
+        uint8_t* q = dp + off;
+        if (align_dst >= 16u) {
+          st16_nt(q, v);
+        } else if (align_dst >= 8u) {
+          *reinterpret_cast<uint2*>(q) = make_uint2(v.x, v.y);
+          *reinterpret_cast<uint2*>(q + 8) = make_uint2(v.z, v.w);
+        } else if (align_dst >= 4u) {
+          *reinterpret_cast<uint32_t*>(q) = v.x;
+          *reinterpret_cast<uint32_t*>(q + 4) = v.y;
+          *reinterpret_cast<uint32_t*>(q + 8) = v.z;
+          *reinterpret_cast<uint32_t*>(q + 12) = v.w;
+        } else {
+          const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+          for (int h = 0; h < 8; ++h) *reinterpret_cast<uint16_t*>(q + 2 * h) = (uint16_t)(w[h >> 1] >> (16 * (h & 1)));
+        }
         cs.add16(v, pos);
       } else {
         for (uint32_t e = 0; e < n * S::EO; ++e) {
@@ -200,12 +216,14 @@ __device__ __forceinline__ void store_chunk(const uint4& v, uint32_t jj, uint32_
 }
 
 // Moves one sub-tile.  FULL: the sub-tile is complete and both sides allow 16-byte accesses,
-// so nothing is predicated.  Otherwise rows / columns beyond (ni, nj) are skipped and chunks
-// that cannot use a 16-byte access are moved byte-wise.
+// so nothing is predicated.  Otherwise rows / columns beyond (ni, nj) are skipped, whole chunks
+// move in pieces as wide as the side's alignment allows (8, 4 or 2 bytes) and ragged chunks
+// byte-wise.
 template <int ES, int OP, bool FULL>
 __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uint8_t* __restrict__ dp, uint32_t ni,
                                              uint32_t nj, uint64_t si_bytes, uint64_t dj_bytes, uint32_t csum_base,
-                                             bool vec_src, bool vec_dst, uint32_t nan_bits, uint8_t* lds, Csum& cs) {
+                                             uint32_t align_src, uint32_t align_dst, uint32_t nan_bits, uint8_t* lds,
+                                             Csum& cs) {
   using S = Sub<ES, OP>;
   const uint32_t lane = threadIdx.x & 63u;
   {
@@ -220,8 +238,24 @@ __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uin
       } else {
         x[k] = make_uint4(0, 0, 0, 0);
         if (row < ni && c * S::VJ < nj) {
-          if (vec_src && c * S::VJ + S::VJ <= nj) {
-            x[k] = ld16_nt(g);
+          if (c * S::VJ + S::VJ <= nj && align_src >= 2u) {
+            // a whole chunk: the widest loads the source's alignment allows
+            if (align_src >= 16u) {
+              x[k] = ld16_nt(g);
+            } else if (align_src >= 8u) {
+              const uint2 lo = *reinterpret_cast<const uint2*>(g), hi = *reinterpret_cast<const uint2*>(g + 8);
+              x[k] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+            } else if (align_src >= 4u) {
+              x[k] = make_uint4(*reinterpret_cast<const uint32_t*>(g), *reinterpret_cast<const uint32_t*>(g + 4),
+                                *reinterpret_cast<const uint32_t*>(g + 8), *reinterpret_cast<const uint32_t*>(g + 12));
+            } else {
+              uint32_t w[4];
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                w[q] = (uint32_t)*reinterpret_cast<const uint16_t*>(g + 4 * q) |
+                       ((uint32_t)*reinterpret_cast<const uint16_t*>(g + 4 * q + 2) << 16);
+              x[k] = make_uint4(w[0], w[1], w[2], w[3]);
+            }
           } else {
             const uint32_t n = min((uint32_t)S::VJ, nj - c * S::VJ) * ES;
             for (uint32_t e = 0; e < n; ++e) or_byte(x[k], e, g[e]);
@@ -259,12 +293,12 @@ __device__ __forceinline__ void move_subtile(const uint8_t* __restrict__ sp, uin
       }
     }
     const uint32_t jj0 = a * (uint32_t)S::VJ + dlo * S::CPR;
-    store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 0>(w, nan_bits), jj0, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+    store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 0>(w, nan_bits), jj0, ci, dp, ni, nj, dj_bytes, csum_base, align_dst, cs);
     if constexpr (S::CPR >= 2)
-      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 1>(w, nan_bits), jj0 + 1, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 1>(w, nan_bits), jj0 + 1, ci, dp, ni, nj, dj_bytes, csum_base, align_dst, cs);
     if constexpr (S::CPR == 4) {
-      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 2>(w, nan_bits), jj0 + 2, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
-      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 3>(w, nan_bits), jj0 + 3, ci, dp, ni, nj, dj_bytes, csum_base, vec_dst, cs);
+      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 2>(w, nan_bits), jj0 + 2, ci, dp, ni, nj, dj_bytes, csum_base, align_dst, cs);
+      store_chunk<ES, OP, FULL>(make_chunk<ES, OP, 3>(w, nan_bits), jj0 + 3, ci, dp, ni, nj, dj_bytes, csum_base, align_dst, cs);
     }
   }
 }
@@ -305,11 +339,11 @@ __device__ __forceinline__ void transpose_tile(const uint8_t* __restrict__ src, 
     uint8_t* dp = dst + d_el * S::EO;
     const uint32_t csum_base = (uint32_t)(d_el * S::EO) + d.csum_bias;
     uint8_t* my_lds = lds + wave * S::kLdsBytes;
-    if (d.vec_src && d.vec_dst && ni == (uint32_t)S::RI && nj == (uint32_t)S::TJ)
-      move_subtile<ES, OP, true>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, true, true, nan_bits, my_lds, cs);
+    if (d.align_src >= 16u && d.align_dst >= 16u && ni == (uint32_t)S::RI && nj == (uint32_t)S::TJ)
+      move_subtile<ES, OP, true>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, 16u, 16u, nan_bits, my_lds, cs);
     else
-      move_subtile<ES, OP, false>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, d.vec_src != 0, d.vec_dst != 0,
-                                  nan_bits, my_lds, cs);
+      move_subtile<ES, OP, false>(sp, dp, ni, nj, d.si * ES, d.dj * S::EO, csum_base, d.align_src, d.align_dst, nan_bits,
+                                  my_lds, cs);
   }
 }
 
