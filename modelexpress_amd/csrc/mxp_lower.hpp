@@ -43,23 +43,26 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
     if (pitched && (b.dst_pitch % m_dst || b.src_pitch % m_src)) return false;
     return true;
   };
+  // The unit is set by the destination side (whole, aligned stores); the source only has to be
+  // element aligned, the device reads it with loads that carry no alignment promise.
   uint32_t unit;
   if (op_narrows(b.op)) {
-    if (all_mult(8, 16)) unit = 8;
+    if (all_mult(8, 4)) unit = 8;
     else if (all_mult(2, 4)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
   } else if (op_widens(b.op)) {
-    if (all_mult(16, 8)) unit = 16;
-    else if (all_mult(4, 2)) unit = 4;
+    const uint64_t se = op_dst_elem(b.op) / 2;  // source element
+    if (all_mult(16, se)) unit = 16;
+    else if (all_mult(4, se)) unit = 4;
     else if (op_dst_elem(b.op) == 2 && all_mult(2, 1)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
   } else if (op_recodes16(b.op)) {
-    if (all_mult(16, 16)) unit = 16;
-    else if (all_mult(4, 4)) unit = 4;
+    if (all_mult(16, 2)) unit = 16;
+    else if (all_mult(4, 2)) unit = 4;
     else if (all_mult(2, 2)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
   } else {
-    unit = all_mult(16, 16) ? 16 : all_mult(4, 4) ? 4 : 1;
+    unit = all_mult(16, 1) ? 16 : all_mult(4, 1) ? 4 : 1;
   }
   const uint64_t max_pitch = pitched ? std::max(b.src_pitch, b.dst_pitch) : std::max(b.row_bytes, src_row);
   if (max_pitch >= (1ull << 31)) throw std::invalid_argument("row pitch of 2 GiB or more is not supported");
@@ -103,7 +106,6 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
                       std::vector<WorkItem>& work) {
   if (in.rows == 0 || in.row_bytes == 0) return;
   const uint32_t op = in.op;
-  const bool is_cast = op_narrows(op) || op_widens(op) || op_recodes16(op);
   BoxCopy b = in;
   // Rows that abut in both layouts are one contiguous run.
   if (b.rows > 1 && b.src_pitch == op_src_bytes(op, b.row_bytes) && b.dst_pitch == b.row_bytes) {
@@ -111,10 +113,21 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
     b.rows = 1;
   }
   if (b.rows == 1) {
-    // Contiguous run: full virtual rows of flat_row_bytes, then one short row.
+    // Contiguous run: a head up to the destination's next 16-byte boundary (so that the rest
+    // moves in whole aligned stores whatever the source's alignment), full virtual rows of
+    // flat_row_bytes, then one short row.
     const uint64_t W = o.flat_row_bytes;
-    uint64_t full = b.row_bytes / W;
     uint64_t done = 0;
+    if (b.dst_off % 16 && op != kOpChecksumOnly) {
+      const uint64_t head = std::min<uint64_t>(16 - b.dst_off % 16, b.row_bytes);
+      BoxCopy m = b;
+      m.row_bytes = head;
+      m.src_pitch = op_src_bytes(op, head);
+      m.dst_pitch = head;
+      emit_seg(m, o, segs, work);
+      done = head;
+    }
+    uint64_t full = (b.row_bytes - done) / W;
     while (full) {
       const uint64_t n = std::min<uint64_t>(full, 0x80000000ull);
       BoxCopy m = b;
@@ -131,7 +144,7 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
     const uint64_t rem = b.row_bytes - done;
     if (rem) {
       // Keep the 16-byte path for as much of the remainder as possible.
-      const uint64_t body = is_cast ? rem : (rem / 16) * 16;
+      const uint64_t body = (rem / 16) * 16;
       BoxCopy m = b;
       m.rows = 1;
       if (body) {
