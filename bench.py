@@ -38,7 +38,7 @@ HBM_PEAK_GBPS = 8000.0
 # counter scaled by its reading for a plain 1 GiB device copy).  Counters cannot be read
 # from inside this process, so the figure is carried here and reported only when the
 # workload is the profiled one.
-PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_097_600_000}
+PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_097_800_000}
 
 
 def _log(msg: str) -> None:
