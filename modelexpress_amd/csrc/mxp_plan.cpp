@@ -489,12 +489,12 @@ struct Planner {
         if (contains(t.name, g.member + ".") || ends_with(t.name, g.member + ".weight")) {
           const int64_t fp = find_param(replace_all(t.name, g.member, g.fused));
           if (fp < 0) continue;
-          auto it = group_index.find(fp);
-          if (it == group_index.end()) {
-            it = group_index.emplace(fp, groups.size()).first;
+          auto slot = group_index.find(fp);
+          if (slot == group_index.end()) {
+            slot = group_index.emplace(fp, groups.size()).first;
             groups.emplace_back(fp, std::vector<Member>());
           }
-          groups[it->second].second.push_back(Member{g.order, t.name, t.shape});
+          groups[slot->second].second.push_back(Member{g.order, t.name, t.shape});
           break;
         }
       }
