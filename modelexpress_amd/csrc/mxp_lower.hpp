@@ -162,6 +162,23 @@ inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>
     }
     return;
   }
+  // Pitched box whose rows all start at the same distance from a 16-byte boundary of the
+  // destination, but not on one (or do not end on one): a column of head bytes, a body that is
+  // stored whole and aligned, a column of tail bytes.
+  if (op != kOpChecksumOnly && b.dst_pitch % 16 == 0 && (b.dst_off % 16 || b.row_bytes % 16) && b.row_bytes >= 64) {
+    const uint64_t head = (16 - b.dst_off % 16) % 16;
+    const uint64_t body = (b.row_bytes - head) / 16 * 16;
+    const uint64_t cuts[4] = {0, head, head + body, b.row_bytes};
+    for (int k = 0; k < 3; ++k) {
+      if (cuts[k + 1] == cuts[k]) continue;
+      BoxCopy m = b;
+      m.src_off = b.src_off + op_src_bytes(op, cuts[k]);
+      m.dst_off = b.dst_off + cuts[k];
+      m.row_bytes = cuts[k + 1] - cuts[k];
+      lower_box(m, o, segs, work);  // the body is aligned now, the edge columns are narrower than 64 bytes
+    }
+    return;
+  }
   // Pitched box: split columns so a row fits max_row_bytes, rows so the count fits 32 bits.
   for (uint64_t c = 0; c < b.row_bytes; c += o.max_row_bytes) {
     const uint64_t cw = std::min<uint64_t>(o.max_row_bytes, b.row_bytes - c);

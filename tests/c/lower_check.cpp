@@ -4,6 +4,8 @@
 //   * every destination byte of the box is written exactly once, from the source byte the box
 //     pairs it with (through the conversion's size ratio), and nothing else is written;
 //   * every store is whole and aligned to its unit, every load is element aligned;
+//   * a contiguous run, and a pitched box whose destination pitch is a multiple of 16, move
+//     all but fewer than 32 bytes per row through the widest path, whatever the offsets are;
 //   * the reciprocal multiplication the kernel uses in place of a division is exact for every
 //     unit of every tile, in-tile offsets fit 32 bits, and a tile of the wide paths is at most
 //     one batch of the workgroup.
@@ -50,6 +52,7 @@ void check_box(const BoxCopy& b, const LowerOptions& lo) {
   // destination byte -> source byte (relative to the box origins), or -1 where the box writes nothing
   std::vector<int64_t> want(d_span, -1), got(d_span, -1);
   std::vector<uint8_t> hits(d_span, 0);
+  uint64_t wide_bytes = 0;
   const uint64_t ratio_n = op_narrows(b.op) ? 2 : 1, ratio_d = op_widens(b.op) ? 2 : 1;  // src = dst * n / d
   for (uint64_t r = 0; r < b.rows; ++r)
     for (uint64_t c = 0; c < b.row_bytes; ++c) {
@@ -57,7 +60,6 @@ void check_box(const BoxCopy& b, const LowerOptions& lo) {
       // byte c of a destination row comes from the element c / e of the source row
       want[r * b.dst_pitch + c] = (int64_t)(r * b.src_pitch + (c / e) * e * ratio_n / ratio_d);
     }
-  (void)src_row;
   for (const WorkItem& w : work) {
     REQUIRE(w.seg < segs.size(), "work item names segment %u of %zu", w.seg, segs.size());
     const Seg& s = segs[w.seg];
@@ -84,6 +86,7 @@ void check_box(const BoxCopy& b, const LowerOptions& lo) {
       if (s.op != kOpChecksumOnly) REQUIRE(da % unit == 0, "store of %u bytes at destination offset %" PRIu64, unit, da);
       REQUIRE(sa % src_elem(s.op) == 0, "load at source offset %" PRIu64 " is not element aligned", sa);
       REQUIRE(da >= b.dst_off && da + unit <= b.dst_off + d_span, "store outside the box");
+      if (unit == 16 || (narrow && unit == 8)) wide_bytes += unit;
       for (uint32_t k = 0; k < unit; ++k) {
         const uint64_t at = da - b.dst_off + k;
         REQUIRE(hits[at] == 0, "destination byte %" PRIu64 " written twice", at);
@@ -92,6 +95,11 @@ void check_box(const BoxCopy& b, const LowerOptions& lo) {
         got[at] = (int64_t)(sa - b.src_off + (k / e) * e * ratio_n / ratio_d);
       }
     }
+  }
+  const bool abut = b.rows == 1 || (b.src_pitch == src_row && b.dst_pitch == b.row_bytes);
+  if (b.op != kOpChecksumOnly && (abut || (b.dst_pitch % 16 == 0 && b.row_bytes >= 64))) {
+    const uint64_t total = b.rows * b.row_bytes, slack = abut ? 32 : 32 * b.rows;
+    REQUIRE(wide_bytes + slack > total, "only %" PRIu64 " of %" PRIu64 " bytes take the wide path", wide_bytes, total);
   }
   for (uint64_t i = 0; i < d_span; ++i)
     REQUIRE(got[i] == want[i], "destination byte %" PRIu64 ": source %" PRId64 ", expected %" PRId64, i, got[i], want[i]);
@@ -129,7 +137,7 @@ BoxCopy random_box(std::mt19937_64& g) {
     b.dst_pitch = b.row_bytes;
     b.src_pitch = src_row;
   }
-  b.dst_off = (tidy ? 16 : de) * pick(0, 40);
+  b.dst_off = (tidy && g() % 2 ? 16 : de) * pick(0, 40);
   b.src_off = se * pick(0, 40);
   return b;
 }
