@@ -195,45 +195,60 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
       }
     }
   } else {
-    for (uint32_t v = threadIdx.x; v < n_units; v += kPlaceThreads) {
-      uint32_t so, d_o;
-      locate(v, so, d_o);
-      uint32_t x;
+    // The narrow paths (boxes the 16-byte grid does not fit): one unit of at most four bytes per
+    // lane and step, eight steps at a time - all their loads first, then the stores - so a lane
+    // keeps eight loads in flight here too.
+    auto load_raw = [&](uint32_t so) -> uint32_t {
       if constexpr (NARROW) {
         static_assert(UNIT == 2, "the element-wise cast path moves one element per lane");
-        x = narrow1<OP>(*reinterpret_cast<const uint32_t*>(src + so), nan_bits);
-        *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+        return *reinterpret_cast<const uint32_t*>(src + so);
       } else if constexpr (op_recodes16(OP)) {
-        if constexpr (UNIT == 4) {  // two elements per lane
-          x = recode2<OP>(*reinterpret_cast<const u32_u*>(src + so), nan_bits);
-          *reinterpret_cast<uint32_t*>(dst + d_o) = x;
-        } else {
-          static_assert(UNIT == 2, "one element per lane");
-          x = recode1<OP>(*reinterpret_cast<const uint16_t*>(src + so), nan_bits);
-          *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
-        }
+        static_assert(UNIT == 4 || UNIT == 2, "two elements or one per lane");
+        if constexpr (UNIT == 4) return *reinterpret_cast<const u32_u*>(src + so);
+        else return *reinterpret_cast<const uint16_t*>(src + so);
       } else if constexpr (OP == kOpCastF8E4M3Bf16) {
-        if constexpr (UNIT == 4) {  // two elements per lane
-          const uint32_t w = *reinterpret_cast<const u16_u*>(src + so);
-          x = f8e4m3_to_bf16_bits(w & 0xFFu) | (f8e4m3_to_bf16_bits(w >> 8) << 16);
-          *reinterpret_cast<uint32_t*>(dst + d_o) = x;
-        } else {
-          static_assert(UNIT == 2, "one element per lane");
-          x = f8e4m3_to_bf16_bits(src[so]);
-          *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
-        }
+        static_assert(UNIT == 4 || UNIT == 2, "two elements or one per lane");
+        if constexpr (UNIT == 4) return *reinterpret_cast<const u16_u*>(src + so);
+        else return src[so];
       } else if constexpr (WIDEN) {
         static_assert(UNIT == 4, "the element-wise cast path moves one element per lane");
-        x = widen1<OP>(*reinterpret_cast<const uint16_t*>(src + so));
-        *reinterpret_cast<uint32_t*>(dst + d_o) = x;
+        return *reinterpret_cast<const uint16_t*>(src + so);
       } else if constexpr (UNIT == 4) {
-        x = *reinterpret_cast<const u32_u*>(src + so);
-        if constexpr (OP != kOpChecksumOnly) *reinterpret_cast<uint32_t*>(dst + d_o) = x;
+        return *reinterpret_cast<const u32_u*>(src + so);
+      } else if constexpr (UNIT == 2) {
+        return *reinterpret_cast<const u16_u*>(src + so);
       } else {
-        x = src[so];
-        if constexpr (OP != kOpChecksumOnly) dst[d_o] = (uint8_t)x;
+        return src[so];
+      }
+    };
+    auto finish = [&](uint32_t raw, uint32_t d_o) {
+      uint32_t x;
+      if constexpr (NARROW) x = narrow1<OP>(raw, nan_bits);
+      else if constexpr (op_recodes16(OP)) x = UNIT == 4 ? recode2<OP>(raw, nan_bits) : recode1<OP>(raw, nan_bits);
+      else if constexpr (OP == kOpCastF8E4M3Bf16)
+        x = UNIT == 4 ? (f8e4m3_to_bf16_bits(raw & 0xFFu) | (f8e4m3_to_bf16_bits(raw >> 8) << 16)) : f8e4m3_to_bf16_bits(raw);
+      else if constexpr (WIDEN) x = widen1<OP>(raw);
+      else x = raw;
+      if constexpr (OP != kOpChecksumOnly) {
+        if constexpr (UNIT == 4) *reinterpret_cast<uint32_t*>(dst + d_o) = x;
+        else if constexpr (UNIT == 2) *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
+        else dst[d_o] = (uint8_t)x;
       }
       cs.add4(x, csum_base + d_o);
+    };
+    constexpr uint32_t G = 8;
+    for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += G * kPlaceThreads) {
+      uint32_t so[G], d_o[G], raw[G];
+#pragma unroll
+      for (uint32_t k = 0; k < G; ++k) {
+        const uint32_t v = v0 + k * kPlaceThreads;
+        locate(v < n_units ? v : v0, so[k], d_o[k]);  // a step past the end re-reads the lane's first unit and drops it
+      }
+#pragma unroll
+      for (uint32_t k = 0; k < G; ++k) raw[k] = load_raw(so[k]);
+#pragma unroll
+      for (uint32_t k = 0; k < G; ++k)
+        if (v0 + k * kPlaceThreads < n_units) finish(raw[k], d_o[k]);
     }
   }
 }
@@ -261,6 +276,7 @@ __device__ __forceinline__ void place_body(
     switch (s.unit) {
       case 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
       case 4u: run_tile<kOpChecksumOnly, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+      case 2u: run_tile<kOpChecksumOnly, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
       case 1u: run_tile<kOpChecksumOnly, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
       default: break;
     }
@@ -268,6 +284,7 @@ __device__ __forceinline__ void place_body(
   switch (s.op * 32u + s.unit) {
     case kOpCopy * 32u + 16u: run_tile<kOpCopy, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCopy * 32u + 4u: run_tile<kOpCopy, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpCopy * 32u + 2u: run_tile<kOpCopy, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCopy * 32u + 1u: run_tile<kOpCopy, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF32Bf16 * 32u + 8u: run_tile<kOpCastF32Bf16, 8>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpCastF32Bf16 * 32u + 2u: run_tile<kOpCastF32Bf16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;

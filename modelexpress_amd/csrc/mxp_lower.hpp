@@ -62,7 +62,7 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
     else if (all_mult(2, 2)) unit = 2;
     else throw std::invalid_argument("cast box is not element aligned");
   } else {
-    unit = all_mult(16, 1) ? 16 : all_mult(4, 1) ? 4 : 1;
+    unit = all_mult(16, 1) ? 16 : all_mult(4, 1) ? 4 : all_mult(2, 1) ? 2 : 1;
   }
   const uint64_t max_pitch = pitched ? std::max(b.src_pitch, b.dst_pitch) : std::max(b.row_bytes, src_row);
   if (max_pitch >= (1ull << 31)) throw std::invalid_argument("row pitch of 2 GiB or more is not supported");
