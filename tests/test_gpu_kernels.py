@@ -137,6 +137,19 @@ def test_cast_nan_image_is_a_parameter(mxp, oracle):
     assert d[:8].cpu().numpy().view(np.uint16).tolist() == [0xFFFF, 0xFFFF, 0xFFFF, 0x3F80]
     ref = torch.from_numpy(src.view(np.float32).copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
     assert ref[3] == 0x3F80 and all((int(v) & 0x7FFF) > 0x7F80 for v in ref[:3])
+    # the same image through the wide path (eight elements per lane), a converting transpose and fp16 -> bf16
+    big = np.tile(src, 4096)
+    d = torch.zeros(big.size * 2, dtype=torch.uint8, device="cuda")
+    eng.cast_f32_bf16(_dev(big), d, big.size)
+    assert np.array_equal(d.cpu().numpy().view(np.uint16), np.tile(np.array([0xFFFF, 0xFFFF, 0xFFFF, 0x3F80], dtype=np.uint16), 4096))
+    m = big.reshape(128, 128)
+    d = torch.zeros(m.size * 2, dtype=torch.uint8, device="cuda")
+    eng.copy_view(_dev(m), d, (128, 128), 2, src_strides=(1, 128), cast=oracle.CAST_CODES[("F32", "BF16")], checksum=False)
+    assert np.array_equal(d.cpu().numpy().view(np.uint16).reshape(128, 128), oracle.cast_f32_bf16_bits(m, 0xFFFF).astype(np.uint16).T)
+    h = np.tile(np.array([0x7C01, 0xFE00, 0x3C00, 0x7C00], dtype=np.uint16), 4096)
+    d = torch.zeros(h.size * 2, dtype=torch.uint8, device="cuda")
+    eng.cast(_dev(h), d, h.size, "F16", "BF16")
+    assert np.array_equal(d.cpu().numpy().view(np.uint16), np.tile(np.array([0xFFFF, 0xFFFF, 0x3F80, 0x7F80], dtype=np.uint16), 4096))
     eng.close()
 
 
