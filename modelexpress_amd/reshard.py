@@ -83,13 +83,25 @@ def execute_recorded_copies(engine: PlacementEngine, copies: Sequence[RecordedCo
             raise UnsupportedReshard(f"{c.param_name}: destination view leaves the parameter's storage")
         resolved.append((src.data_ptr() + off * src.element_size(), dst.data_ptr() + c.dest_offset * dst.element_size(),
                          shape, stride, tuple(int(s) for s in c.dest_stride), dst.element_size(), cast))
+    # One call moves every view whose destination span is clear of the others'; a view whose span
+    # (first to last byte it can touch, holes included - the conservative test of
+    # refit/reshard/receiver.py:289-321) meets an earlier one's starts a new call, so overlapping
+    # views land in plan order as the reference's sequential fallback does.
     written = 0
-    views = []
+    batch: list[dict] = []
+    spans: list[tuple[int, int]] = []
     for sp, dp, shape, ss, ds, es, cast in resolved:
-        views.append({"src": sp, "dst": dp, "shape": shape, "elem_size": es, "src_strides": ss, "dst_strides": ds, "cast": cast})
+        lo = dp
+        hi = dp + (sum((n - 1) * st for n, st in zip(shape, ds)) + 1) * es
+        if any(lo < b and a < hi for a, b in spans):
+            engine.copy_views(batch, stream=stream)
+            batch, spans = [], []
+        batch.append({"src": sp, "dst": dp, "shape": shape, "elem_size": es, "src_strides": ss, "dst_strides": ds, "cast": cast})
+        spans.append((lo, hi))
         n = es
         for v in shape:
             n *= v
         written += n
-    engine.copy_views(views, stream=stream)  # one launch for every row / element box, one per transposed view
+    if batch:
+        engine.copy_views(batch, stream=stream)  # one launch for every row / element box, one per kind of transposed view
     return written

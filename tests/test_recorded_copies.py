@@ -211,3 +211,91 @@ def test_many_transposed_copies_share_launches(gpu_engine):
             assert torch.equal(params[name].cpu().view(torch.uint8), want.view(torch.uint8)), name
         for p in params.values():
             p.fill_(7)
+
+
+def test_expert_unbind_chain_resolves_to_the_rank_slice():
+    # test_reshard_refit_moe_experts.py:127-158: expert 1's up_proj, TP rank 0 of 2, INTER=8, HIDDEN=4 fp32 -
+    # unsqueeze(0) / unbind() cancel, the view is this rank's INTER/2 rows from the start of the source
+    chain = (("unsqueeze", (0,), ()), ("unbind", (), ()), ("__getitem__", (0,), ()), ("narrow", (0, 0, 4), ()))
+    off, shape, stride = replay_view(chain, (8, 4))
+    assert (off, shape, stride) == (0, (4, 4), (4, 1))
+    assert shape[0] * shape[1] * 4 == 64  # "pulled == INTER_PER_TP * HIDDEN * 4"; rank 0 reads from source byte 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("inter,hidden,experts,tp", [(8, 4, 2, 2), (768, 2048, 8, 4)])
+def test_per_expert_sources_into_fused_w13(gpu_engine, inter, hidden, experts, tp):
+    """Per-expert HF sources (``experts.<e>.gate_proj`` / ``up_proj``) scattered into the fused grouped-expert
+    buffer ``w13 [local_experts, 2 * inter / tp, hidden]`` through the chain vLLM's expert loader records
+    (test_reshard_refit_moe_experts.py:41-78): one copy per (expert, projection), against the loader run on the CPU."""
+    per = inter // tp
+    g = torch.Generator().manual_seed(3)
+    for rank in (0, tp - 1):
+        want = torch.full((experts, 2 * per, hidden), 7, dtype=torch.bfloat16)
+        sources, copies = {}, []
+        for e in range(experts):
+            for member, proj in enumerate(("gate_proj", "up_proj")):
+                name = f"model.layers.0.mlp.experts.{e}.{proj}.weight"
+                src = torch.randn(inter, hidden, generator=g)  # the trainer publishes fp32
+                sources[name] = src.cuda()
+                want[e].narrow(0, member * per, per).copy_(src.unsqueeze(0).unbind()[0].narrow(0, rank * per, per))
+                chain = (("unsqueeze", (0,), ()), ("unbind", (), ()), ("__getitem__", (0,), ()), ("narrow", (0, rank * per, per), ()))
+                copies.append(RecordedCopy(name, chain, "w13_weight", (e * 2 * per + member * per) * hidden, (per, hidden), (hidden, 1),
+                                           torch.bfloat16))
+        param = torch.full((experts, 2 * per, hidden), 7, dtype=torch.bfloat16, device="cuda")
+        n = execute_recorded_copies(gpu_engine, copies, sources, {"w13_weight": param})
+        assert n == want.numel() * 2
+        assert torch.equal(param.cpu().view(torch.int16), want.view(torch.int16)), rank
+
+
+def _batch_install_plan():
+    """test_reshard_refit_batch_install.py:62-160: a 4x6 fp32 source re-sliced into three column blocks
+    (q, k, v) and a 4x4 source re-sliced into two row blocks of one buffer - five views over two sources."""
+    sources = {"qkv": torch.arange(24, dtype=torch.float32).reshape(4, 6),
+               "rows": torch.arange(100, 116, dtype=torch.float32).reshape(4, 4)}
+    copies = [RecordedCopy("qkv", (("narrow", (1, start, 2), ()),), name, 0, (4, 2), (2, 1))
+              for name, start in (("q", 0), ("k", 2), ("v", 4))]
+    copies += [RecordedCopy("rows", (("narrow", (0, start, 2), ()),), "rows", start * 4, (2, 4), (4, 1)) for start in (0, 2)]
+    params = {"q": torch.zeros(4, 2), "k": torch.zeros(4, 2), "v": torch.zeros(4, 2), "rows": torch.zeros(4, 4)}
+    return sources, copies, params
+
+
+@pytest.mark.gpu
+def test_batch_install_reconstructs_the_expected_values(gpu_engine):
+    # test_reshard_refit_batch_install.py:183-196
+    sources, copies, params = _batch_install_plan()
+    dev = {k: v.cuda() for k, v in params.items()}
+    n = execute_recorded_copies(gpu_engine, copies, {k: v.cuda() for k, v in sources.items()}, dev)
+    assert n == (24 + 16) * 4
+    for name, start in (("q", 0), ("k", 2), ("v", 4)):
+        assert torch.equal(dev[name].cpu(), sources["qkv"][:, start:start + 2]), name
+    assert torch.equal(dev["rows"].cpu(), sources["rows"])
+
+
+@pytest.mark.gpu
+def test_overlapping_destinations_land_in_plan_order(gpu_engine):
+    # test_reshard_refit_batch_install.py:219-238: both row blocks aimed at offset 0 - the later copy wins
+    sources, copies, params = _batch_install_plan()
+    for c in copies[3:]:
+        c.dest_offset = 0
+    dev = {k: v.cuda() for k, v in params.items()}
+    execute_recorded_copies(gpu_engine, copies, {k: v.cuda() for k, v in sources.items()}, dev)
+    assert torch.equal(dev["rows"].cpu()[:2], torch.arange(108, 116, dtype=torch.float32).reshape(2, 4))
+    assert torch.equal(dev["rows"].cpu()[2:], torch.zeros(2, 4))
+
+
+@pytest.mark.gpu
+def test_interleaved_column_blocks_of_one_parameter(gpu_engine):
+    """Three column blocks written into ONE fused parameter: their spans interleave (the conservative
+    test of receiver.py:289-321 calls that overlapping), so they run one after another - same bytes."""
+    src = torch.arange(24, dtype=torch.float32).reshape(4, 6).cuda()
+    fused = torch.zeros(4, 6, device="cuda")
+    copies = [RecordedCopy("qkv", (("narrow", (1, start, 2), ()),), "fused", start, (4, 2), (6, 1)) for start in (4, 0, 2)]
+    execute_recorded_copies(gpu_engine, copies, {"qkv": src}, {"fused": fused})
+    assert torch.equal(fused, src)
+
+
+@pytest.mark.gpu
+def test_no_copies_is_a_no_op(gpu_engine):
+    # test_reshard_refit_batch_install.py:269-284
+    assert execute_recorded_copies(gpu_engine, [], {}, {}) == 0
