@@ -122,3 +122,31 @@ def test_gated_virtuals_and_coverage_gate(oracle, mxp, tmp_path):
     with pytest.raises(MxpError, match="not in the checkpoint"):
         PlacementPlan(ck, [], virtual_tensors=[VirtualTensor("x", (2, 3), (("nope", (0, 0), (0, 0), (2, 3)),))],
                       allow_unmapped=True, allow_uncovered=True)
+
+
+def test_reference_alias_vectors():
+    """The reference's own alias cases (tests/test_reshard_megatron.py:345-470), as virtual-tensor shards
+    ``(source, offset in the source, offset in the HF tensor, shape)``."""
+    from modelexpress_amd.megatron import gated_virtuals, qkv_virtuals
+
+    # :345-368 a [gate; up] shard of TP rank 1 of 2, local (8, 4) of global (16, 4): gate and up are (8, 4)
+    # globally, this rank's halves are (4, 4) at rows 4.., read from local rows 0 and 4
+    gate, up = gated_virtuals([("linear_fc1.weight", 1, 2)], ("gate_proj.weight", "up_proj.weight"), (4,), global_rows=16)
+    assert gate.shape == up.shape == (8, 4)
+    assert gate.shards == (("linear_fc1.weight", (0, 0), (4, 0), (4, 4)),)
+    assert up.shards == (("linear_fc1.weight", (4, 0), (4, 0), (4, 4)),)
+    # :372-417 the storage order must be stated and must be gate-then-up
+    with pytest.raises(ValueError, match="gate_then_up"):
+        gated_virtuals([("linear_fc1.weight", 1, 2)], ("gate_proj.weight", "up_proj.weight"), (4,), global_rows=16, order="up_then_gate")
+    # :443-475 fused QKV rows 12..24 of 24 (TP rank 1 of 2; 4 local query heads, 1 local KV head, head_dim 2):
+    # q is (16, 4) globally and this rank's 8 rows land at row 8 from local row 0; k and v are (4, 4) and
+    # this rank's 2 rows land at row 2, from local rows 8 and 10
+    q, k, v = qkv_virtuals([("linear_qkv.weight", 12, 24)], ("q_proj.weight", "k_proj.weight", "v_proj.weight"), 4,
+                           head_dim=2, q_heads=8, kv_heads=2)
+    assert (q.shape, k.shape, v.shape) == ((16, 4), (4, 4), (4, 4))
+    assert q.shards == (("linear_qkv.weight", (0, 0), (8, 0), (8, 4)),)
+    assert k.shards == (("linear_qkv.weight", (8, 0), (2, 0), (2, 4)),)
+    assert v.shards == (("linear_qkv.weight", (10, 0), (2, 0), (2, 4)),)
+    # :503-527 a shard range beyond the global extent is rejected
+    with pytest.raises(ValueError, match="row interval"):
+        qkv_virtuals([("linear_qkv.weight", 12, 26)], ("q", "k", "v"), 4, head_dim=2, q_heads=8, kv_heads=2)

@@ -288,6 +288,36 @@ def test_paired_runs_reference_vectors(oracle):
     assert list(oracle.paired_runs([(2, 4), (0, 8)], (0, 0), [8, 1], (2, 0), [8, 1])) == [(16, 0, 16)]
 
 
+@pytest.mark.parametrize("tp_size,tp_rank,expected_bytes,expected_segments", [(2, 1, 272, 3), (4, 2, 144, 10)])
+def test_paired_runs_megatron_target_vectors(oracle, tp_size, tp_rank, expected_bytes, expected_segments):
+    """tests/test_reshard_megatron.py:30-113: bf16 sources published by two trainer ranks - expert_fc1 (16, 8)
+    split on rows, expert_fc2 (8, 16) split on columns, a replicated norm (8,) - pulled by a TP rank that owns
+    rows / columns / everything.  The reference expects 272 bytes in 3 segments (TP 2, rank 1) and 144 bytes in
+    10 segments (TP 4, rank 2): every (destination box x source shard) intersection decomposed into runs."""
+    sources = {"expert_fc1": ((16, 8), [((0, 0), (8, 8)), ((8, 0), (8, 8))]),
+               "expert_fc2": ((8, 16), [((0, 0), (8, 8)), ((0, 8), (8, 8))]),
+               "norm": ((8,), [((0,), (8,))])}
+    wanted = {"expert_fc1": 0, "expert_fc2": 1, "norm": None}  # the axis the destination rank owns a slice of
+    n_bytes = n_segments = 0
+    for name, (shape, shards) in sources.items():
+        axis = wanted[name]
+        dst_box = [(0, n) for n in shape]
+        if axis is not None:
+            per = shape[axis] // tp_size
+            dst_box[axis] = (tp_rank * per, (tp_rank + 1) * per)
+        dst_shape = [hi - lo for lo, hi in dst_box]
+        for off, sshape in shards:
+            src_box = [(o, o + n) for o, n in zip(off, sshape)]
+            overlap = oracle.intersect(dst_box, src_box)
+            if overlap is None:
+                continue
+            for _s, _d, run in oracle.paired_runs(overlap, off, oracle.row_major_strides(sshape), [lo for lo, _ in dst_box],
+                                                  oracle.row_major_strides(dst_shape)):
+                n_bytes += run * 2
+                n_segments += 1
+    assert (n_bytes, n_segments) == (expected_bytes, expected_segments)
+
+
 def test_paired_runs_brute_force(oracle):
     rng = np.random.default_rng(4)
     for _ in range(50):
