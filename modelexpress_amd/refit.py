@@ -28,6 +28,7 @@ from typing import Any
 import torch
 
 from .adapter import PlacementLayout
+from ._lib import DTYPE_SIZE
 from .engine import Checkpoint, PlacementEngine, PlacementPlan
 from .timing import RefitTimingRecorder
 
@@ -41,6 +42,10 @@ class RefitInputs:
     layout_signature: str = ""
     expected_digests: dict = field(default_factory=dict)  # parameter name -> 32 hex chars
     require_digests: bool = False
+    # parameter name -> [(shard_offset, shape, digest or None), ...]: the digest of each publisher's
+    # region of the parameter, the granularity the reference stamps and checks
+    # (modelexpress_rl/inference/nixl_staged_transfer.py:529-549: one digest per source shard)
+    expected_shard_digests: dict = field(default_factory=dict)
 
     @property
     def physical_fingerprint(self) -> tuple:
@@ -132,6 +137,25 @@ class HipRefitAdapter:
             if want != got:
                 raise RuntimeError(f"refit {inputs.version_id}: digest mismatch for {name}: "
                                    f"published {want}, staged {got}")
+        if not inputs.expected_shard_digests:
+            return
+        params = {p.name: (p, buf) for p, buf in zip(staged.plan.plan.params, staged.buffers)}
+        regions, wanted = [], []
+        for name, shards in inputs.expected_shard_digests.items():
+            if name not in params:
+                raise RuntimeError(f"refit {inputs.version_id}: source {name!r} is not a parameter of this plan")
+            spec, buf = params[name]
+            itemsize = DTYPE_SIZE[spec.dtype]
+            for offset, shape, digest in shards:
+                if not digest:
+                    raise RuntimeError(f"source {name!r} did not publish a verification digest")
+                region, _ = self.engine.shard_region(buf, spec.shape, offset, shape, itemsize)
+                regions.append(region)
+                wanted.append((name, tuple(offset), digest))
+        got = self.engine.digest(regions, [r.numel() for r in regions]) if regions else []
+        for (name, offset, want), have in zip(wanted, got):
+            if want != have:
+                raise RuntimeError(f"staged weight digest mismatch for source {name!r} at offset {offset}")
 
     def apply_weight(self, staged: StagedWeights) -> dict:
         names = [p.name for p in staged.plan.plan.params]

@@ -210,8 +210,36 @@ def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
     plan = ad.create_transfer_plan(RefitInputs("v1", str(new), "sig", {}, require_digests=True))
     with pytest.raises(RuntimeError, match="no published digest"):
         ad.stage_weight(plan)
+    # digests per publisher shard (nixl_staged_transfer.py:529-549; tests/test_refit_nixl_staged_transfer.py:192-203):
+    # every 2-D parameter as two row halves, each with the digest of its own region
+    def shard_table(tamper=None, drop=None):
+        table = {}
+        for n, t in want.items():
+            if len(t.shape) != 2 or t.shape[0] % 2:
+                continue
+            half = t.shape[0] // 2
+            rows = []
+            for k in range(2):
+                region = oracle.shard_region(t, t.shape, (k * half, 0), (half, t.shape[1]))
+                d = oracle.tensor_digest(region)
+                if (n, k) == tamper:
+                    d = "f" * 32
+                if (n, k) == drop:
+                    d = None
+                rows.append(((k * half, 0), (half, t.shape[1]), d))
+            table[n] = rows
+        return table
+
+    victim = next(iter(shard_table()))
+    plan = ad.create_transfer_plan(RefitInputs("v1", str(new), "sig", digests, True, shard_table(tamper=(victim, 1))))
+    with pytest.raises(RuntimeError, match=r"staged weight digest mismatch for source .* at offset \(\d+, 0\)"):
+        ad.stage_weight(plan)
+    plan = ad.create_transfer_plan(RefitInputs("v1", str(new), "sig", digests, True, shard_table(drop=(victim, 0))))
+    with pytest.raises(RuntimeError, match="did not publish a verification digest"):
+        ad.stage_weight(plan)
+    assert {n: p.data.view(torch.uint8).cpu().numpy().tobytes() for n, p in model.named_parameters()} == v0
     # the good path
-    inputs = RefitInputs("v1", str(new), "sig", digests, require_digests=True)
+    inputs = RefitInputs("v1", str(new), "sig", digests, require_digests=True, expected_shard_digests=shard_table())
     plan = ad.create_transfer_plan(inputs)
     assert ad.validate_transfer_plan(plan, inputs)
     assert not ad.validate_transfer_plan(plan, RefitInputs("v2", str(new), "other-layout", digests))
