@@ -23,6 +23,16 @@ def _env_int(name: str, default: int) -> int:
         return default
 
 
+def _env_float(name: str, default: float) -> float:
+    raw = os.environ.get(name, "").strip()
+    if not raw:
+        return default
+    try:
+        return float(raw)
+    except ValueError:
+        return default
+
+
 def _env_bool(name: str, default: bool) -> bool:
     raw = os.environ.get(name)
     if raw is None or not raw.strip():
@@ -48,6 +58,10 @@ environment_variables: dict[str, Callable[[], Any]] = {
     "MXP_VERIFY_CHECKSUMS": lambda: _env_bool("MXP_VERIFY_CHECKSUMS", True),
     # Allow fp32 checkpoints to be cast into bf16 parameters (refit).
     "MXP_ALLOW_CAST": lambda: _env_bool("MXP_ALLOW_CAST", False),
+    # Coverage gate of a refit, same names and defaults as the reference (modelexpress/envs.py:266-272):
+    # refuse a refit that writes less than the floor fraction of the engine's parameter bytes.
+    "MX_RESHARD_REQUIRE_FULL_COVERAGE": lambda: _env_bool("MX_RESHARD_REQUIRE_FULL_COVERAGE", False),
+    "MX_RESHARD_COVERAGE_FLOOR": lambda: _env_float("MX_RESHARD_COVERAGE_FLOOR", 0.995),
 }
 
 

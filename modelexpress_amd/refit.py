@@ -22,15 +22,22 @@ that waives the "untouched until verified" guarantee and is therefore explicit.
 
 from __future__ import annotations
 
+import json
+import logging
 from dataclasses import dataclass, field
 from typing import Any
 
 import torch
 
+from . import envs
 from .adapter import PlacementLayout
 from ._lib import DTYPE_SIZE
+from .mla import IncompleteRefit
 from .engine import Checkpoint, PlacementEngine, PlacementPlan
 from .timing import RefitTimingRecorder
+
+
+logger = logging.getLogger("modelexpress_amd.refit")
 
 
 @dataclass(frozen=True)
@@ -78,6 +85,70 @@ def _null():
     return contextlib.nullcontext()
 
 
+def coverage_floor() -> float:
+    """The fraction of engine parameter bytes a gated refit must install; outside [0, 1] is an
+    error rather than a gate that passes or rejects everything (refit/reshard/receiver.py:236-259)."""
+    floor = float(envs.MX_RESHARD_COVERAGE_FLOOR)
+    if not 0.0 <= floor <= 1.0:
+        raise ValueError(f"MX_RESHARD_COVERAGE_FLOOR must be a fraction in [0.0, 1.0], got {floor}")
+    return floor
+
+
+def log_coverage(param_layout: dict, all_params, *, rank: int = 0, copies_captured: int = 0, unsupported=(),
+                 plan_stats: dict | None = None) -> dict:
+    """What a refit will write against what the engine holds, as one ``MX_REFIT_COVERAGE`` JSON record
+    (refit/reshard/receiver.py:661-755, schema ``refit-coverage-v1``).  ``param_layout`` maps every engine
+    parameter to ``(shape, torch dtype or safetensors dtype name)``; ``all_params`` names the ones this refit
+    writes.  Coverage is a byte ratio: half the parameters can be far from half the bytes.  INFO when
+    complete, WARNING otherwise; with ``MX_RESHARD_REQUIRE_FULL_COVERAGE`` set, coverage below
+    ``MX_RESHARD_COVERAGE_FLOOR`` raises ``IncompleteRefit``.  Returns the record."""
+    installed = set(all_params)
+    dest_bytes = engine_bytes = 0
+    missed = []
+    for name, (shape, dtype) in param_layout.items():
+        count = 1
+        for dim in shape:
+            count *= int(dim)
+        width = DTYPE_SIZE[dtype] if isinstance(dtype, str) else torch.empty(0, dtype=dtype).element_size()
+        engine_bytes += count * width
+        if name in installed:
+            dest_bytes += count * width
+        else:
+            missed.append(name)
+    coverage = (dest_bytes / engine_bytes) if engine_bytes else 0.0
+    unsupported = list(unsupported or [])
+    stats = plan_stats or {}
+    record = {
+        "schema": "refit-coverage-v1",
+        "rank": rank,
+        "params_installed": len(list(all_params)),
+        "engine_params": len(param_layout),
+        "dest_bytes": dest_bytes,
+        "engine_bytes": engine_bytes,
+        "coverage_pct": round(100.0 * coverage, 4),
+        "params_never_written": len(missed),
+        "params_never_written_sample": sorted(missed)[:10],
+        "copies_captured": copies_captured,
+        "unsupported": len(unsupported),
+        "unsupported_sample": [str(u)[:120] for u in unsupported[:10]],
+        # the plan's economics ride on the same record: bytes over the wire (here: over PCIe) against useful bytes
+        "planned_wire_bytes": int(stats.get("planned_wire_bytes", 0)),
+        "extra_wire_bytes": int(stats.get("extra_wire_bytes", 0)),
+        "descriptors": int(stats.get("descriptors", 0)),
+        "converts": int(stats.get("converts", 0)),
+        "fallback": int(stats.get("fallback", 0)),
+    }
+    complete = not missed and not unsupported and not record["fallback"]
+    logger.log(logging.INFO if complete else logging.WARNING, "MX_REFIT_COVERAGE %s", json.dumps(record))
+    if envs.MX_RESHARD_REQUIRE_FULL_COVERAGE and coverage < coverage_floor():
+        raise IncompleteRefit(
+            f"refit covers {100.0 * coverage:.2f}% of the engine's parameter bytes ({dest_bytes} of {engine_bytes}); "
+            f"{len(missed)} of {len(param_layout)} params would keep their previous values, e.g. {sorted(missed)[:5]}. "
+            f"No digest gate can detect this - bytes that are never requested are never checked. "
+            f"Set MX_RESHARD_REQUIRE_FULL_COVERAGE=0 for an intentionally partial refit.")
+    return record
+
+
 class HipRefitAdapter:
     """Refit executor for one rank's resident parameters."""
 
@@ -87,6 +158,7 @@ class HipRefitAdapter:
                  in_place: bool = False):
         self.timing: RefitTimingRecorder | None = None  # the record of the cycle in progress
         self._plans_built = 0
+        self.coverage: dict | None = None  # the MX_REFIT_COVERAGE record of the last plan
         self.layout = layout
         self.device = device
         self.in_place = in_place
@@ -103,6 +175,16 @@ class HipRefitAdapter:
                                  stacked_params_mapping=lay.stacked_params_mapping, expert_mapping=lay.expert_mapping,
                                  skip_prefixes=lay.skip_prefixes, allow_cast=True)
         self._plans_built += 1
+        # What this refit will write against everything the engine holds; with the gate on, an
+        # incomplete plan stops here, before any byte moves.
+        info = plan.param_info()
+        self.engine.prepare(plan)  # lowers the plan for this engine: its byte totals are complete afterwards
+        totals = plan.totals()
+        self.coverage = log_coverage(
+            {p["name"]: (p["shape"], p["dtype"]) for p in info}, [p["name"] for p in info if p["bytes_written"] == p["nbytes"]],
+            rank=lay.tp_rank, copies_captured=sum(p["n_writes"] for p in info),
+            plan_stats={"planned_wire_bytes": totals["h2d_bytes"], "extra_wire_bytes": totals["h2d_bytes"] - totals["placed_bytes"],
+                        "descriptors": sum(p["n_writes"] for p in info)})
         return RefitPlan(inputs, ck, plan, inputs.physical_fingerprint)
 
     def validate_transfer_plan(self, plan: Any, inputs: RefitInputs) -> bool:

@@ -249,6 +249,9 @@ def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
     for n, p in model.named_parameters():
         assert p.data.view(torch.uint8).cpu().numpy().tobytes() == want[n].tobytes(), n
         assert sums[n] == oracle.safe_checksum(want[n])
+    assert ad.coverage["schema"] == "refit-coverage-v1" and ad.coverage["coverage_pct"] == 100.0
+    assert ad.coverage["engine_bytes"] == ad.coverage["dest_bytes"] == sum(p.nbytes for p in rv.params)
+    assert ad.coverage["planned_wire_bytes"] >= 2 * ad.coverage["dest_bytes"]  # fp32 over PCIe for bf16 parameters
     rec = ad.timing.as_dict()
     assert rec["backend"] == "hip_placement" and rec["version"] == "v1" and rec["bytes"] == sum(p.nbytes for p in rv.params)
     assert {"transfer_planning", "wire_transfer", "receive_sync", "installation"} <= set(rec["stages"])

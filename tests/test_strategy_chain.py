@@ -234,3 +234,75 @@ def test_manifest_comparison_rules(caplog):
     with pytest.raises(ManifestMismatchError, match="No matching tensors"):
         compare_manifests([], [], require_exact_match=True)
     assert compare_manifests([], []) == 0
+
+
+# ---------------------------------------------------------------- refit coverage record
+def _coverage(caplog, **kw):
+    import json
+    import logging
+
+    from modelexpress_amd.refit import log_coverage
+
+    caplog.clear()
+    with caplog.at_level(logging.INFO, logger="modelexpress_amd.refit"):
+        rec = log_coverage(**kw)
+    lines = [r for r in caplog.records if "MX_REFIT_COVERAGE" in r.getMessage()]
+    assert len(lines) == 1 and json.loads(lines[0].getMessage().split("MX_REFIT_COVERAGE ", 1)[1]) == rec
+    return rec, lines[0].levelname
+
+
+def test_coverage_record_reference_cases(caplog, monkeypatch):
+    """tests/test_reshard_refit_coverage.py:116-193: coverage is a byte ratio over the engine's complete
+    parameter set, dtype widths count, the missing names are sampled, severity follows the content."""
+    import torch
+
+    monkeypatch.delenv("MX_RESHARD_REQUIRE_FULL_COVERAGE", raising=False)
+    monkeypatch.delenv("MX_RESHARD_COVERAGE_FLOOR", raising=False)
+    names = [f"layers.{i}.weight" for i in range(4)]
+    rec, level = _coverage(caplog, param_layout={n: ((4, 8), torch.bfloat16) for n in names}, all_params=names)
+    assert (rec["coverage_pct"], rec["params_installed"], rec["engine_params"], rec["params_never_written"]) == (100.0, 4, 4, 0)
+    assert rec["dest_bytes"] == rec["engine_bytes"] and rec["params_never_written_sample"] == [] and level == "INFO"
+    # :127-143 48 engine layers, the first 24 installed: 50 %, and the sample names the missing ones
+    engine = [f"layers.{i}.weight" for i in range(48)]
+    rec, level = _coverage(caplog, param_layout={n: ((4, 8), "BF16") for n in engine}, all_params=engine[:24])
+    assert (rec["coverage_pct"], rec["params_installed"], rec["engine_params"], rec["params_never_written"]) == (50.0, 24, 48, 24)
+    assert rec["params_never_written_sample"][0].startswith("layers.2") and len(rec["params_never_written_sample"]) == 10
+    assert level == "WARNING"
+    # :146-162 bytes, not parameter count
+    rec, _ = _coverage(caplog, param_layout={"big": ((1024, 1024), torch.bfloat16), "small": ((1, 1), torch.bfloat16)},
+                       all_params=["small"])
+    assert rec["params_installed"] == 1 and rec["engine_params"] == 2 and rec["coverage_pct"] < 0.001 and rec["dest_bytes"] == 2
+    # :165-179 dtype widths
+    for dtype, width in ((torch.float8_e4m3fn, 1), (torch.bfloat16, 2), (torch.float32, 4), ("F8_E4M3", 1), ("F32", 4)):
+        rec, _ = _coverage(caplog, param_layout={"w": ((4, 8), dtype)}, all_params=["w"])
+        assert rec["engine_bytes"] == rec["dest_bytes"] == 32 * width, dtype
+    # :182-193 unsupported sources are counted, sampled and clipped
+    rec, level = _coverage(caplog, param_layout={n: ((4, 8), "BF16") for n in "ab"}, all_params=["a", "b"],
+                           unsupported=[f"cannot reshard {i} " + "x" * 200 for i in range(15)])
+    assert rec["unsupported"] == 15 and len(rec["unsupported_sample"]) == 10 and all(len(x) <= 120 for x in rec["unsupported_sample"])
+    assert level == "WARNING"
+    # :337-342 an engine with no parameters does not divide by zero
+    rec, _ = _coverage(caplog, param_layout={}, all_params=[])
+    assert rec["coverage_pct"] == 0.0
+
+
+def test_coverage_gate(caplog, monkeypatch):
+    """:278-366 the gate is off by default, raises below the floor naming what is missing, passes at the
+    floor, rejects a floor outside [0, 1], and reads its settings live."""
+    from modelexpress_amd.mla import IncompleteRefit
+
+    engine = [f"layers.{i}.weight" for i in range(48)]
+    layout = {n: ((4, 8), "BF16") for n in engine}
+    monkeypatch.delenv("MX_RESHARD_REQUIRE_FULL_COVERAGE", raising=False)
+    monkeypatch.delenv("MX_RESHARD_COVERAGE_FLOOR", raising=False)
+    _coverage(caplog, param_layout=layout, all_params=engine[:24])  # off: a partial refit goes through
+    monkeypatch.setenv("MX_RESHARD_REQUIRE_FULL_COVERAGE", "1")
+    with pytest.raises(IncompleteRefit, match=r"covers 50\.00% .* 24 of 48 params .*layers\.24\.weight"):
+        _coverage(caplog, param_layout=layout, all_params=engine[:24])
+    assert any("MX_REFIT_COVERAGE" in r.getMessage() for r in caplog.records)  # recorded before it is rejected
+    monkeypatch.setenv("MX_RESHARD_COVERAGE_FLOOR", "0.5")
+    _coverage(caplog, param_layout=layout, all_params=engine[:24])  # at the floor: passes
+    for floor in ("-0.1", "1.5"):
+        monkeypatch.setenv("MX_RESHARD_COVERAGE_FLOOR", floor)
+        with pytest.raises(ValueError, match="MX_RESHARD_COVERAGE_FLOOR"):
+            _coverage(caplog, param_layout=layout, all_params=engine[:24])
