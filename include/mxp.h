@@ -375,6 +375,19 @@ typedef struct mxp_view_copy {
  * individual kernel launches", refit/reshard/receiver.py:920-923).  Destinations must not
  * overlap one another: the launches give no order between views. */
 int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, void* stream);
+/* The same n copies lowered once and run many times - a refit loop re-slices the same views
+ * every step (the reference caches its descriptor lists for that reason,
+ * refit/reshard/receiver.py:787-801).  mxp_view_plan_create lowers the views, builds the descriptor
+ * tables and uploads them; nothing moves.  mxp_view_plan_run only launches (one kernel for all
+ * row / element boxes, one per kind of transposed view): it allocates nothing, copies nothing
+ * from the host and does not synchronise, so it can be recorded into a HIP graph.  The source
+ * and destination addresses are the ones given at create; when a buffer moves, build a new
+ * plan.  Destinations must not overlap one another.  *out_bytes = destination bytes per run. */
+typedef struct mxp_view_plan mxp_view_plan;
+int mxp_view_plan_create(mxp_engine* engine, const mxp_view_copy* views, int64_t n, mxp_view_plan** out);
+int mxp_view_plan_run(mxp_engine* engine, mxp_view_plan* plan, void* stream);
+int mxp_view_plan_bytes(const mxp_view_plan* plan, uint64_t* out_bytes);
+void mxp_view_plan_destroy(mxp_view_plan* plan);
 /* n independent contiguous device copies in one launch, with the checksum of each
  * destination in out_checksums[k] when not NULL: the device form of the batched
  * torch._foreach_copy_ install (refit/reshard/receiver.py:939-955).  Destinations must

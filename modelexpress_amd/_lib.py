@@ -154,6 +154,10 @@ SIGNATURES = {
     "mxp_copy_view": (C.c_int, [_P, _P, _P, C.c_int32, C.POINTER(C.c_int64), C.POINTER(C.c_int64),
                                 C.POINTER(C.c_int64), C.c_int32, C.c_int32, _U32P, _P]),
     "mxp_copy_views": (C.c_int, [_P, C.POINTER(ViewCopy), C.c_int64, _P]),
+    "mxp_view_plan_create": (C.c_int, [_P, C.POINTER(ViewCopy), C.c_int64, C.POINTER(C.c_void_p)]),
+    "mxp_view_plan_run": (C.c_int, [_P, _P, _P]),
+    "mxp_view_plan_bytes": (C.c_int, [_P, _U64P]),
+    "mxp_view_plan_destroy": (None, [_P]),
     "mxp_copy_batch": (C.c_int, [_P, _PP, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_digest_from_scalars": (C.c_int, [_U64P, C.POINTER(C.c_uint8)]),

@@ -1129,27 +1129,35 @@ void copy_view(mxp_engine& e, const void* src, void* dst, std::vector<uint64_t> 
   if (checksum) *checksum = sum;
 }
 
-// Runs transposes that report no checksum: those that share a kernel instance and workgroup
-// size go out as one launch, the rest one by one.
-void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStream_t stream) {
+// Transposes that share a kernel instance and workgroup size, laid out for one launch each.
+struct TransposeGroup {
+  size_t first, count;  // slice of the item table
+  uint64_t tiles;
+  uint32_t waves;
+  int elem_size;
+  uint32_t op;
+};
+
+// Sorts `jobs` into launch groups (`items` receives their descriptor table) and `singles`
+// (a kind of its own: launched with the descriptor as a kernel argument).
+void group_transposes(const std::vector<TransposeJob>& jobs, std::vector<TransposeItem>& items,
+                      std::vector<TransposeGroup>& groups, std::vector<TransposeJob>& singles) {
   std::vector<size_t> order;
   for (size_t k = 0; k < jobs.size(); ++k) {
     if (jobs[k].td.n_tiles) order.push_back(k);  // descriptors were checked when the views were lowered
   }
   auto key = [&](size_t k) { return ((uint64_t)jobs[k].op << 16) | ((uint64_t)jobs[k].elem_size << 8) | jobs[k].td.waves; };
-  std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return key(a) < key(b); });
-  std::vector<TransposeItem> items;
-  struct Group { size_t first, count; uint64_t tiles; size_t job; };  // job: any member, for the shared op / element / waves
-  std::vector<Group> groups;
+  std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) { return key(x) < key(y); });
   for (size_t q = 0; q < order.size();) {
     size_t r = q;
     uint64_t tiles = 0;
     while (r < order.size() && key(order[r]) == key(order[q]) && tiles + jobs[order[r]].td.n_tiles <= 0x7FFFFFFFull)
       tiles += jobs[order[r++]].td.n_tiles;
     if (r - q == 1) {
-      run_transpose(e, jobs[order[q]], nullptr, stream);
+      singles.push_back(jobs[order[q]]);
     } else {
-      groups.push_back(Group{items.size(), r - q, tiles, order[q]});
+      const TransposeJob& j0 = jobs[order[q]];
+      groups.push_back(TransposeGroup{items.size(), r - q, tiles, j0.td.waves, j0.elem_size, j0.op});
       uint64_t first = 0;
       for (size_t k = q; k < r; ++k) {
         const TransposeJob& j = jobs[order[k]];
@@ -1159,6 +1167,16 @@ void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStr
     }
     q = r;
   }
+}
+
+// Runs transposes that report no checksum: those that share a kernel instance and workgroup
+// size go out as one launch, the rest one by one.
+void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStream_t stream) {
+  std::vector<TransposeItem> items;
+  std::vector<TransposeGroup> groups;
+  std::vector<TransposeJob> singles;
+  group_transposes(jobs, items, groups, singles);
+  for (const auto& j : singles) run_transpose(e, j, nullptr, stream);
   if (groups.empty()) return;
   if (e.items_recorded) HIP_OK(hipEventSynchronize(e.items_busy));
   if (items.size() > e.items_cap) {
@@ -1172,11 +1190,9 @@ void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStr
   e.items_dev.reserve(e.items_cap);
   std::memcpy(e.items_host, items.data(), items.size() * sizeof(TransposeItem));
   HIP_OK(hipMemcpyAsync(e.items_dev.p, e.items_host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
-  for (const Group& g : groups) {
-    const TransposeJob& j = jobs[g.job];
-    HIP_OK(launch_transpose_batch(e.items_dev.p + g.first, (uint32_t)g.count, g.tiles, j.td.waves, j.elem_size, j.op,
+  for (const TransposeGroup& g : groups)
+    HIP_OK(launch_transpose_batch(e.items_dev.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
                                   e.opt.nan_bits, stream));
-  }
   HIP_OK(hipEventRecord(e.items_busy, stream));
   e.items_recorded = true;
 }
@@ -1202,8 +1218,41 @@ void check_view_args(const mxp_engine* engine, int32_t ndim, const int64_t* shap
     if (shape[d] < 0) throw Error(MXP_ERR_ARG, std::string(what) + ": negative extent");
 }
 
+// Lowers n view copies into row / element boxes and transposes; nothing is launched.
+void lower_views(const mxp_engine* engine, const mxp_view_copy* views, int64_t n, std::vector<BoxCopy>& boxes,
+                 std::vector<const void*>& srcs, std::vector<void*>& dsts, std::vector<TransposeJob>& transposes,
+                 const char* what) {
+  for (int64_t k = 0; k < n; ++k) {
+    const mxp_view_copy& v = views[k];
+    check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
+    if (v.cast < MXP_CAST_NONE || v.cast > MXP_CAST_LAST) throw Error(MXP_ERR_ARG, std::string(what) + ": unknown conversion code");
+    if (v.cast != MXP_CAST_NONE && v.elem_size != (int32_t)op_dst_elem(seg_op_of_cast(v.cast)))
+      throw Error(MXP_ERR_ARG, std::string(what) + ": elem_size is not the destination element size of the conversion");
+    std::vector<uint64_t> size;
+    for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
+    TransposeJob tr{};
+    const auto s_st = strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what);
+    const auto d_st = strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what);
+    const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts, tr, what);
+    if (kind == kViewTranspose) transposes.push_back(tr);
+  }
+}
+
 }  // namespace
 }  // extern "C++"
+
+// View copies lowered once (mxp_view_plan_create): descriptor tables resident on the device,
+// nothing to build, upload or allocate when it runs.
+struct mxp_view_plan {
+  int device = 0;
+  DevBuf<uint8_t> tables;  // [segments][work items][source pointers][destination pointers]
+  size_t o_work = 0, o_src = 0, o_dst = 0;
+  uint32_t n_work = 0;
+  std::vector<TransposeJob> singles;
+  std::vector<TransposeGroup> groups;
+  DevBuf<TransposeItem> items;
+  uint64_t bytes = 0;  // destination bytes one run writes
+};
 
 int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
                      const int64_t* src_strides, const int32_t* perm, int32_t elem_size, uint32_t* checksum,
@@ -1248,32 +1297,96 @@ int mxp_copy_view(mxp_engine* engine, const void* src, void* dst, int32_t ndim, 
 
 int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, void* stream_v) {
   return guard([&] {
-    const char* what = "mxp_copy_views";
     if (!engine || n < 0 || (n && !views)) throw Error(MXP_ERR_ARG, "mxp_copy_views: bad argument");
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     std::vector<BoxCopy> boxes;
     std::vector<const void*> srcs;
     std::vector<void*> dsts;
     std::vector<TransposeJob> transposes;
-    for (int64_t k = 0; k < n; ++k) {  // everything is lowered before anything is launched
-      const mxp_view_copy& v = views[k];
-      check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
-      if (v.cast < MXP_CAST_NONE || v.cast > MXP_CAST_LAST) throw Error(MXP_ERR_ARG, "mxp_copy_views: unknown conversion code");
-      if (v.cast != MXP_CAST_NONE && v.elem_size != (int32_t)op_dst_elem(seg_op_of_cast(v.cast)))
-        throw Error(MXP_ERR_ARG, "mxp_copy_views: elem_size is not the destination element size of the conversion");
-      std::vector<uint64_t> size;
-      for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
-      TransposeJob tr{};
-      const auto s_st = strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what);
-      const auto d_st = strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what);
-      const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts,
-                                       tr, what);
-      if (kind == kViewTranspose) transposes.push_back(tr);
-    }
+    lower_views(engine, views, n, boxes, srcs, dsts, transposes, "mxp_copy_views");  // before anything is launched
     HIP_OK(hipSetDevice(engine->opt.device));
     if (!boxes.empty()) run_boxes(*engine, boxes, srcs, dsts, 1, nullptr, stream);
     run_transposes(*engine, transposes, stream);
   });
+}
+
+int mxp_view_plan_create(mxp_engine* engine, const mxp_view_copy* views, int64_t n, mxp_view_plan** out) {
+  return guard([&] {
+    if (!out) throw Error(MXP_ERR_ARG, "mxp_view_plan_create: null out");
+    *out = nullptr;
+    if (!engine || n < 0 || (n && !views)) throw Error(MXP_ERR_ARG, "mxp_view_plan_create: bad argument");
+    std::vector<BoxCopy> boxes;
+    std::vector<const void*> srcs;
+    std::vector<void*> dsts;
+    std::vector<TransposeJob> transposes;
+    lower_views(engine, views, n, boxes, srcs, dsts, transposes, "mxp_view_plan_create");
+    auto vp = std::make_unique<mxp_view_plan>();
+    vp->device = engine->opt.device;
+    HIP_OK(hipSetDevice(vp->device));
+    LowerOptions lo;
+    lo.tile_bytes = engine->opt.tile_bytes;
+    std::vector<Seg> segs;
+    std::vector<WorkItem> work;
+    for (const auto& b : boxes) {
+      lower_box(b, lo, segs, work);
+      vp->bytes += b.rows * b.row_bytes;
+    }
+    vp->n_work = (uint32_t)work.size();
+    if (!work.empty()) {
+      // one table: [segments][work items][source pointers][destination pointers]
+      vp->o_work = align_up(segs.size() * sizeof(Seg), 256);
+      vp->o_src = align_up(vp->o_work + work.size() * sizeof(WorkItem), 256);
+      vp->o_dst = align_up(vp->o_src + srcs.size() * sizeof(void*), 256);
+      std::vector<uint8_t> host(align_up(vp->o_dst + dsts.size() * sizeof(void*), 256), 0);
+      std::memcpy(host.data(), segs.data(), segs.size() * sizeof(Seg));
+      std::memcpy(host.data() + vp->o_work, work.data(), work.size() * sizeof(WorkItem));
+      std::memcpy(host.data() + vp->o_src, srcs.data(), srcs.size() * sizeof(void*));
+      std::memcpy(host.data() + vp->o_dst, dsts.data(), dsts.size() * sizeof(void*));
+      vp->tables.upload(host.data(), host.size());
+    }
+    std::vector<TransposeItem> items;
+    group_transposes(transposes, items, vp->groups, vp->singles);
+    if (!items.empty()) vp->items.upload(items.data(), items.size());
+    for (const auto& t : transposes) {
+      uint64_t elems = t.td.ni * t.td.nj;
+      for (int q = 0; q < kMaxBatchDims; ++q) elems *= t.td.batch_size[q];
+      vp->bytes += elems * (t.op == kOpCopy ? (uint64_t)t.elem_size : (uint64_t)op_dst_elem(t.op));
+    }
+    *out = vp.release();
+  });
+}
+
+int mxp_view_plan_run(mxp_engine* engine, mxp_view_plan* plan, void* stream_v) {
+  return guard([&] {
+    if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_view_plan_run: null handle");
+    if (plan->device != engine->opt.device) throw Error(MXP_ERR_ARG, "mxp_view_plan_run: the plan was built for another device");
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    HIP_OK(hipSetDevice(plan->device));
+    if (plan->n_work) {
+      uint8_t* d = plan->tables.p;
+      HIP_OK(launch_place(reinterpret_cast<const Seg*>(d), reinterpret_cast<const WorkItem*>(d + plan->o_work), plan->n_work,
+                          reinterpret_cast<const void* const*>(d + plan->o_src), reinterpret_cast<void* const*>(d + plan->o_dst),
+                          nullptr, engine->opt.nan_bits, stream));
+    }
+    for (const auto& t : plan->singles)
+      HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, engine->opt.nan_bits, nullptr, stream));
+    for (const auto& g : plan->groups)
+      HIP_OK(launch_transpose_batch(plan->items.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
+                                    engine->opt.nan_bits, stream));
+  });
+}
+
+int mxp_view_plan_bytes(const mxp_view_plan* plan, uint64_t* out_bytes) {
+  return guard([&] {
+    if (!plan || !out_bytes) throw Error(MXP_ERR_ARG, "mxp_view_plan_bytes: null argument");
+    *out_bytes = plan->bytes;
+  });
+}
+
+void mxp_view_plan_destroy(mxp_view_plan* plan) {
+  if (!plan) return;
+  (void)hipSetDevice(plan->device);
+  delete plan;
 }
 
 int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dsts, const uint64_t* nbytes, int64_t n,

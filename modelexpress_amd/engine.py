@@ -429,6 +429,14 @@ class PlacementEngine:
                     getattr(o, key)[d] = int(x)
         L.check(L.lib().mxp_copy_views(self._h, arr, len(views), C.c_void_p(stream)))
 
+    def copy_views_array(self, arr, n: int, *, stream: int = 0) -> None:
+        """``copy_views`` on an ``_lib.ViewCopy`` array the caller built (and may keep between calls)."""
+        L.check(L.lib().mxp_copy_views(self._h, arr, n, C.c_void_p(stream)))
+
+    def view_plan(self, arr, n: int) -> "ViewPlan":
+        """The views of an ``_lib.ViewCopy`` array lowered once; ``ViewPlan.run`` only launches."""
+        return ViewPlan(self, arr, n)
+
     def copy_batch(self, srcs: Sequence, dsts: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
                    checksums: bool = True) -> list[str] | None:
         """n contiguous device copies in one launch (optionally with destination checksums)."""
@@ -444,6 +452,33 @@ class PlacementEngine:
         out = C.c_double()
         L.check(L.lib().mxp_measure_h2d(self._h, nbytes, repeats, C.byref(out)))
         return float(out.value)
+
+
+class ViewPlan:
+    """Handle of ``mxp_view_plan``: descriptor tables resident on the device for a fixed set of view copies
+    at fixed addresses.  ``run`` allocates nothing, copies nothing from the host and does not synchronise."""
+
+    def __init__(self, engine: PlacementEngine, arr, n: int):
+        self._engine = engine
+        self._h = C.c_void_p()
+        L.check(L.lib().mxp_view_plan_create(engine._h, arr, n, C.byref(self._h)))
+        out = C.c_uint64()
+        L.check(L.lib().mxp_view_plan_bytes(self._h, C.byref(out)))
+        self.bytes = int(out.value)
+
+    def run(self, *, stream: int = 0) -> None:
+        L.check(L.lib().mxp_view_plan_run(self._engine._h, self._h, C.c_void_p(stream)))
+
+    def close(self) -> None:
+        if self._h:
+            L.lib().mxp_view_plan_destroy(self._h)
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # noqa: BLE001
+            pass
 
 
 def digest_from_scalars(scalars: Sequence[int]) -> str:

@@ -299,3 +299,98 @@ def test_interleaved_column_blocks_of_one_parameter(gpu_engine):
 def test_no_copies_is_a_no_op(gpu_engine):
     # test_reshard_refit_batch_install.py:269-284
     assert execute_recorded_copies(gpu_engine, [], {}, {}) == 0
+
+
+def test_reslice_plan_splits_only_where_spans_meet():
+    """The split into calls is decided when the plan is built, on CPU tensors: disjoint row blocks share one
+    call; views whose spans meet start a new call at that point, in plan order."""
+    from modelexpress_amd.reshard import ReslicePlan
+
+    src = {"w": torch.zeros(8, 4)}
+    p = {"p": torch.zeros(8, 4), "q": torch.zeros(8, 4)}
+    rows = lambda name, start, off: RecordedCopy("w", (("narrow", (0, start, 2), ()),), name, off, (2, 4), (4, 1))  # noqa: E731
+    plan = ReslicePlan([rows("p", 0, 0), rows("p", 2, 8), rows("q", 0, 0), rows("p", 4, 16)], src, p)
+    assert plan.batches == [[0, 1, 2, 3]] and plan.bytes == 4 * 2 * 4 * 4
+    plan = ReslicePlan([rows("p", 0, 0), rows("p", 2, 8), rows("p", 4, 4), rows("q", 0, 0), rows("p", 6, 8)], src, p)
+    assert plan.batches == [[0, 1], [2, 3], [4]]  # copy 2 meets copies 0 and 1; copy 4 meets copy 2
+    assert ReslicePlan([], src, p).batches == []
+
+
+@pytest.mark.gpu
+def test_reslice_plan_is_reused_across_steps_and_follows_moved_tensors(gpu_engine):
+    """A plan built once serves every step (refit/reshard/receiver.py:787-801): new source values, the same
+    addresses; then a parameter that moved; then a source whose shape changed, which is refused."""
+    from modelexpress_amd.reshard import ReslicePlan
+
+    g = torch.Generator().manual_seed(8)
+    sources = {f"s{k}": torch.randn(64, 48, generator=g).cuda() for k in range(6)}
+    param = torch.zeros(6 * 32, 48, dtype=torch.bfloat16, device="cuda")
+    copies = [RecordedCopy(f"s{k}", (("narrow", (0, 16, 32), ()),), "fused", k * 32 * 48, (32, 48), (48, 1)) for k in range(6)]
+    plan = ReslicePlan(copies, sources, {"fused": param})
+
+    def want():
+        return torch.cat([sources[f"s{k}"][16:48] for k in range(6)]).to(torch.bfloat16)
+
+    assert plan.run(gpu_engine, sources, {"fused": param}) == param.numel() * 2
+    assert torch.equal(param, want())
+    arrays = plan._arrays
+    for t in sources.values():
+        t.normal_(generator=None)
+    plan.run(gpu_engine, sources, {"fused": param})
+    assert torch.equal(param, want()) and plan._arrays is arrays  # same addresses: the descriptor arrays are kept
+    for t in sources.values():
+        t.normal_(generator=None)
+    assert plan.replay() == param.numel() * 2 and torch.equal(param, want())  # launches only, same tensors
+    moved = torch.zeros_like(param)
+    plan.run(gpu_engine, sources, {"fused": moved})
+    assert torch.equal(moved, want()) and plan._arrays is not arrays
+    sources["s0"] = torch.randn(32, 48).cuda()
+    with pytest.raises(UnsupportedReshard, match="changed shape"):
+        plan.run(gpu_engine, sources, {"fused": moved})
+
+
+@pytest.mark.gpu
+def test_view_plan_runs_from_a_hip_graph(gpu_engine):
+    """``mxp_view_plan_run`` only launches kernels (no allocation, no host copy, no memset node), so a refit's
+    re-slice can be recorded into a HIP graph: every replay is checked against the eager result, with eager
+    work and synchronisation between replays, for row boxes, a batch of transposes and a converting one."""
+    g = torch.Generator().manual_seed(12)
+    srcs = [torch.randn(96, 64, generator=g).cuda() for _ in range(5)]
+    dsts = [torch.zeros(48, 64, dtype=torch.bfloat16, device="cuda"),      # row box, fp32 -> bf16
+            torch.zeros(64, 96, device="cuda"), torch.zeros(64, 96, device="cuda"), torch.zeros(64, 96, device="cuda"),  # transposes
+            torch.zeros(64, 96, dtype=torch.bfloat16, device="cuda")]      # converting transpose
+    views = [{"src": srcs[0][24:], "dst": dsts[0], "shape": (48, 64), "elem_size": 2, "src_strides": (64, 1), "cast": 1}]
+    views += [{"src": srcs[k], "dst": dsts[k], "shape": (64, 96), "elem_size": 4, "src_strides": (1, 64)} for k in (1, 2, 3)]
+    views += [{"src": srcs[4], "dst": dsts[4], "shape": (64, 96), "elem_size": 2, "src_strides": (1, 64), "cast": 1}]
+
+    def want():
+        return [srcs[0][24:72].to(torch.bfloat16)] + [srcs[k].t().contiguous() for k in (1, 2, 3)] + [srcs[4].t().to(torch.bfloat16).contiguous()]
+
+    from modelexpress_amd import _lib as L
+
+    arr = (L.ViewCopy * len(views))()
+    for o, v in zip(arr, views):
+        o.src, o.dst, o.ndim, o.elem_size, o.cast = v["src"].data_ptr(), v["dst"].data_ptr(), 2, v["elem_size"], v.get("cast", 0)
+        o.contiguous_dst = 1
+        for d in range(2):
+            o.shape[d], o.src_strides[d] = v["shape"][d], v["src_strides"][d]
+    plan = gpu_engine.view_plan(arr, len(views))
+    assert plan.bytes == sum(d.numel() * d.element_size() for d in dsts)
+    plan.run()
+    torch.cuda.synchronize()
+    assert all(torch.equal(d, w) for d, w in zip(dsts, want()))
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            plan.run(stream=torch.cuda.current_stream().cuda_stream)
+    for step in range(3):
+        for s in srcs:
+            s.normal_()           # eager work between replays: new source values, same addresses
+        for d in dsts:
+            d.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert all(torch.equal(d, w) for d, w in zip(dsts, want())), step
+    plan.close()
