@@ -230,3 +230,106 @@ def test_capture_then_device_execution_rebuilds_the_loaders_result(gpu_engine, t
     assert written == sum(p.numel() * 4 for p in recon.values())
     for name, p in truth_model.named_parameters():
         assert torch.equal(recon[name].cpu(), p.detach()), name
+
+
+class MiniDecoderLayer(torch.nn.Module):
+    """One decoder layer with the loader shapes an inference engine uses: fused QKV with per-member shard ids
+    (grouped-query: fewer K/V heads), a merged [gate; up] fed either by two sources or by one pre-merged source
+    (``chunk``), row-parallel projections (column slices), a vocabulary-parallel embedding with a padded tail,
+    a Conv1D-style weight stored transposed, and a norm loaded by the framework's default loader."""
+
+    def __init__(self, tp_size, tp_rank, hidden=256, heads=8, kv_heads=2, head_dim=32, inter=768, vocab=1000, dtype=torch.bfloat16):
+        super().__init__()
+        self.tp_size, self.tp_rank = tp_size, tp_rank
+        self.q_rows, self.kv_rows = heads * head_dim // tp_size, kv_heads * head_dim // tp_size
+        self.inter_local = inter // tp_size
+        self.vocab_local = (vocab + tp_size - 1) // tp_size
+        self.vocab = vocab
+        P = lambda *shape: torch.nn.Parameter(torch.zeros(*shape, dtype=dtype), requires_grad=False)  # noqa: E731
+        self.qkv = P(self.q_rows + 2 * self.kv_rows, hidden)
+        self.qkv.weight_loader = self._qkv_loader
+        self.gate_up = P(2 * self.inter_local, hidden)
+        self.gate_up.weight_loader = self._gate_up_loader
+        self.o_proj = P(hidden, heads * head_dim // tp_size)
+        self.o_proj.weight_loader = self._row_loader
+        self.down = P(hidden, self.inter_local)
+        self.down.weight_loader = self._row_loader
+        self.embed = P(self.vocab_local, hidden)
+        self.embed.weight_loader = self._vocab_loader
+        self.c_fc = P(self.inter_local, hidden)
+        self.c_fc.weight_loader = self._conv1d_loader
+        self.norm = P(hidden)
+
+    def _qkv_loader(self, param, loaded, shard_id):
+        rows = self.q_rows if shard_id == "q" else self.kv_rows
+        offset = {"q": 0, "k": self.q_rows, "v": self.q_rows + self.kv_rows}[shard_id]
+        param.data.narrow(0, offset, rows).copy_(loaded.narrow(0, self.tp_rank * rows, rows))
+
+    def _gate_up_loader(self, param, loaded, shard_id=None):
+        if shard_id is None:  # one pre-merged [gate; up] source: split, then shard each half
+            for k, half in enumerate(loaded.chunk(2, dim=0)):
+                self._gate_up_loader(param, half, k)
+            return
+        n = self.inter_local
+        param.data.narrow(0, shard_id * n, n).copy_(loaded.narrow(0, self.tp_rank * n, n))
+
+    def _row_loader(self, param, loaded):
+        param.data.copy_(loaded.narrow(1, self.tp_rank * param.shape[1], param.shape[1]))
+
+    def _vocab_loader(self, param, loaded):
+        start = self.tp_rank * self.vocab_local
+        n = min(self.vocab_local, self.vocab - start)  # the last rank's tail stays as it is
+        param.data[:n].copy_(loaded.narrow(0, start, n))
+
+    def _conv1d_loader(self, param, loaded):
+        param.data.copy_(loaded.t().narrow(0, self.tp_rank * self.inter_local, self.inter_local))  # stored [in, out]
+
+    def load_weights(self, weights):
+        params = dict(self.named_parameters())
+        for name, loaded in weights:
+            if name in ("q", "k", "v"):
+                self.qkv.weight_loader(self.qkv, loaded, name)
+            elif name in ("gate", "up"):
+                self.gate_up.weight_loader(self.gate_up, loaded, 0 if name == "gate" else 1)
+            elif name == "gate_up_merged":
+                self.gate_up.weight_loader(self.gate_up, loaded)
+            else:
+                getattr(params[name], "weight_loader", _plain_default_loader)(params[name], loaded)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tp_size,tp_rank,premerged", [(1, 0, False), (2, 1, False), (4, 3, True)])
+def test_decoder_layer_loaders_captured_and_replayed_on_the_device(gpu_engine, tp_size, tp_rank, premerged):
+    """fp32 trainer tensors into bf16 engine parameters through the engine's own loaders: the captured plan,
+    run on the device (and replayed after the sources changed), gives the bytes the loaders give on the CPU."""
+    from modelexpress_amd.reshard import ReslicePlan
+
+    hidden, heads, kv_heads, head_dim, inter, vocab = 256, 8, 4, 32, 768, 1000
+    shapes = {"q": (heads * head_dim, hidden), "k": (kv_heads * head_dim, hidden), "v": (kv_heads * head_dim, hidden),
+              "o_proj": (hidden, heads * head_dim), "down": (hidden, inter), "embed": (vocab, hidden), "c_fc": (hidden, inter), "norm": (hidden,)}
+    shapes.update({"gate_up_merged": (2 * inter, hidden)} if premerged else {"gate": (inter, hidden), "up": (inter, hidden)})
+    kw = dict(hidden=hidden, heads=heads, kv_heads=kv_heads, head_dim=head_dim, inter=inter, vocab=vocab)
+    g = torch.Generator().manual_seed(70 + tp_rank)
+    with torch.device("meta"):
+        twin = MiniDecoderLayer(tp_size, tp_rank, **kw)
+    capture = capture_geometry(twin, [(n, torch.float32, list(s)) for n, s in shapes.items()], default_weight_loader=_plain_default_loader)
+    assert capture.unsupported == [] and capture.unattributed == 0
+    assert len(capture.copies) == len(shapes) + (1 if premerged else 0)  # the pre-merged source yields two copies
+    live = MiniDecoderLayer(tp_size, tp_rank, **kw).cuda()
+    params = dict(live.named_parameters())
+    plan = None
+    for step in range(2):
+        srcs = {n: torch.randn(s, generator=g) * 2 for n, s in shapes.items()}
+        truth = MiniDecoderLayer(tp_size, tp_rank, **kw)
+        truth.load_weights(list(srcs.items()))
+        dev = {n: t.cuda() for n, t in srcs.items()} if step == 0 else dev
+        if step == 0:
+            plan = ReslicePlan(capture.copies, dev, params)
+            plan.run(gpu_engine, dev, params)
+        else:
+            for n, t in srcs.items():
+                dev[n].copy_(t)   # new values at the same addresses
+            plan.replay()
+        for name, p in truth.named_parameters():
+            assert torch.equal(params[name].cpu().view(torch.int16), p.view(torch.int16)), (step, name)
+    plan.close()
