@@ -66,3 +66,43 @@ def test_copy_to_device_snapshot_matches_copy_(gpu_engine, oracle):
     torch.cuda.synchronize()
     assert torch.equal(out["served"]["embed"], moved["embed"].to(WIRE_DTYPE)) and out["served"]["embed"].data_ptr() == addrs["embed"]
     st.close()
+
+
+@pytest.mark.gpu
+def test_colocated_refit_trainer_snapshot_to_engine_parameters(gpu_engine):
+    """Both ends on one GPU: the trainer's fp32 state dict is snapshotted into bf16 arenas (one launch), the
+    engine's own loaders are captured once on a meta twin, and each step re-slices the arenas into the live
+    parameters (one launch) - the bytes are those of the loaders fed the bf16 tensors on the CPU."""
+    from test_capture import MiniDecoderLayer, _plain_default_loader
+    from modelexpress_amd.capture import capture_geometry
+    from modelexpress_amd.reshard import ReslicePlan
+
+    tp_size, tp_rank = 2, 1
+    kw = dict(hidden=256, heads=8, kv_heads=4, head_dim=32, inter=768, vocab=1000)
+    shapes = {"q": (256, 256), "k": (128, 256), "v": (128, 256), "gate": (768, 256), "up": (768, 256), "o_proj": (256, 256),
+              "down": (256, 768), "embed": (1000, 256), "c_fc": (256, 768), "norm": (256,)}
+    g = torch.Generator().manual_seed(33)
+    trainer = {n: torch.randn(s, generator=g).cuda() for n, s in shapes.items()}
+    with torch.device("meta"):
+        twin = MiniDecoderLayer(tp_size, tp_rank, **kw)
+    capture = capture_geometry(twin, [(n, WIRE_DTYPE, list(s)) for n, s in shapes.items()], default_weight_loader=_plain_default_loader)
+    live = MiniDecoderLayer(tp_size, tp_rank, **kw).cuda()
+    params = dict(live.named_parameters())
+    stager = WireStager(gpu_engine)
+    plan = None
+    for step in range(3):
+        served = stager.stage(trainer)["served"]
+        if plan is None:
+            plan = ReslicePlan(capture.copies, served, params)
+            plan.run(gpu_engine, served, params)
+        else:
+            plan.replay()
+        torch.cuda.synchronize()
+        truth = MiniDecoderLayer(tp_size, tp_rank, **kw)
+        truth.load_weights([(n, t.cpu().to(WIRE_DTYPE)) for n, t in trainer.items()])
+        for name, p in truth.named_parameters():
+            assert torch.equal(params[name].cpu().view(torch.int16), p.view(torch.int16)), (step, name)
+        for t in trainer.values():
+            t.add_(torch.randn(t.shape, generator=g).cuda() * 0.01)  # an optimizer step
+    plan.close()
+    stager.close()
