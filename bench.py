@@ -241,6 +241,17 @@ def main() -> int:
                                 "gbps_wall": round(placed / dt / 1e9, 1),
                                 "note": "one batched launch; wall time includes descriptor upload, result copy and sync"}
             ops["checksum32"]["matches_fused"] = eng.checksum32(dst, sizes) == resident_sums
+            # the same placement with the tensor_digest sums accumulated in the placement kernel (no second pass)
+            eng.set_fused_digests(True)
+            k_fd = []
+            for _ in range(5):
+                k_fd.append(eng.execute_resident(plan, staged, dst, timed=True)["kernel_ms"])
+            fused_digests = eng.digests(plan)
+            eng.set_fused_digests(False)
+            ops["place_with_fused_digests"] = {"kernel_ms_avg": round(sum(k_fd) / len(k_fd), 4), "kernel_ms_min": round(min(k_fd), 4),
+                                               "gbps_algorithmic": round(algo / (sum(k_fd) / len(k_fd) * 1e-3) / 1e9, 1),
+                                               "matches_stand_alone_digest": fused_digests == eng.digest(dst, sizes),
+                                               "checksums_unchanged": eng.checksums(plan) == resident_sums}
             # context only: the platform's own device copy of as many bytes as one step places
             a = torch.empty(placed, dtype=torch.uint8, device="cuda").random_(0, 256)
             b = torch.empty_like(a)

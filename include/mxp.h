@@ -282,6 +282,16 @@ int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* 
 /* Checksums accumulated by the last execute, one per parameter (tensor_utils.py:27-44
  * over the parameter's row-major bytes).  Synchronises the engine first. */
 int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_t n);
+/* Fused verification: with this switched on, every placement (mxp_execute, mxp_execute_resident)
+ * also accumulates, inside the same kernel, the sums tensor_digest is made of
+ * (refit/reshard/verify.py:112-150) for every parameter buffer, so the digests of what was placed
+ * cost no second pass over the buffers - in place of the reference's recompute-after-transfer
+ * (modelexpress_rl/inference/nixl_staged_transfer.py:529-549).  mxp_plan_digests waits for the
+ * device and writes 16 bytes per parameter (the blake2b-128 of the scalar list, as mxp_digest
+ * gives for the finished buffer); it fails if the last execute ran with the switch off or if the
+ * plan leaves part of a parameter unwritten.  The checksums are still produced. */
+int mxp_engine_set_fused_digests(mxp_engine* engine, int32_t on);
+int mxp_plan_digests(mxp_engine* engine, mxp_plan* plan, uint8_t* out16, int64_t n);
 
 /* =========================================================================
  * 4. Stand-alone device operators (all batched: one launch for n tensors)

@@ -137,6 +137,8 @@ SIGNATURES = {
     "mxp_plan_param_info": (C.c_int, [_P, C.c_int64, C.POINTER(ParamInfo)]),
     "mxp_plan_write_info": (C.c_int, [_P, C.c_int64, C.POINTER(WriteInfo)]),
     "mxp_plan_totals": (C.c_int, [_P, _U64P, _U64P, _U64P, _U64P]),
+    "mxp_engine_set_fused_digests": (C.c_int, [_P, C.c_int32]),
+    "mxp_plan_digests": (C.c_int, [_P, _P, C.POINTER(C.c_uint8), C.c_int64]),
     "mxp_engine_create": (C.c_int, [C.POINTER(EngineOptions), _PP]),
     "mxp_engine_destroy": (None, [_P]),
     "mxp_prepare": (C.c_int, [_P, _P]),

@@ -94,6 +94,14 @@ constexpr uint32_t kDigestRowsPerBlock = 32; // 128 KiB per workgroup, two rows 
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
                         uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only = false);
+// launch_place that also accumulates the tensor_digest sums of the bytes it stores: five 64-bit
+// words per destination buffer (whole-row sum, row-weighted sum, tail sum, tail-weighted sum,
+// ragged-byte sum), added to `digest_sums_dev` (cleared by the caller); `dst_sizes_dev[b]` is
+// the byte size of destination buffer b, segment offsets are offsets inside their buffer.
+hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
+                               const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev,
+                               const unsigned long long* dst_sizes_dev, unsigned long long* digest_sums_dev,
+                               uint16_t nan_bits, hipStream_t stream);
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
                          unsigned long long* out_dev, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);

@@ -94,6 +94,9 @@ struct mxp_plan::Lowered {
   DevBuf<void*> dst_bases;
   DevBuf<const void*> src_bases;
   DevBuf<uint32_t> sums;
+  DevBuf<unsigned long long> dst_sizes;    // byte size of every parameter (fused digests)
+  DevBuf<unsigned long long> digest_sums;  // five sums per parameter, accumulated by place_digest_kernel
+  bool digests_valid = false;              // the last execute accumulated them
   std::vector<void*> dst_host;        // what dst_bases currently holds
   std::vector<const void*> src_host;  // what src_bases currently holds
   uint64_t file_bytes = 0, h2d_bytes = 0, placed_bytes = 0, algo_bytes = 0;
@@ -111,6 +114,7 @@ struct mxp_engine {
   size_t desc_host_cap = 0;
   DevBuf<uint8_t> desc_dev;
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
+  bool fused_digests = false;       // placements also accumulate the tensor_digest sums (mxp_engine_set_fused_digests)
   hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
   bool arena_recorded = false;
   // descriptor table of batched transposes: same protocol as the arena, its own event
@@ -354,6 +358,12 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   L->dst_bases.reserve(pl.params.size() ? pl.params.size() : 1);
   L->src_bases.reserve(ck.files.size() ? ck.files.size() : 1);
   L->sums.reserve(pl.params.size() ? pl.params.size() : 1);
+  {
+    std::vector<unsigned long long> sizes;
+    for (const auto& p : pl.params) sizes.push_back(p.nbytes);
+    L->dst_sizes.upload(sizes.data(), sizes.size());
+    L->digest_sums.reserve(pl.params.size() ? 5 * pl.params.size() : 1);
+  }
   pl.lowered = L.release();
   pl.lowered_free = free_lowered;
 }
@@ -577,6 +587,9 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
   // Everything below may change destination bytes.
   upload_dst(L, pl, dst_ptrs);
   HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, e.streams[0]));
+  const bool digests = e.fused_digests;
+  L.digests_valid = false;
+  if (digests) HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(L.digest_sums.p), 10 * pl.params.size(), 0u, e.streams[0]));
   HIP_OK(hipStreamSynchronize(e.streams[0]));
   for (auto& s : e.slots) s->submitted = 0;
 
@@ -629,8 +642,13 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
         hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
         HIP_OK(hipMemcpyAsync(sl.dev, sl.host, ch.used_bytes, hipMemcpyHostToDevice, st));
         mutated.store(1);
-        HIP_OK(launch_place(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
-                            e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, e.opt.nan_bits, st));
+        if (digests)
+          HIP_OK(launch_place_digest(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
+                                     e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, L.dst_sizes.p, L.digest_sums.p,
+                                     e.opt.nan_bits, st));
+        else
+          HIP_OK(launch_place(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
+                              e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, e.opt.nan_bits, st));
         HIP_OK(hipEventRecord(sl.done, st));
         {
           std::lock_guard<std::mutex> lk(sl.mu);
@@ -675,6 +693,7 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
   }
   if (first_err) throw *first_err;
   if (sync_err != hipSuccess) throw Error(MXP_ERR_DEVICE, std::string("stream synchronize: ") + hipGetErrorString(sync_err));
+  L.digests_valid = digests;
 }
 
 void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_dev_ptrs, void* const* dst_ptrs,
@@ -696,9 +715,15 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
     L.src_host.assign(file_dev_ptrs, file_dev_ptrs + ck.files.size());
   }
   HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, stream));
+  L.digests_valid = e.fused_digests;
+  if (e.fused_digests) HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(L.digest_sums.p), 10 * pl.params.size(), 0u, stream));
   if (stats) HIP_OK(hipEventRecord(e.ev_a, stream));
-  HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
-                      e.opt.nan_bits, stream));
+  if (e.fused_digests)
+    HIP_OK(launch_place_digest(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
+                               L.dst_sizes.p, L.digest_sums.p, e.opt.nan_bits, stream));
+  else
+    HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
+                        e.opt.nan_bits, stream));
   if (stats) {
     HIP_OK(hipEventRecord(e.ev_b, stream));
     HIP_OK(hipEventSynchronize(e.ev_b));
@@ -750,6 +775,35 @@ int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_
     HIP_OK(hipSetDevice(engine->opt.device));
     HIP_OK(hipDeviceSynchronize());
     if (n) HIP_OK(hipMemcpy(out, plan->lowered->sums.p, (size_t)n * 4, hipMemcpyDeviceToHost));
+  });
+}
+
+int mxp_engine_set_fused_digests(mxp_engine* engine, int32_t on) {
+  return guard([&] {
+    if (!engine) throw Error(MXP_ERR_ARG, "mxp_engine_set_fused_digests: null engine");
+    engine->fused_digests = on != 0;
+  });
+}
+
+int mxp_plan_digests(mxp_engine* engine, mxp_plan* plan, uint8_t* out16, int64_t n) {
+  return guard([&] {
+    if (!engine || !plan || !out16) throw Error(MXP_ERR_ARG, "mxp_plan_digests: null argument");
+    if (!plan->lowered || !plan->lowered->digests_valid)
+      throw Error(MXP_ERR_STATE, "the plan's last execute did not accumulate digests (mxp_engine_set_fused_digests)");
+    if (n != (int64_t)plan->params.size()) throw Error(MXP_ERR_ARG, "mxp_plan_digests: n must equal the parameter count");
+    HIP_OK(hipSetDevice(engine->opt.device));
+    HIP_OK(hipDeviceSynchronize());
+    std::vector<unsigned long long> sums(5 * (size_t)n);
+    if (n) HIP_OK(hipMemcpy(sums.data(), plan->lowered->digest_sums.p, sums.size() * 8, hipMemcpyDeviceToHost));
+    for (int64_t i = 0; i < n; ++i) {
+      const auto& p = plan->params[(size_t)i];
+      if (p.bytes_written != p.nbytes)
+        throw Error(MXP_ERR_STATE, "parameter '" + p.name + "' is not fully written by the plan: its digest is undefined");
+      const uint64_t scalars[7] = {p.nbytes, sums[5 * i], sums[5 * i + 1], sums[5 * i + 2], sums[5 * i + 3], sums[5 * i + 4],
+                                   p.nbytes % 4};
+      const int rc = mxp_digest_from_scalars(scalars, out16 + 16 * i);
+      if (rc != MXP_OK) throw Error(rc, mxp_last_error());
+    }
   });
 }
 

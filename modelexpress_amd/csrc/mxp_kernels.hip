@@ -57,6 +57,9 @@ struct Csum {
     Q += s0;
     P += i * s0;
   }
+  // One unit of UNIT <= 4 bytes (the narrow paths).
+  template <int UNIT>
+  __device__ __forceinline__ void addn(uint32_t x, uint32_t i) { add4(x, i); }
   __device__ __forceinline__ uint32_t fold() const { return kKnuth * (P + R) + Q; }
 };
 
@@ -71,6 +74,79 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
   for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
   return v;
 }
+
+// Checksum plus the tensor_digest sums of the bytes being stored (reference:
+// modelexpress/refit/reshard/verify.py:112-150), for launches that verify what they place
+// without a second pass over the finished buffers.  The digest reads a buffer as little-endian
+// signed 32-bit words: whole 1024-word rows contribute sum(w) and sum(w) * (row + 1), the
+// words after the last whole row sum(w) and sum(w * (k + 1)), the 1..3 bytes after the last
+// whole word their unsigned sum - every term is linear in the stored bytes, so each lane adds
+// the share of the bytes it stores, weighted by where they land in the destination buffer,
+// and the sums wrap mod 2^64 exactly as the reference's int64 arithmetic does.
+struct DigestAcc {
+  Csum cs;
+  unsigned long long S = 0, SW = 0, T = 0, TW = 0, RG = 0;
+  uint64_t base = 0;        // position of the tile's first destination byte inside its buffer
+  uint32_t base32 = 0;      // the 32-bit checksum position the callers count from
+  uint64_t tail_word0 = 0;  // first word after the last whole row
+  uint64_t body_end = 0;    // first ragged byte
+  __device__ __forceinline__ void init(uint64_t buffer_bytes, uint64_t tile_pos, uint32_t tile_pos32) {
+    base = tile_pos;
+    base32 = tile_pos32;
+    body_end = buffer_bytes & ~3ull;
+    tail_word0 = (buffer_bytes >> 2) / kDigestRowWords * kDigestRowWords;
+  }
+  // Whole words starting at byte position p (a multiple of 4; all in one row): `sum` of the
+  // words and `ramp` = sum of word k times k, both as signed 64-bit values.
+  __device__ __forceinline__ void words(long long sum, long long ramp, uint64_t p) {
+    const uint64_t wi = p >> 2;
+    if (wi < tail_word0) {
+      S += (unsigned long long)sum;
+      SW += (unsigned long long)sum * (unsigned long long)(wi / kDigestRowWords + 1);
+    } else {
+      T += (unsigned long long)sum;
+      TW += (unsigned long long)sum * (unsigned long long)(wi - tail_word0 + 1) + (unsigned long long)ramp;
+    }
+  }
+  __device__ __forceinline__ void add16(const uint4& x, uint32_t i) {
+    cs.add16(x, i);
+    const long long a = (int32_t)x.x, b = (int32_t)x.y, c = (int32_t)x.z, d = (int32_t)x.w;
+    words(a + b + c + d, b + 2 * c + 3 * d, base + (uint32_t)(i - base32));
+  }
+  __device__ __forceinline__ void add8(uint32_t lo, uint32_t hi, uint32_t i) {
+    cs.add8(lo, hi, i);
+    const long long a = (int32_t)lo, b = (int32_t)hi;
+    words(a + b, b, base + (uint32_t)(i - base32));
+  }
+  template <int UNIT>
+  __device__ __forceinline__ void addn(uint32_t x, uint32_t i) {
+    cs.add4(x, i);
+    const uint64_t p = base + (uint32_t)(i - base32);
+    if constexpr (UNIT == 4) {
+      words((long long)(int32_t)x, 0, p);
+    } else {  // part of a word, or ragged bytes: byte by byte
+#pragma unroll
+      for (int e = 0; e < UNIT; ++e) {
+        const uint32_t b = (x >> (8 * e)) & 0xFFu;
+        const uint64_t q = p + e;
+        if (q >= body_end) {
+          RG += b;
+          continue;
+        }
+        const uint32_t j = (uint32_t)q & 3u;
+        const long long v = j == 3u ? (long long)(int32_t)(b << 24) : (long long)(b << (8u * j));
+        const uint64_t wi = q >> 2;
+        if (wi < tail_word0) {
+          S += (unsigned long long)v;
+          SW += (unsigned long long)v * (unsigned long long)(wi / kDigestRowWords + 1);
+        } else {
+          T += (unsigned long long)v;
+          TW += (unsigned long long)v * (unsigned long long)(wi - tail_word0 + 1);
+        }
+      }
+    }
+  }
+};
 
 // 128-bit non-temporal accesses: every byte is touched exactly once, so nothing is worth
 // keeping in L2 / Infinity Cache (measured: +3..4% over plain accesses on this copy).
@@ -105,10 +181,10 @@ __device__ __forceinline__ void st8(uint8_t* p, const uint2& v) {
 // Lanes walk the tile in flattened (row, unit) order, so neighbouring lanes touch
 // neighbouring 16-byte units of the same row: every wavefront access is a run of
 // contiguous 1 KiB pieces in both the source and the destination.
-template <int OP, int UNIT>
+template <int OP, int UNIT, class ACC>
 __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict__ src,
                                          uint8_t* __restrict__ dst, uint32_t csum_base,
-                                         uint32_t n_units, uint32_t nan_bits, Csum& cs) {
+                                         uint32_t n_units, uint32_t nan_bits, ACC& cs) {
   constexpr bool NARROW = op_narrows(OP), WIDEN = op_widens(OP);
   constexpr int SRC_UNIT = NARROW ? 2 * UNIT : WIDEN ? UNIT / 2 : UNIT;
   const uint32_t upr = s.units_per_row;
@@ -234,7 +310,7 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
         else if constexpr (UNIT == 2) *reinterpret_cast<uint16_t*>(dst + d_o) = (uint16_t)x;
         else dst[d_o] = (uint8_t)x;
       }
-      cs.add4(x, csum_base + d_o);
+      cs.template addn<UNIT>(x, csum_base + d_o);
     };
     constexpr uint32_t G = 8;
     for (uint32_t v0 = threadIdx.x; v0 < n_units; v0 += G * kPlaceThreads) {
@@ -253,11 +329,12 @@ __device__ __forceinline__ void run_tile(const Seg& s, const uint8_t* __restrict
   }
 }
 
-template <bool CHECKSUM_ONLY>
+template <bool CHECKSUM_ONLY, bool DIGEST = false>
 __device__ __forceinline__ void place_body(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
-    uint32_t* __restrict__ sums, uint32_t nan_bits) {
+    uint32_t* __restrict__ sums, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes = nullptr,
+    unsigned long long* __restrict__ digest_sums = nullptr) {
   const WorkItem w = work[blockIdx.x];
   const Seg s = segs[w.seg];
   const uint32_t r0 = w.tile * s.rows_per_tile;
@@ -271,7 +348,8 @@ __device__ __forceinline__ void place_body(
   // Checksum positions are taken mod 2^32, exactly as the weights are.
   const uint32_t csum_base = (uint32_t)(s.dst_off + (uint64_t)r0 * s.dst_pitch) + s.csum_bias;
 
-  Csum cs;
+  typename std::conditional<DIGEST, DigestAcc, Csum>::type cs;
+  if constexpr (DIGEST) cs.init(dst_sizes[s.dst_buf], s.dst_off + (uint64_t)r0 * s.dst_pitch, csum_base);
   if constexpr (CHECKSUM_ONLY) {
     switch (s.unit) {
       case 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
@@ -309,7 +387,31 @@ __device__ __forceinline__ void place_body(
     default: break;  // the host validates (op, unit) before upload
   }
 
-  if (s.csum_slot != 0xFFFFFFFFu) {
+  if constexpr (DIGEST) {
+    // five 64-bit sums and the checksum per workgroup: wavefront reductions, then one lane adds them up
+    __shared__ unsigned long long dpart[kPlaceThreads / 64][5];
+    __shared__ uint32_t part[kPlaceThreads / 64];
+    const unsigned long long v0 = wave_sum_u64(cs.S), v1 = wave_sum_u64(cs.SW), v2 = wave_sum_u64(cs.T),
+                             v3 = wave_sum_u64(cs.TW), v4 = wave_sum_u64(cs.RG);
+    const uint32_t wsum = wave_sum_u32(cs.cs.fold());
+    if ((threadIdx.x & 63) == 0) {
+      unsigned long long* row = dpart[threadIdx.x >> 6];
+      row[0] = v0; row[1] = v1; row[2] = v2; row[3] = v3; row[4] = v4;
+      part[threadIdx.x >> 6] = wsum;
+    }
+    __syncthreads();
+    if (threadIdx.x < 5) {
+      unsigned long long t = 0;
+#pragma unroll
+      for (int k = 0; k < kPlaceThreads / 64; ++k) t += dpart[k][threadIdx.x];
+      if (t) atomicAdd(&digest_sums[5ull * s.dst_buf + threadIdx.x], t);
+    } else if (threadIdx.x == 64 && s.csum_slot != 0xFFFFFFFFu) {
+      uint32_t t = 0;
+#pragma unroll
+      for (int k = 0; k < kPlaceThreads / 64; ++k) t += part[k];
+      atomicAdd(&sums[s.csum_slot], t);
+    }
+  } else if (s.csum_slot != 0xFFFFFFFFu) {
     __shared__ uint32_t part[kPlaceThreads / 64];
     const uint32_t wsum = wave_sum_u32(cs.fold());
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = wsum;
@@ -329,6 +431,16 @@ __global__ __launch_bounds__(kPlaceThreads) void place_kernel(
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
     uint32_t* __restrict__ sums, uint32_t nan_bits) {
   place_body<false>(segs, work, src_bases, dst_bases, sums, nan_bits);
+}
+
+// place_kernel that also accumulates the tensor_digest sums of every destination buffer
+// (five 64-bit words per buffer in `digest_sums`; `dst_sizes` holds the buffers' byte sizes).
+__global__ __launch_bounds__(kPlaceThreads) void place_digest_kernel(
+    const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
+    const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
+    uint32_t* __restrict__ sums, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes,
+    unsigned long long* __restrict__ digest_sums) {
+  place_body<false, true>(segs, work, src_bases, dst_bases, sums, nan_bits, dst_sizes, digest_sums);
 }
 
 // Read-only variant for batches made of checksum-only segments.
@@ -355,6 +467,9 @@ hipError_t configure_place_kernels() {
   if (e == hipSuccess)
     e = hipFuncSetAttribute(reinterpret_cast<const void*>(checksum_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)kOnePerCu);
+  if (e == hipSuccess)
+    e = hipFuncSetAttribute(reinterpret_cast<const void*>(place_digest_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)kOnePerCu);
   if (e == hipSuccess) configured.fetch_or(bit, std::memory_order_release);
   return e;
 }
@@ -372,6 +487,17 @@ hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t 
   }
   hipLaunchKernelGGL(place_kernel, dim3(n_work), dim3(kPlaceThreads), lds_place, stream, segs_dev,
                      work_dev, src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits);
+  return hipGetLastError();
+}
+
+hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
+                               const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev,
+                               const unsigned long long* dst_sizes_dev, unsigned long long* digest_sums_dev,
+                               uint16_t nan_bits, hipStream_t stream) {
+  if (n_work == 0) return hipSuccess;
+  if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
+  hipLaunchKernelGGL(place_digest_kernel, dim3(n_work), dim3(kPlaceThreads), kOnePerCu, stream, segs_dev, work_dev,
+                     src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits, dst_sizes_dev, digest_sums_dev);
   return hipGetLastError();
 }
 

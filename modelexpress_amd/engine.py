@@ -274,6 +274,17 @@ class PlacementEngine:
                                              C.byref(stats) if timed else None))
         return stats.as_dict() if timed else None
 
+    def set_fused_digests(self, on: bool = True) -> None:
+        """Placements also accumulate the ``tensor_digest`` sums of every parameter inside the placement kernel."""
+        L.check(L.lib().mxp_engine_set_fused_digests(self._h, 1 if on else 0))
+
+    def digests(self, plan: PlacementPlan) -> list[str]:
+        """The ``tensor_digest`` of every parameter as the last execute of ``plan`` left it (fused digests on)."""
+        n = len(plan.params)
+        out = (C.c_uint8 * (16 * max(1, n)))()
+        L.check(L.lib().mxp_plan_digests(self._h, plan._h, out, n))
+        return [bytes(out[16 * i: 16 * i + 16]).hex() for i in range(n)]
+
     def checksums(self, plan: PlacementPlan) -> list[str]:
         n = len(plan.params)
         out = (C.c_uint32 * max(1, n))()

@@ -197,12 +197,17 @@ class HipRefitAdapter:
         with rec.span("setup_registration"):
             buffers = list(self.layout.destinations) if self.in_place else eng.allocate(plan.plan)
         with rec.span("wire_transfer"):
-            stats = eng.execute(plan.plan, buffers)
+            # checksums and tensor_digest sums are accumulated by the placement kernel itself: what is
+            # verified below is what was written, with no second pass over the staged buffers
+            eng.set_fused_digests(True)
+            try:
+                stats = eng.execute(plan.plan, buffers)
+            finally:
+                eng.set_fused_digests(False)
             sums = eng.checksums(plan.plan)
         rec.bytes = stats["placed_bytes"]
         with rec.span("receive_sync"):
-            sizes = [p.nbytes for p in plan.plan.params]
-            digests = eng.digest(buffers, sizes)
+            digests = eng.digests(plan.plan)
             staged = StagedWeights(plan, buffers, sums, digests, stats, self.in_place)
             self._verify(staged)
         return staged

@@ -168,3 +168,81 @@ def test_empty_and_scalar_tensors(gpu_engine, gpu_engine_band, oracle, tmp_path,
             assert d.cpu().numpy().tobytes() == oparams[p.name].tobytes(), p.name
             assert s == oracle.safe_checksum(oparams[p.name]), p.name
     assert gpu_engine.checksum32([torch.empty(0, dtype=torch.uint8, device="cuda")]) == ["00000000"]
+
+
+@pytest.mark.parametrize("name", list(tiny_layouts()))
+def test_fused_digests_match_oracle(name, oracle, tmp_path, mxp):
+    """With fused digests on, the placement kernel accumulates the ``tensor_digest`` sums of what it stores
+    (refit/reshard/verify.py:112-150): for every family, every execution mode and the casts, the digest of
+    each parameter equals the oracle's digest of the expected bytes and the stand-alone digest of the
+    finished buffer; bytes and checksums are unchanged."""
+    from modelexpress_amd.engine import PlacementEngine
+
+    layout, tp, ep, shards, ck_kw = tiny_layouts()[name]
+    ck_kw, param_dtype, cast, _ratio = cast_setup(ck_kw)
+    synth.write_checkpoint(layout.checkpoint(**ck_kw), str(tmp_path), n_shards=shards, seed=17)
+    tp_rank = tp - 1
+    rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=tp_rank % ep, param_dtype=param_dtype)
+    want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
+    ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
+    for mode, kw in (("ingest", {}), ("ingest_band", dict(ring_slots=3, slot_bytes=1 << 16, pack_strided_on_host=False)), ("resident", {})):
+        eng = PlacementEngine(0, **kw)
+        dst = eng.allocate(plan, fill=0x5A)
+        with pytest.raises(mxp.MxpError, match="did not accumulate digests"):
+            eng.execute(plan, dst) if mode != "resident" else eng.execute_resident(plan, _stage_files(ck), dst)
+            torch.cuda.synchronize()
+            eng.digests(plan)
+        eng.set_fused_digests(True)
+        for _ in range(2):  # the sums are cleared by every execute
+            if mode == "resident":
+                eng.execute_resident(plan, _stage_files(ck), dst)
+            else:
+                eng.execute(plan, dst)
+        fused = eng.digests(plan)
+        alone = eng.digest(dst, [p.nbytes for p in plan.params])
+        sums = eng.checksums(plan)
+        for p, d, f, a, s in zip(plan.params, dst, fused, alone, sums):
+            assert d.cpu().numpy().tobytes() == want[p.name].tobytes(), (name, mode, p.name)
+            assert f == a == oracle.tensor_digest(want[p.name]), (name, mode, p.name)
+            assert s == oracle.safe_checksum(want[p.name]), (name, mode, p.name)
+        eng.close()
+
+
+def test_fused_digests_on_odd_sizes_and_narrow_paths(oracle, tmp_path, mxp):
+    """Buffers whose size is not a multiple of 4 (ragged bytes), of 4 KiB (tail words) or of 16 (head / tail
+    pieces moved by the 4-, 2- and 1-byte paths), a column slice with odd row length, and a narrowing cast with
+    an odd element count: the fused digest still equals the oracle's and the stand-alone one."""
+    from safetensors.numpy import save_file
+
+    from modelexpress_amd.engine import Checkpoint, ParamSpec, PlacementEngine, PlacementPlan
+
+    rng = np.random.default_rng(5)
+    tensors = {
+        "u8_ragged": rng.integers(0, 256, 4096 * 3 + 4 * 17 + 3, dtype=np.uint8),   # rows + tail words + 3 ragged bytes
+        "u8_tiny": rng.integers(0, 256, 7, dtype=np.uint8),                           # one word + ragged
+        "u8_one": rng.integers(0, 256, 1, dtype=np.uint8),
+        "f16_odd": rng.integers(0, 1 << 16, 4099, dtype=np.uint16).view(np.float16),  # n % 4 == 2
+        "f32_odd": rng.standard_normal(2051).astype(np.float32),                      # cast to bf16: n % 4 == 2
+        "cols": rng.integers(0, 256, (37, 52), dtype=np.uint8),                       # TP column slice: 26-byte rows off the 4-byte grid
+        "rows": rng.integers(-2 ** 31, 2 ** 31, (6, 1027), dtype=np.int64).astype(np.int32),  # negative words, row slice
+    }
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    ck = Checkpoint(str(tmp_path))
+    params = [ParamSpec("u8_ragged", "U8", (tensors["u8_ragged"].size,)), ParamSpec("u8_tiny", "U8", (7,)), ParamSpec("u8_one", "U8", (1,)),
+              ParamSpec("f16_odd", "F16", (4099,)), ParamSpec("f32_odd", "BF16", (2051,)), ParamSpec("cols", "U8", (37, 26)),
+              ParamSpec("rows", "I32", (3, 1027))]
+    plan = PlacementPlan(ck, params, tp_size=2, tp_rank=1, allow_cast=True)
+    want = {"u8_ragged": tensors["u8_ragged"], "u8_tiny": tensors["u8_tiny"], "u8_one": tensors["u8_one"], "f16_odd": tensors["f16_odd"],
+            "f32_odd": oracle.cast_f32_bf16_bits(tensors["f32_odd"].view(np.uint32)).astype(np.uint16)}
+    want["cols"] = np.ascontiguousarray(tensors["cols"][:, 26:])  # 26-byte rows: 2-byte units
+    want["rows"] = np.ascontiguousarray(tensors["rows"][3:])
+    eng = PlacementEngine(0)
+    eng.set_fused_digests(True)
+    dst = eng.allocate(plan, fill=0)
+    eng.execute(plan, dst)
+    fused, alone = eng.digests(plan), eng.digest(dst, [p.nbytes for p in plan.params])
+    for p, d, f, a in zip(plan.params, dst, fused, alone):
+        got = d.cpu().numpy().tobytes()
+        assert got == np.ascontiguousarray(want[p.name]).tobytes(), p.name
+        assert f == a == oracle.tensor_digest_bytes(got), p.name
+    eng.close()
