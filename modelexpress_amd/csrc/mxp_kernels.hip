@@ -86,44 +86,108 @@ __device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v)
 struct DigestAcc {
   Csum cs;
   unsigned long long S = 0, SW = 0, T = 0, TW = 0, RG = 0;
+  // Whole-row words of this tile, kept as 32-bit sums until the tile is done: low halves
+  // (unsigned) and high halves (signed) of the words apart, plain and weighted by the row's
+  // distance from the tile's first row.  A lane adds at most 64 units of at most 4 words at
+  // distances below 64, so nothing wraps; rows further away take the 64-bit route.
+  uint32_t a_lo = 0, b_lo = 0;
+  int32_t a_hi = 0, b_hi = 0;
+  uint64_t row0 = 0;        // row (4 KiB of the buffer) the tile starts in
   uint64_t base = 0;        // position of the tile's first destination byte inside its buffer
   uint32_t base32 = 0;      // the 32-bit checksum position the callers count from
-  uint64_t tail_word0 = 0;  // first word after the last whole row
+  uint64_t tail_byte0 = 0;  // first byte after the last whole row
   uint64_t body_end = 0;    // first ragged byte
   __device__ __forceinline__ void init(uint64_t buffer_bytes, uint64_t tile_pos, uint32_t tile_pos32) {
     base = tile_pos;
     base32 = tile_pos32;
+    row0 = tile_pos >> 12;
     body_end = buffer_bytes & ~3ull;
-    tail_word0 = (buffer_bytes >> 2) / kDigestRowWords * kDigestRowWords;
+    tail_byte0 = buffer_bytes / (4ull * kDigestRowWords) * (4ull * kDigestRowWords);
   }
-  // Whole words starting at byte position p (a multiple of 4; all in one row): `sum` of the
-  // words and `ramp` = sum of word k times k, both as signed 64-bit values.
-  __device__ __forceinline__ void words(long long sum, long long ramp, uint64_t p) {
-    const uint64_t wi = p >> 2;
-    if (wi < tail_word0) {
-      S += (unsigned long long)sum;
-      SW += (unsigned long long)sum * (unsigned long long)(wi / kDigestRowWords + 1);
-    } else {
-      T += (unsigned long long)sum;
-      TW += (unsigned long long)sum * (unsigned long long)(wi - tail_word0 + 1) + (unsigned long long)ramp;
-    }
+  static_assert(kDigestRowWords == 1024, "rows are 4 KiB: the row of byte p is p >> 12");
+  typedef short s16x2 __attribute__((ext_vector_type(2)));
+  typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+  static __device__ __forceinline__ uint32_t lo_add(uint32_t w, uint32_t acc) {
+    u16x2 v;
+    __builtin_memcpy(&v, &w, 4);
+    const u16x2 one_zero = {1, 0};
+    return __builtin_amdgcn_udot2(v, one_zero, acc, false);
+  }
+  static __device__ __forceinline__ int32_t hi_add(uint32_t w, int32_t acc) {
+    s16x2 v;
+    __builtin_memcpy(&v, &w, 4);
+    const s16x2 zero_one = {0, 1};
+    return __builtin_amdgcn_sdot2(v, zero_one, acc, false);
+  }
+  // Words after the last whole row: `sum` of the words and `ramp` = sum of word k times k.
+  __device__ __forceinline__ void tail_words(long long sum, long long ramp, uint64_t p) {
+    T += (unsigned long long)sum;
+    TW += (unsigned long long)sum * (unsigned long long)(((p - tail_byte0) >> 2) + 1) + (unsigned long long)ramp;
+  }
+  // Whole-row words far from the tile's first row (pitched boxes with a large pitch).
+  __device__ __forceinline__ void far_words(long long sum, uint64_t p) {
+    S += (unsigned long long)sum;
+    SW += (unsigned long long)sum * (unsigned long long)((p >> 12) + 1);
   }
   __device__ __forceinline__ void add16(const uint4& x, uint32_t i) {
     cs.add16(x, i);
-    const long long a = (int32_t)x.x, b = (int32_t)x.y, c = (int32_t)x.z, d = (int32_t)x.w;
-    words(a + b + c + d, b + 2 * c + 3 * d, base + (uint32_t)(i - base32));
+    const uint64_t p = base + (uint32_t)(i - base32);
+    const uint64_t dr = (p >> 12) - row0;
+    if (p < tail_byte0 && dr < 64) {
+      const uint32_t lo = lo_add(x.w, lo_add(x.z, lo_add(x.y, lo_add(x.x, 0u))));
+      const int32_t hi = hi_add(x.w, hi_add(x.z, hi_add(x.y, hi_add(x.x, 0))));
+      a_lo += lo;
+      a_hi += hi;
+      b_lo += lo * (uint32_t)dr;
+      b_hi += hi * (int32_t)dr;
+    } else {
+      const long long a = (int32_t)x.x, b = (int32_t)x.y, c = (int32_t)x.z, d = (int32_t)x.w;
+      if (p < tail_byte0) far_words(a + b + c + d, p);
+      else tail_words(a + b + c + d, b + 2 * c + 3 * d, p);
+    }
   }
-  __device__ __forceinline__ void add8(uint32_t lo, uint32_t hi, uint32_t i) {
-    cs.add8(lo, hi, i);
-    const long long a = (int32_t)lo, b = (int32_t)hi;
-    words(a + b, b, base + (uint32_t)(i - base32));
+  __device__ __forceinline__ void add8(uint32_t lo_w, uint32_t hi_w, uint32_t i) {
+    cs.add8(lo_w, hi_w, i);
+    const uint64_t p = base + (uint32_t)(i - base32);
+    const uint64_t dr = (p >> 12) - row0;
+    if (p < tail_byte0 && dr < 64) {
+      const uint32_t lo = lo_add(hi_w, lo_add(lo_w, 0u));
+      const int32_t hi = hi_add(hi_w, hi_add(lo_w, 0));
+      a_lo += lo;
+      a_hi += hi;
+      b_lo += lo * (uint32_t)dr;
+      b_hi += hi * (int32_t)dr;
+    } else {
+      const long long a = (int32_t)lo_w, b = (int32_t)hi_w;
+      if (p < tail_byte0) far_words(a + b, p);
+      else tail_words(a + b, b, p);
+    }
+  }
+  // Folds the tile's 32-bit sums into the 64-bit ones; call once, after the last add.
+  __device__ __forceinline__ void flush() {
+    const long long s = (long long)a_hi * 65536 + (long long)a_lo;
+    const long long sw = (long long)b_hi * 65536 + (long long)b_lo;
+    S += (unsigned long long)s;
+    SW += (unsigned long long)sw + (unsigned long long)s * (unsigned long long)(row0 + 1);
   }
   template <int UNIT>
   __device__ __forceinline__ void addn(uint32_t x, uint32_t i) {
     cs.add4(x, i);
     const uint64_t p = base + (uint32_t)(i - base32);
     if constexpr (UNIT == 4) {
-      words((long long)(int32_t)x, 0, p);
+      const uint64_t dr = (p >> 12) - row0;
+      if (p < tail_byte0 && dr < 64) {
+        const uint32_t lo = lo_add(x, 0u);
+        const int32_t hi = hi_add(x, 0);
+        a_lo += lo;
+        a_hi += hi;
+        b_lo += lo * (uint32_t)dr;
+        b_hi += hi * (int32_t)dr;
+      } else if (p < tail_byte0) {
+        far_words((long long)(int32_t)x, p);
+      } else {
+        tail_words((long long)(int32_t)x, 0, p);
+      }
     } else {  // part of a word, or ragged bytes: byte by byte
 #pragma unroll
       for (int e = 0; e < UNIT; ++e) {
@@ -135,14 +199,8 @@ struct DigestAcc {
         }
         const uint32_t j = (uint32_t)q & 3u;
         const long long v = j == 3u ? (long long)(int32_t)(b << 24) : (long long)(b << (8u * j));
-        const uint64_t wi = q >> 2;
-        if (wi < tail_word0) {
-          S += (unsigned long long)v;
-          SW += (unsigned long long)v * (unsigned long long)(wi / kDigestRowWords + 1);
-        } else {
-          T += (unsigned long long)v;
-          TW += (unsigned long long)v * (unsigned long long)(wi - tail_word0 + 1);
-        }
+        if (q < tail_byte0) far_words(v, q);
+        else tail_words(v, 0, q & ~3ull);
       }
     }
   }
@@ -391,6 +449,7 @@ __device__ __forceinline__ void place_body(
     // five 64-bit sums and the checksum per workgroup: wavefront reductions, then one lane adds them up
     __shared__ unsigned long long dpart[kPlaceThreads / 64][5];
     __shared__ uint32_t part[kPlaceThreads / 64];
+    cs.flush();
     const unsigned long long v0 = wave_sum_u64(cs.S), v1 = wave_sum_u64(cs.SW), v2 = wave_sum_u64(cs.T),
                              v3 = wave_sum_u64(cs.TW), v4 = wave_sum_u64(cs.RG);
     const uint32_t wsum = wave_sum_u32(cs.cs.fold());
