@@ -62,6 +62,8 @@ environment_variables: dict[str, Callable[[], Any]] = {
     # refuse a refit that writes less than the floor fraction of the engine's parameter bytes.
     "MX_RESHARD_REQUIRE_FULL_COVERAGE": lambda: _env_bool("MX_RESHARD_REQUIRE_FULL_COVERAGE", False),
     "MX_RESHARD_COVERAGE_FLOOR": lambda: _env_float("MX_RESHARD_COVERAGE_FLOOR", 0.995),
+    # Publishers stamp every served tensor with its digest (modelexpress/envs.py:304); off by default, read live.
+    "MX_RESHARD_PUBLISH_DIGEST": lambda: _env_bool("MX_RESHARD_PUBLISH_DIGEST", False),
 }
 
 

@@ -20,6 +20,7 @@ from typing import Any
 import torch
 
 from . import _lib as L
+from . import envs
 from .engine import CAST_CODES, PlacementEngine
 from .load_strategy import safetensors_dtype_of
 
@@ -34,9 +35,9 @@ class WireStager:
 
     supported_staging_modes = frozenset({COPY_TO_DEVICE, IN_PLACE})
 
-    def __init__(self, engine: PlacementEngine, *, publish_digests: bool = False):
+    def __init__(self, engine: PlacementEngine, *, publish_digests: bool | None = None):
         self.engine = engine
-        self.publish_digests = publish_digests
+        self._publish_digests = publish_digests  # None: follow MX_RESHARD_PUBLISH_DIGEST, read at every stage
         self._initialized = False
         self._staging_mode: str | None = None
         self._expected_layout: dict[str, tuple] = {}
@@ -111,7 +112,7 @@ class WireStager:
                                               "use COPY_TO_DEVICE")
             served = shards
         digests = None
-        if self.publish_digests:
+        if envs.MX_RESHARD_PUBLISH_DIGEST if self._publish_digests is None else self._publish_digests:
             names = list(served)
             digests = dict(zip(names, self.engine.digest([served[n] for n in names], stream=stream)))
         wire = torch.empty((), dtype=WIRE_DTYPE).element_size()

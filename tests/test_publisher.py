@@ -69,6 +69,21 @@ def test_copy_to_device_snapshot_matches_copy_(gpu_engine, oracle):
 
 
 @pytest.mark.gpu
+def test_digest_publication_follows_the_environment_live(gpu_engine, monkeypatch):
+    # tests/test_reshard_refit_verify.py:175-194: off by default, read at every stage, not frozen at import
+    st = WireStager(gpu_engine)
+    state = {"w": torch.arange(64, dtype=torch.float32).cuda()}
+    monkeypatch.delenv("MX_RESHARD_PUBLISH_DIGEST", raising=False)
+    assert st.stage(state)["digests"] is None
+    monkeypatch.setenv("MX_RESHARD_PUBLISH_DIGEST", "1")
+    out = st.stage(state)
+    assert out["digests"] == {"w": gpu_engine.digest([out["served"]["w"]])[0]}
+    monkeypatch.setenv("MX_RESHARD_PUBLISH_DIGEST", "0")
+    assert st.stage(state)["digests"] is None
+    st.close()
+
+
+@pytest.mark.gpu
 def test_colocated_refit_trainer_snapshot_to_engine_parameters(gpu_engine):
     """Both ends on one GPU: the trainer's fp32 state dict is snapshotted into bf16 arenas (one launch), the
     engine's own loaders are captured once on a meta twin, and each step re-slices the arenas into the live
