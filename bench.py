@@ -458,7 +458,7 @@ def main() -> int:
             agree = agree and [applied[p.name] for p in rv.params] == resident_sums
             out["refit_cycle"] = {"wall_s": best["wall_s"], "placed_gbps": round(placed / best["wall_s"] / 1e9, 2),
                                   "stages_s": {k: v["duration_s"] for k, v in best["stages"].items()},
-                                  "note": "plan + ingest with fp32->bf16 cast into staging + device digests + one batched install "
+                                  "note": "plan + ingest with fp32->bf16 cast into staging (checksums and digest sums fused) + verify + one batched install "
                                           "into the live buffers, through HipRefitAdapter (best of 3)",
                                   "checksums_match_resident": [applied[p.name] for p in rv.params] == resident_sums}
             _log(f"refit_cycle: {out['refit_cycle']}")
