@@ -246,3 +246,34 @@ def test_fused_digests_on_odd_sizes_and_narrow_paths(oracle, tmp_path, mxp):
         assert got == np.ascontiguousarray(want[p.name]).tobytes(), p.name
         assert f == a == oracle.tensor_digest_bytes(got), p.name
     eng.close()
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_models_on_the_device(seed, oracle, tmp_path, mxp):
+    """The seeded random models of test_planner_random (odd extents down to one element, 0-D to 4-D tensors, TP
+    on any axis, fused groups on either axis, premerged pairs, fp32 into bf16) executed on the device, ingest and
+    resident, with fused digests: bytes, checksums and digests against the oracle."""
+    from test_planner_random import build_random_model, oracle_result
+
+    from modelexpress_amd.engine import Checkpoint, ParamSpec, PlacementEngine, PlacementPlan
+
+    path, params, tp, rank, cast = build_random_model(seed, tmp_path)
+    want = oracle_result(oracle, path, params, tp, rank, cast)
+    if want is None:
+        pytest.skip("the oracle refuses this model (the planner's refusal is checked on the CPU)")
+    ck = Checkpoint(str(path))
+    plan = PlacementPlan(ck, [ParamSpec(n, dt, tuple(shape)) for n, (dt, shape) in params.items()], tp_size=tp, tp_rank=rank,
+                         allow_cast=cast)
+    eng = PlacementEngine(0, ring_slots=3, slot_bytes=1 << 16)
+    eng.set_fused_digests(True)
+    for mode in ("ingest", "resident"):
+        dst = eng.allocate(plan, fill=0x3C)
+        if mode == "resident":
+            eng.execute_resident(plan, _stage_files(ck), dst)
+        else:
+            eng.execute(plan, dst)
+        sums, digests = eng.checksums(plan), eng.digests(plan)
+        for p, d, s, g in zip(plan.params, dst, sums, digests):
+            assert d.cpu().numpy().tobytes()[: p.nbytes] == want[p.name].tobytes(), (seed, mode, p.name)
+            assert s == oracle.safe_checksum(want[p.name]) and g == oracle.tensor_digest(want[p.name]), (seed, mode, p.name)
+    eng.close()

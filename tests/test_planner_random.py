@@ -24,8 +24,8 @@ def _rand(rng, shape, dt):
     return torch.from_numpy(rng.integers(-3000, 3000, n, dtype=np.int16)).reshape(shape)
 
 
-@pytest.mark.parametrize("seed", range(40))
-def test_random_model(seed, oracle, mxp, tmp_path):
+def build_random_model(seed, tmp_path):
+    """Writes the seeded random checkpoint; returns (directory, {param: (dtype, shape)}, tp, rank, cast)."""
     rng = np.random.default_rng(1000 + seed)
     tp = int(rng.choice([1, 2, 3, 4]))
     rank = int(rng.integers(0, tp))
@@ -72,6 +72,22 @@ def test_random_model(seed, oracle, mxp, tmp_path):
     path = tmp_path / "ck"
     path.mkdir()
     save_file({n: t.contiguous() for n, t in tensors.items()}, str(path / "model.safetensors"))
+    return path, params, tp, rank, cast
+
+
+def oracle_result(oracle, path, params, tp, rank, cast):
+    """The oracle's parameters, or None where it refuses the model (ambiguous shapes)."""
+    oparams = {n: oracle.OTensor.zeros(shape, dt) for n, (dt, shape) in params.items()}
+    try:
+        oracle.MdlOracle(oparams, tp, rank, allow_cast=cast).load_weights(oracle.load_checkpoint(str(path)))
+    except oracle.CoverageError:
+        return None
+    return oparams
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_model(seed, oracle, mxp, tmp_path):
+    path, params, tp, rank, cast = build_random_model(seed, tmp_path)
     OT = oracle.OTensor
     oparams = {n: OT.zeros(shape, dt) for n, (dt, shape) in params.items()}
     try:
