@@ -22,7 +22,6 @@ resolution order, but the bytes go file -> pinned ring -> HBM -> placement kerne
 from __future__ import annotations
 
 import logging
-import os
 from abc import ABC, abstractmethod
 from dataclasses import dataclass, field
 from typing import Any, Callable, ClassVar, Generic, Iterator, Sequence, TypeVar

@@ -11,13 +11,12 @@ from __future__ import annotations
 import ctypes as C
 import json
 import mmap
-import os
 import struct
 import zlib
 from pathlib import Path
 
 from . import _lib as L
-from .models import FP8_FINITE, NORMAL, SCALE, TensorSpec
+from .models import FP8_FINITE, SCALE, TensorSpec
 
 
 def tensor_seed(base_seed: int, name: str) -> int:
