@@ -36,6 +36,10 @@ VIEW_OPS: dict[Callable, str] = {
     torch.Tensor.transpose: "transpose", torch.Tensor.t: "t", torch.Tensor.permute: "permute",
     torch.Tensor.flatten: "flatten", torch.Tensor.contiguous: "contiguous", torch.Tensor.chunk: "chunk",
     torch.Tensor.unbind: "unbind",
+    # the same calls spelled as functions (torch.narrow(w, ...)): replayed as the method
+    torch.narrow: "narrow", torch.reshape: "reshape", torch.unsqueeze: "unsqueeze", torch.squeeze: "squeeze",
+    torch.transpose: "transpose", torch.t: "t", torch.permute: "permute", torch.flatten: "flatten", torch.chunk: "chunk",
+    torch.unbind: "unbind",
 }
 
 

@@ -200,6 +200,9 @@ def test_probe_reports_metadata_without_dispatching():
     v = p.narrow(0, 2, 3).t()
     assert v.shape == (10, 3) and v.dtype == torch.bfloat16 and v.dim() == 2 and v.size(0) == 10 and not v.is_contiguous()
     assert v._probe_ops == (("narrow", (0, 2, 3), ()), ("t", (), ()))
+    f = torch.narrow(torch.t(p), 1, 1, 4)  # function spellings record the same ops
+    assert f.shape == (10, 4) and f._probe_ops == (("t", (), ()), ("narrow", (1, 1, 4), ()))
+    assert replay_view(f._probe_ops, (6, 10)) == (10, (10, 4), (1, 10))
     a, b = p.chunk(2, dim=1)
     assert a.shape == (6, 5) and b._probe_ops == (("chunk", (2,), (("dim", 1),)), ("__getitem__", (1,), ()))
     assert isinstance(CaptureResult().copies, list)
