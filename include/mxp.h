@@ -300,6 +300,18 @@ int mxp_plan_digests(mxp_engine* engine, mxp_plan* plan, uint8_t* out16, int64_t
  *   out[k] = sum_i byte_i * ((i * 2654435761 + 1) mod 2^32) mod 2^32. */
 int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
                    uint32_t* out, void* stream);
+/* mxp_checksum32 for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+ * results as mxp_checksum32; the descriptor tables and accumulators its kernel reads live in a
+ * 1 MiB device array that is part of the library image (one copy per GPU, held until the process
+ * ends) and in a pinned mirror allocated by mxp_engine_create, so the call itself allocates and
+ * frees nothing on the host or the device.  Limits: n <= 1024 buffers and at most 98,304
+ * workgroups of 128 KiB in all (about 12 GiB); beyond them the call fails with MXP_ERR_ARG and
+ * launches nothing.  Every call on a GPU - from any engine - uses that GPU's one array: calls
+ * that overlap in time on one GPU race and must be serialised by the caller.  Blocks until
+ * `stream` is idle, like mxp_checksum32. */
+int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
+                          uint32_t* out, void* stream);
 /* tensor_digest (refit/reshard/verify.py:79-155) of n device buffers: 16 bytes each
  * (blake2b-128 over the little-endian u64 scalars).  `scalars`, if not NULL, receives
  * 7 u64 per tensor: n, sum_rows, sum_rows_weighted, sum_tail, sum_tail_weighted,

@@ -146,6 +146,7 @@ SIGNATURES = {
     "mxp_execute_resident": (C.c_int, [_P, _P, _PP, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_plan_checksums": (C.c_int, [_P, _P, _U32P, C.c_int64]),
     "mxp_checksum32": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
+    "mxp_checksum32_static": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_digest": (C.c_int, [_P, _PP, _U64P, C.c_int64, C.POINTER(C.c_uint8), _U64P, _P]),
     "mxp_cast_f32_bf16": (C.c_int, [_P, _P, _P, C.c_uint64, _U32P, _P]),
     "mxp_cast": (C.c_int, [_P, _P, _P, C.c_uint64, C.c_int32, _U32P, _P]),

@@ -34,6 +34,55 @@ namespace {
       throw Error(MXP_ERR_DEVICE, std::string(#expr) + ": " + hipGetErrorString(e_));         \
   } while (0)
 
+// Scratch of the entry point that allocates nothing (mxp_checksum32_static): descriptor tables,
+// source pointers and checksum accumulators of one call.  One copy per GPU, held until the
+// process ends; every call on a GPU shares it.  Host code never uses the array's name as an
+// address: mxp_engine_create looks the device address up once per device (static_scratch_for)
+// and everything else goes through that pointer.
+constexpr size_t kStaticMaxBuffers = 1024;                       // buffers per call
+constexpr size_t kStaticMaxSegs = 3 * kStaticMaxBuffers;         // a contiguous run lowers to at most 3 segments
+constexpr size_t kStaticMaxWork = 96 * 1024;                     // workgroups per call (128 KiB each: 12 GiB)
+constexpr size_t kStaticOffSegs = 0;
+constexpr size_t kStaticOffWork = kStaticOffSegs + kStaticMaxSegs * sizeof(Seg);
+constexpr size_t kStaticOffPtrs = kStaticOffWork + kStaticMaxWork * sizeof(WorkItem);
+constexpr size_t kStaticOffSums = kStaticOffPtrs + kStaticMaxBuffers * sizeof(void*);
+constexpr size_t kStaticScratchBytes = 1u << 20;
+static_assert(kStaticOffSums + kStaticMaxBuffers * sizeof(uint32_t) <= kStaticScratchBytes, "scratch layout");
+static_assert(kStaticOffWork % 256 == 0 && kStaticOffPtrs % 256 == 0 && kStaticOffSums % 256 == 0, "scratch layout");
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};  // device address of `scratch` on each GPU
+
+// Device address of this GPU's copy of `scratch`; `device` must be current.
+unsigned char* static_scratch_for(int device) {
+  if (device < 0 || device >= kMaxDevices) throw Error(MXP_ERR_ARG, "device ordinal out of range");
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[device]) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      throw Error(MXP_ERR_DEVICE, std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(e));
+    g_scratch_ptr[device] = static_cast<unsigned char*>(p);
+  }
+  return g_scratch_ptr[device];
+}
+
+// push_back / size over memory the caller owns; refuses to grow.
+template <typename T>
+struct FixedTable {
+  T* p;
+  size_t cap, n = 0;
+  const char* what;
+  FixedTable(void* mem, size_t capacity, const char* name) : p(static_cast<T*>(mem)), cap(capacity), what(name) {}
+  void push_back(const T& v) {
+    if (n == cap) throw Error(MXP_ERR_ARG, std::string(what));
+    p[n++] = v;
+  }
+  size_t size() const { return n; }
+};
+
 double now_s() {
   return std::chrono::duration<double>(std::chrono::steady_clock::now().time_since_epoch()).count();
 }
@@ -123,8 +172,12 @@ struct mxp_engine {
   DevBuf<TransposeItem> items_dev;
   hipEvent_t items_busy = nullptr;
   bool items_recorded = false;
+  // mxp_checksum32_static: this GPU's scratch array and a pinned mirror of it, both set up at create
+  unsigned char* static_dev = nullptr;
+  unsigned char* static_host = nullptr;  // pinned
 
   ~mxp_engine() {
+    if (static_host) (void)hipHostFree(static_host);
     if (arena_busy) (void)hipEventDestroy(arena_busy);
     if (items_busy) (void)hipEventDestroy(items_busy);
     if (items_host) (void)hipHostFree(items_host);
@@ -523,6 +576,8 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     HIP_OK(hipEventCreate(&e->ev_b));
     HIP_OK(hipEventCreateWithFlags(&e->arena_busy, hipEventDisableTiming));
     HIP_OK(hipEventCreateWithFlags(&e->items_busy, hipEventDisableTiming));
+    e->static_dev = static_scratch_for(o.device);
+    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e->static_host), kStaticScratchBytes, hipHostMallocDefault));
     *out = e.release();
   });
 }
@@ -848,6 +903,55 @@ int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* 
       boxes.push_back(b);
     }
     run_boxes(*engine, boxes, srcs, {}, (uint32_t)n, out, static_cast<hipStream_t>(stream));
+  });
+}
+
+int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
+                          uint32_t* out, void* stream_v) {
+  return guard([&] {
+    if (!engine || !out || n < 0 || (n && (!ptrs || !nbytes))) throw Error(MXP_ERR_ARG, "mxp_checksum32_static: bad argument");
+    if (n == 0) return;
+    if ((uint64_t)n > kStaticMaxBuffers)
+      throw Error(MXP_ERR_ARG, "mxp_checksum32_static: " + std::to_string(n) + " buffers in one call, the static scratch holds " +
+                                   std::to_string(kStaticMaxBuffers));
+    mxp_engine& e = *engine;
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    HIP_OK(hipSetDevice(e.opt.device));
+    // Tables are lowered straight into the pinned mirror; the previous call synchronised
+    // `stream` before it returned, so nothing still reads it.
+    unsigned char* h = e.static_host;
+    unsigned char* d = e.static_dev;
+    FixedTable<Seg> segs(h + kStaticOffSegs, kStaticMaxSegs, "mxp_checksum32_static: too many segments for the static scratch");
+    FixedTable<WorkItem> work(h + kStaticOffWork, kStaticMaxWork,
+                              "mxp_checksum32_static: the buffers need more than 98304 workgroups (about 12 GiB in all), "
+                              "the limit of the static scratch");
+    const void** src_tab = reinterpret_cast<const void**>(h + kStaticOffPtrs);
+    uint32_t* sums = reinterpret_cast<uint32_t*>(h + kStaticOffSums);
+    LowerOptions lo;
+    lo.tile_bytes = e.opt.tile_bytes;
+    for (int64_t k = 0; k < n; ++k) {
+      if (nbytes[k] && !ptrs[k]) throw Error(MXP_ERR_ARG, "mxp_checksum32_static: null pointer");
+      uint64_t off;
+      split_ptr(ptrs[k], src_tab[k], off);
+      BoxCopy b;
+      b.src_buf = (uint32_t)k;
+      b.src_off = off;
+      b.row_bytes = nbytes[k];
+      b.op = kOpChecksumOnly;
+      b.csum_slot = (uint32_t)k;
+      lower_box(b, lo, segs, work);
+      sums[k] = 0;  // the accumulators keep the last call's values: they are cleared by the upload below
+    }
+    if (segs.size()) HIP_OK(hipMemcpyAsync(d + kStaticOffSegs, h + kStaticOffSegs, segs.size() * sizeof(Seg), hipMemcpyHostToDevice, stream));
+    if (work.size()) HIP_OK(hipMemcpyAsync(d + kStaticOffWork, h + kStaticOffWork, work.size() * sizeof(WorkItem), hipMemcpyHostToDevice, stream));
+    // pointers and zeroed accumulators are neighbours: one copy up to the end of the used sums
+    HIP_OK(hipMemcpyAsync(d + kStaticOffPtrs, h + kStaticOffPtrs, kStaticOffSums - kStaticOffPtrs + (size_t)n * 4, hipMemcpyHostToDevice, stream));
+    HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + kStaticOffSegs), reinterpret_cast<const WorkItem*>(d + kStaticOffWork),
+                        (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + kStaticOffPtrs), nullptr,
+                        reinterpret_cast<uint32_t*>(d + kStaticOffSums), e.opt.nan_bits, stream, true));
+    HIP_OK(hipMemcpyAsync(h + kStaticOffSums, d + kStaticOffSums, (size_t)n * 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipStreamSynchronize(stream));
+    std::memcpy(out, sums, (size_t)n * 4);
   });
 }
 

@@ -30,8 +30,10 @@ struct LowerOptions {
   uint32_t max_row_bytes = 32768;   // wider pitched rows are split by columns
 };
 
-inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& segs,
-                     std::vector<WorkItem>& work) {
+// `SegTable` / `WorkTable` are anything with push_back and size: std::vector, or a fixed-capacity
+// view over memory the caller already owns.
+template <class SegTable, class WorkTable>
+inline void emit_seg(const BoxCopy& b, const LowerOptions& o, SegTable& segs, WorkTable& work) {
   if (b.rows == 0 || b.row_bytes == 0) return;
   if (b.rows > 0xFFFFFFFFull || b.row_bytes > o.max_row_bytes)
     throw std::logic_error("emit_seg: box not normalised");
@@ -102,8 +104,8 @@ inline void emit_seg(const BoxCopy& b, const LowerOptions& o, std::vector<Seg>& 
 }
 
 // Split one logical box into device segments.
-inline void lower_box(const BoxCopy& in, const LowerOptions& o, std::vector<Seg>& segs,
-                      std::vector<WorkItem>& work) {
+template <class SegTable, class WorkTable>
+inline void lower_box(const BoxCopy& in, const LowerOptions& o, SegTable& segs, WorkTable& work) {
   if (in.rows == 0 || in.row_bytes == 0) return;
   const uint32_t op = in.op;
   BoxCopy b = in;
