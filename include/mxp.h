@@ -269,13 +269,26 @@ int mxp_prepare(mxp_engine* engine, mxp_plan* plan);
  * the engine's streams, and the placement kernel for that slot runs on the same
  * stream.  `dst_ptrs[i]` is the device address of parameter i (16-byte aligned,
  * mxp_plan_param_info().nbytes long).  Blocks until every stream is idle.  Per
- * parameter checksums are left in the plan (mxp_plan_checksums). */
+ * parameter checksums are left in the plan (mxp_plan_checksums).
+ *
+ * Ordering: the engine's streams are private.  Before the first byte moves they wait for the
+ * work already queued on the caller's stream - the default (null) stream for mxp_execute,
+ * `caller_stream` for mxp_execute_after - so kernels still pending on the destinations
+ * (initialisation, reads of memory the caller's allocator has recycled into them) finish
+ * first, as they would ahead of destination.copy_(source) on that stream
+ * (installer.py:419-424).  Work the caller queues on other streams is the caller's to order.
+ * On return everything has completed, so later work needs no further ordering. */
 int mxp_execute(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs, mxp_exec_stats* stats);
+int mxp_execute_after(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs, void* caller_stream,
+                      mxp_exec_stats* stats);
 
 /* Same placement with the checkpoint already staged in HBM: `file_dev_ptrs[f]` holds
  * the complete bytes of shard file f (16-byte aligned).  One kernel launch on `stream`
  * for the whole plan; asynchronous unless `stats` is non-NULL (then it synchronises and
- * reports the HIP-event time of the launch in stats->kernel_ms). */
+ * reports the HIP-event time of the launch in stats->kernel_ms).  A plan's pointer tables and
+ * accumulators are its own: launches of one plan are serialised (a call on another stream than
+ * the previous one waits for that launch), and changed `dst_ptrs` / `file_dev_ptrs` reach the
+ * device by copies ordered on `stream`, never under a launch that still runs. */
 int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* file_dev_ptrs,
                          void* const* dst_ptrs, void* stream, mxp_exec_stats* stats);
 

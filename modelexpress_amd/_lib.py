@@ -143,6 +143,7 @@ SIGNATURES = {
     "mxp_engine_destroy": (None, [_P]),
     "mxp_prepare": (C.c_int, [_P, _P]),
     "mxp_execute": (C.c_int, [_P, _P, _PP, C.POINTER(ExecStats)]),
+    "mxp_execute_after": (C.c_int, [_P, _P, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_execute_resident": (C.c_int, [_P, _P, _PP, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_plan_checksums": (C.c_int, [_P, _P, _U32P, C.c_int64]),
     "mxp_checksum32": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),

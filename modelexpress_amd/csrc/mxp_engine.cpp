@@ -148,7 +148,20 @@ struct mxp_plan::Lowered {
   bool digests_valid = false;              // the last execute accumulated them
   std::vector<void*> dst_host;        // what dst_bases currently holds
   std::vector<const void*> src_host;  // what src_bases currently holds
+  // The pointer tables are rewritten with stream-ordered copies out of this pinned block
+  // ([destinations][sources]); `upload_done` guards the block, `launch_done` marks the last
+  // launch that reads the tables and accumulators, so a call on another stream waits for it.
+  void** tab_host = nullptr;
+  size_t tab_cap = 0;
+  hipEvent_t upload_done = nullptr, launch_done = nullptr;
+  bool upload_rec = false, launch_rec = false;
+  hipStream_t last_stream = nullptr;
   uint64_t file_bytes = 0, h2d_bytes = 0, placed_bytes = 0, algo_bytes = 0;
+  ~Lowered() {
+    if (tab_host) (void)hipHostFree(tab_host);
+    if (upload_done) (void)hipEventDestroy(upload_done);
+    if (launch_done) (void)hipEventDestroy(launch_done);
+  }
 };
 
 struct mxp_engine {
@@ -163,6 +176,7 @@ struct mxp_engine {
   size_t desc_host_cap = 0;
   DevBuf<uint8_t> desc_dev;
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
+  hipEvent_t caller_ev = nullptr;   // what the caller had queued when an ingest started
   bool fused_digests = false;       // placements also accumulate the tensor_digest sums (mxp_engine_set_fused_digests)
   hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
   bool arena_recorded = false;
@@ -179,6 +193,7 @@ struct mxp_engine {
   ~mxp_engine() {
     if (static_host) (void)hipHostFree(static_host);
     if (arena_busy) (void)hipEventDestroy(arena_busy);
+    if (caller_ev) (void)hipEventDestroy(caller_ev);
     if (items_busy) (void)hipEventDestroy(items_busy);
     if (items_host) (void)hipHostFree(items_host);
     for (auto s : streams) (void)hipStreamDestroy(s);
@@ -411,6 +426,10 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   L->dst_bases.reserve(pl.params.size() ? pl.params.size() : 1);
   L->src_bases.reserve(ck.files.size() ? ck.files.size() : 1);
   L->sums.reserve(pl.params.size() ? pl.params.size() : 1);
+  L->tab_cap = pl.params.size() + ck.files.size() + 1;
+  HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&L->tab_host), L->tab_cap * sizeof(void*), hipHostMallocDefault));
+  HIP_OK(hipEventCreateWithFlags(&L->upload_done, hipEventDisableTiming));
+  HIP_OK(hipEventCreateWithFlags(&L->launch_done, hipEventDisableTiming));
   {
     std::vector<unsigned long long> sizes;
     for (const auto& p : pl.params) sizes.push_back(p.nbytes);
@@ -431,12 +450,55 @@ void check_dst(const mxp_plan& pl, void* const* dst_ptrs) {
   }
 }
 
-// Pointer tables are re-sent only when the caller's pointers changed since the last call.
-void upload_dst(mxp_plan::Lowered& L, const mxp_plan& pl, void* const* dst_ptrs) {
+// Brings the plan's device pointer tables up to date, ordered on `stream` (the stream the
+// launch that reads them goes to).  The tables and the accumulators belong to the plan, so
+// launches of one plan are serialised: a call on another stream than the last one first waits
+// for that launch.  Tables are re-sent only when the caller's pointers changed, by copies that
+// `stream` orders behind whatever it still runs; the pinned block they come from is reused
+// only once the previous upload has left it.
+// A stream under capture records neither the waits nor the events of this protocol (they would
+// tie the plan's events to the graph): a captured launch is the caller's to order, and its
+// tables must already be on the device.
+bool is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &st) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return st != hipStreamCaptureStatusNone;
+}
+
+void upload_tables(mxp_plan::Lowered& L, const mxp_plan& pl, void* const* dst_ptrs, const void* const* file_ptrs,
+                   size_t n_files, hipStream_t stream) {
+  const bool capturing = is_capturing(stream);
+  if (!capturing && L.launch_rec && L.last_stream != stream) HIP_OK(hipStreamWaitEvent(stream, L.launch_done, 0));
   const size_t n = pl.params.size();
-  if (L.dst_host.size() == n && std::equal(L.dst_host.begin(), L.dst_host.end(), dst_ptrs)) return;
-  L.dst_bases.upload(dst_ptrs, n);
-  L.dst_host.assign(dst_ptrs, dst_ptrs + n);
+  const bool dst_changed = !(L.dst_host.size() == n && std::equal(L.dst_host.begin(), L.dst_host.end(), dst_ptrs));
+  const bool src_changed =
+      file_ptrs && !(L.src_host.size() == n_files && std::equal(L.src_host.begin(), L.src_host.end(), file_ptrs));
+  if (!dst_changed && !src_changed) return;
+  if (capturing)
+    throw Error(MXP_ERR_STATE, "the plan's pointer tables would change under stream capture: run the plan once "
+                               "outside the capture with these pointers first");
+  if (L.upload_rec) HIP_OK(hipEventSynchronize(L.upload_done));
+  if (dst_changed && n) {
+    std::memcpy(L.tab_host, dst_ptrs, n * sizeof(void*));
+    HIP_OK(hipMemcpyAsync(L.dst_bases.p, L.tab_host, n * sizeof(void*), hipMemcpyHostToDevice, stream));
+  }
+  if (src_changed && n_files) {
+    std::memcpy(L.tab_host + n, file_ptrs, n_files * sizeof(void*));
+    HIP_OK(hipMemcpyAsync(L.src_bases.p, L.tab_host + n, n_files * sizeof(void*), hipMemcpyHostToDevice, stream));
+  }
+  HIP_OK(hipEventRecord(L.upload_done, stream));
+  L.upload_rec = true;
+  if (dst_changed) L.dst_host.assign(dst_ptrs, dst_ptrs + n);
+  if (src_changed) L.src_host.assign(file_ptrs, file_ptrs + n_files);
+}
+void mark_launch(mxp_plan::Lowered& L, hipStream_t stream) {
+  if (is_capturing(stream)) return;
+  HIP_OK(hipEventRecord(L.launch_done, stream));
+  L.launch_rec = true;
+  L.last_stream = stream;
 }
 
 // Reads n bytes at off.  `need` (0 = n) is how many of them must exist: a range rounded up
@@ -576,6 +638,7 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     HIP_OK(hipEventCreate(&e->ev_b));
     HIP_OK(hipEventCreateWithFlags(&e->arena_busy, hipEventDisableTiming));
     HIP_OK(hipEventCreateWithFlags(&e->items_busy, hipEventDisableTiming));
+    HIP_OK(hipEventCreateWithFlags(&e->caller_ev, hipEventDisableTiming));
     e->static_dev = static_scratch_for(o.device);
     HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e->static_host), kStaticScratchBytes, hipHostMallocDefault));
     *out = e.release();
@@ -614,7 +677,7 @@ void ensure_ring(mxp_engine& e) {
   e.slot_ptrs.upload(ptrs.data(), ptrs.size());
 }
 
-void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_stats* stats) {
+void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t caller_stream, mxp_exec_stats* stats) {
   const double t_start = now_s();
   HIP_OK(hipSetDevice(e.opt.device));
   check_dst(pl, dst_ptrs);
@@ -639,8 +702,13 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
     if (fds[f] < 0) throw Error(MXP_ERR_IO, "cannot open " + ck.files[f].path + ": " + std::strerror(errno));
   }
 
-  // Everything below may change destination bytes.
-  upload_dst(L, pl, dst_ptrs);
+  // Everything below may change destination bytes.  The engine's streams are private and
+  // non-blocking: they first wait for what the caller already queued on its own stream
+  // (initialisation kernels on the parameters, reads of buffers the allocator has since
+  // handed back), as destination.copy_(source) on that stream would.
+  HIP_OK(hipEventRecord(e.caller_ev, caller_stream));
+  for (auto st : e.streams) HIP_OK(hipStreamWaitEvent(st, e.caller_ev, 0));
+  upload_tables(L, pl, dst_ptrs, nullptr, 0, e.streams[0]);
   HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, e.streams[0]));
   const bool digests = e.fused_digests;
   L.digests_valid = false;
@@ -746,6 +814,7 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, mxp_exec_sta
     stats->n_launches = n_chunks;
     stats->mutated = mutated.load();
   }
+  L.launch_rec = false;  // every stream is idle
   if (first_err) throw *first_err;
   if (sync_err != hipSuccess) throw Error(MXP_ERR_DEVICE, std::string("stream synchronize: ") + hipGetErrorString(sync_err));
   L.digests_valid = digests;
@@ -763,12 +832,7 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
   lower_plan(pl, e);
   auto& L = *pl.lowered;
   if (stats) std::memset(stats, 0, sizeof *stats);
-  // The pointer tables are small; plain synchronous copies keep them ordered before the launch.
-  upload_dst(L, pl, dst_ptrs);
-  if (L.src_host.size() != ck.files.size() || !std::equal(L.src_host.begin(), L.src_host.end(), file_dev_ptrs)) {
-    L.src_bases.upload(file_dev_ptrs, ck.files.size());
-    L.src_host.assign(file_dev_ptrs, file_dev_ptrs + ck.files.size());
-  }
+  upload_tables(L, pl, dst_ptrs, file_dev_ptrs, ck.files.size(), stream);
   HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, stream));
   L.digests_valid = e.fused_digests;
   if (e.fused_digests) HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(L.digest_sums.p), 10 * pl.params.size(), 0u, stream));
@@ -779,6 +843,7 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
   else
     HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
                         e.opt.nan_bits, stream));
+  mark_launch(L, stream);
   if (stats) {
     HIP_OK(hipEventRecord(e.ev_b, stream));
     HIP_OK(hipEventSynchronize(e.ev_b));
@@ -802,7 +867,15 @@ extern "C" {
 int mxp_execute(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs, mxp_exec_stats* stats) {
   return guard([&] {
     if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_execute: null handle");
-    do_execute(*engine, *plan, dst_ptrs, stats);
+    do_execute(*engine, *plan, dst_ptrs, nullptr, stats);
+  });
+}
+
+int mxp_execute_after(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs, void* caller_stream,
+                      mxp_exec_stats* stats) {
+  return guard([&] {
+    if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_execute_after: null handle");
+    do_execute(*engine, *plan, dst_ptrs, static_cast<hipStream_t>(caller_stream), stats);
   });
 }
 

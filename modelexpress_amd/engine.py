@@ -253,11 +253,17 @@ class PlacementEngine:
     def prepare(self, plan: PlacementPlan) -> None:
         L.check(L.lib().mxp_prepare(self._h, plan._h))
 
-    def execute(self, plan: PlacementPlan, dst: Sequence) -> dict:
-        """Ingest from storage into ``dst`` (torch tensors or raw device addresses)."""
+    def execute(self, plan: PlacementPlan, dst: Sequence, *, after_stream: int | None = None) -> dict:
+        """Ingest from storage into ``dst`` (torch tensors or raw device addresses).
+
+        The engine's streams first wait for what is already queued on ``after_stream`` (a raw
+        ``hipStream_t``; default: the calling thread's current torch stream), so pending work on
+        the destinations lands before the placed bytes, as it would ahead of ``copy_``."""
         ptrs = _ptr_array([_addr(t) for t in dst])
         stats = L.ExecStats()
-        rc = L.lib().mxp_execute(self._h, plan._h, ptrs, C.byref(stats))
+        if after_stream is None:
+            after_stream = _current_stream(self.device)
+        rc = L.lib().mxp_execute_after(self._h, plan._h, ptrs, C.c_void_p(after_stream), C.byref(stats))
         if rc < 0:
             err = L.MxpError(int(rc), L.lib().mxp_last_error().decode("utf-8", "replace"))
             err.mutated = bool(stats.mutated)
@@ -506,6 +512,15 @@ def digest_from_scalars(scalars: Sequence[int]) -> str:
     out = (C.c_uint8 * 16)()
     L.check(L.lib().mxp_digest_from_scalars(sc, out))
     return bytes(out).hex()
+
+
+def _current_stream(device: int) -> int:
+    """The raw handle of the calling thread's current torch stream on ``device`` (0 = the default stream)."""
+    import torch
+
+    if not torch.cuda.is_available():
+        return 0
+    return int(torch.cuda.current_stream(device).cuda_stream)
 
 
 def _addr(t) -> int:

@@ -11,6 +11,12 @@ strategy (model_streamer_strategy.py:38-107).  Same contract:
 * any other exception is logged, rolled back and the chain moves on;
 * no strategy left -> ``RuntimeError``.
 
+When the reference package can be imported, ``LoadStrategy``, ``LoadContext``, ``LoadResult``,
+``_as_load_result`` and ``register_tensors`` ARE the reference's (load_strategy/base.py,
+context.py), and ``StrategyFailed`` / ``EngineAdapter`` come from its adapter module (see
+``adapter.py``): the strategies below then subclass and raise exactly what the reference's own
+chain dispatches on.  Otherwise local mirrors with the same behaviour are used.
+
 ``HipPlacementStrategy`` takes the slot the reference gives ``ModelStreamerStrategy``
 (after InstantTensor, before GDS): same activation variable (``MX_MODEL_URI``), same URI
 resolution order, but the bytes go file -> pinned ring -> HBM -> placement kernels ->
@@ -55,67 +61,106 @@ def safetensors_dtype_of(t: torch.Tensor) -> str:
         raise ValueError(f"dtype {t.dtype} has no safetensors name") from exc
 
 
-@dataclass
-class LoadResult(Generic[T]):
-    """Stable envelope passed through strategies and adapter hooks (context.py:39-52)."""
+def _reference_load_strategy():
+    """(base module, context module) of the reference's load_strategy package, or None."""
+    from . import adapter as _adapter
 
-    value: T
-    model: nn.Module | None = None
-    publishable: bool = True
-    metadata: dict[str, Any] = field(default_factory=dict)
-
-
-@dataclass
-class SourceIdentity:
-    """The part of the reference's identity message the load path reads."""
-
-    model_name: str = ""
-
-
-@dataclass
-class LoadContext:
-    """Shared state passed to all loading strategies (context.py:55-87, load-path fields)."""
-
-    model_config: Any
-    load_config: Any = None
-    target_device: torch.device = field(default_factory=lambda: torch.device("cuda", 0))
-    global_rank: int = 0
-    worker_rank: int = 0
-    device_id: int = 0
-    identity: SourceIdentity = field(default_factory=SourceIdentity)
-    adapter: EngineAdapter | None = None
-    accelerator_backend: AcceleratorBackend = field(default_factory=HipAcceleratorBackend)
-    tensors: dict[str, torch.Tensor] = field(default_factory=dict)
-    source_ready_fn: Callable[[], bool] | None = None
-
-
-class LoadStrategy(ABC):
-    """Base class for weight-loading strategies (base.py:37-76)."""
-
-    name: str
-    requires: ClassVar[tuple] = ()
-
-    def is_available(self, ctx: LoadContext) -> bool:
-        if not self.requires:
-            return True
-        if ctx.adapter is None:
-            return False
-        cls = type(ctx.adapter)
-        return all(getattr(cls, m.__name__) is not m for m in self.requires)
-
-    @abstractmethod
-    def load(self, result: LoadResult, ctx: LoadContext) -> LoadResult:
-        """Attempt to load weights and return the updated result."""
-
-    def rollback(self, ctx: LoadContext) -> None:
-        """Clean up strategy-owned state after a failed load attempt."""
+    if not _adapter.BOUND_TO_REFERENCE:
         return None
+    try:
+        from modelexpress.load_strategy import base as ref_base
+    except Exception:  # noqa: BLE001 - the reference's own import-time requirements
+        return None
+    try:
+        from modelexpress.load_strategy import context as ref_ctx
+    except Exception:  # noqa: BLE001
+        ref_ctx = ref_base  # base re-exports both classes (base.py:19)
+    ok = hasattr(ref_base, "LoadStrategy") and hasattr(ref_ctx, "LoadContext") and hasattr(ref_ctx, "LoadResult")
+    return (ref_base, ref_ctx) if ok else None
 
 
-def _as_load_result(result_or_model) -> LoadResult:
-    if isinstance(result_or_model, LoadResult):
-        return result_or_model
-    return LoadResult(value=result_or_model, model=result_or_model)
+_ref = _reference_load_strategy()
+
+if _ref is not None:
+    LoadStrategy = _ref[0].LoadStrategy
+    LoadContext = _ref[1].LoadContext
+    LoadResult = _ref[1].LoadResult
+    _as_load_result = getattr(_ref[0], "_as_load_result", None)
+    # ModelStreamerStrategy registers the loaded tensors itself (model_streamer_strategy.py:96)
+    _register_tensors = getattr(_ref[0], "register_tensors", None)
+
+    @dataclass
+    class SourceIdentity:
+        """Stand-alone identity record for callers of this package's own chain."""
+
+        model_name: str = ""
+else:
+    _register_tensors = None
+    _as_load_result = None
+
+    @dataclass
+    class LoadResult(Generic[T]):
+        """Stable envelope passed through strategies and adapter hooks (context.py:39-52)."""
+
+        value: T
+        model: nn.Module | None = None
+        publishable: bool = True
+        metadata: dict[str, Any] = field(default_factory=dict)
+
+
+    @dataclass
+    class SourceIdentity:
+        """The part of the reference's identity message the load path reads."""
+
+        model_name: str = ""
+
+
+    @dataclass
+    class LoadContext:
+        """Shared state passed to all loading strategies (context.py:55-87, load-path fields)."""
+
+        model_config: Any
+        load_config: Any = None
+        target_device: torch.device = field(default_factory=lambda: torch.device("cuda", 0))
+        global_rank: int = 0
+        worker_rank: int = 0
+        device_id: int = 0
+        identity: SourceIdentity = field(default_factory=SourceIdentity)
+        adapter: EngineAdapter | None = None
+        accelerator_backend: AcceleratorBackend = field(default_factory=HipAcceleratorBackend)
+        tensors: dict[str, torch.Tensor] = field(default_factory=dict)
+        source_ready_fn: Callable[[], bool] | None = None
+
+
+    class LoadStrategy(ABC):
+        """Base class for weight-loading strategies (base.py:37-76)."""
+
+        name: str
+        requires: ClassVar[tuple] = ()
+
+        def is_available(self, ctx: LoadContext) -> bool:
+            if not self.requires:
+                return True
+            if ctx.adapter is None:
+                return False
+            cls = type(ctx.adapter)
+            return all(getattr(cls, m.__name__) is not m for m in self.requires)
+
+        @abstractmethod
+        def load(self, result: LoadResult, ctx: LoadContext) -> LoadResult:
+            """Attempt to load weights and return the updated result."""
+
+        def rollback(self, ctx: LoadContext) -> None:
+            """Clean up strategy-owned state after a failed load attempt."""
+            return None
+
+
+
+if _as_load_result is None:
+    def _as_load_result(result_or_model) -> LoadResult:
+        if isinstance(result_or_model, LoadResult):
+            return result_or_model
+        return LoadResult(value=result_or_model, model=result_or_model)
 
 
 def _resolve_model_uri(ctx: LoadContext) -> str:
@@ -150,6 +195,16 @@ def _engine_from_env(device: int):
         use_o_direct=envs.MXP_O_DIRECT, pack_strided_on_host=None if pack == "" else pack == "1")
 
 
+def _hip_placement_supported(backend) -> bool:
+    """The backend's own answer when it has one (``HipAcceleratorBackend``); for a backend that
+    predates the question (the reference's CUDA backend serves ROCm builds of torch too,
+    accelerators/cuda.py:49-50) the same check is made here."""
+    probe = getattr(backend, "supports_hip_placement", None)
+    if callable(probe):
+        return bool(probe())
+    return HipAcceleratorBackend().supports_hip_placement() and bool(getattr(torch.version, "hip", None))
+
+
 class HipPlacementStrategy(LoadStrategy):
     """Place weights with the HIP engine, straight into the engine's parameters."""
 
@@ -162,10 +217,14 @@ class HipPlacementStrategy(LoadStrategy):
         self._ckpt = None
 
     def is_available(self, ctx: LoadContext) -> bool:
-        if not super().is_available(ctx):
+        # Identity rule of base.py:53-60, tolerant of adapters that do not derive from the
+        # base class the capability was attached to: a missing method means "not overridden".
+        if ctx.adapter is None:
             return False
-        backend = ctx.accelerator_backend
-        if not getattr(backend, "supports_hip_placement", lambda: False)():
+        cls = type(ctx.adapter)
+        if not all(getattr(cls, m.__name__, m) is not m for m in self.requires):
+            return False
+        if not _hip_placement_supported(ctx.accelerator_backend):
             logger.info(f"[Worker {ctx.global_rank}] HIP placement library or device not available, skipping")
             return False
         model_uri = envs.MX_MODEL_URI or ""
@@ -227,10 +286,14 @@ class HipPlacementStrategy(LoadStrategy):
                                {p.name: (tuple(p.shape), p.dtype) for p in layout.params})
             logger.info(f"[Worker {ctx.global_rank}] HIP placement complete: "
                         f"{stats['placed_bytes'] / 1e9:.2f} GB in {stats['wall_seconds']:.3f}s")
-            result = ctx.adapter.after_placement(result)
+            after = getattr(ctx.adapter, "after_placement", None)
+            if callable(after):
+                result = after(result)
         except Exception as e:
             raise StrategyFailed(str(e), mutated=True) from e
         ctx.tensors.update({p.name: d for p, d in zip(layout.params, layout.destinations)})
+        if _register_tensors is not None:
+            _register_tensors(result, ctx)
         return result
 
     def rollback(self, ctx: LoadContext) -> None:

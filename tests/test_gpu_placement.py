@@ -142,6 +142,54 @@ def test_resident_placement_replays_from_a_hip_graph(gpu_engine, oracle, tmp_pat
     assert gpu_engine.checksums(plan)[idx] != eager_sums[idx]
 
 
+@pytest.mark.parametrize("side_stream", [False, True])
+def test_ingest_waits_for_work_already_queued_on_the_callers_stream(side_stream, gpu_engine, oracle, tmp_path):
+    """The engine writes from private streams.  Work the caller queued on its own stream before the call
+    (here: a long spin, then fills of every destination) must land BEFORE the placed bytes, as it
+    would ahead of ``destination.copy_(source)`` on that stream (installer.py:419-424)."""
+    layout, tp, ep, shards, ck_kw = tiny_layouts()["llama_tp4"]
+    synth.write_checkpoint(layout.checkpoint(), str(tmp_path), n_shards=shards, seed=41)
+    rv = layout.rank_view(tp_size=tp, tp_rank=1)
+    want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=1)
+    ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=1)
+    dst = gpu_engine.allocate(plan, fill=0)
+    gpu_engine.prepare(plan)
+    stream = torch.cuda.Stream() if side_stream else torch.cuda.current_stream()
+    with torch.cuda.stream(stream):
+        torch.cuda._sleep(100_000_000)  # a few hundred milliseconds of queued device time
+        for d in dst:
+            d.fill_(0xEE)
+        gpu_engine.execute(plan, dst)  # the calling thread's current stream is the one waited for
+    torch.cuda.synchronize()
+    for p, d, s in zip(plan.params, dst, gpu_engine.checksums(plan)):
+        assert d.cpu().numpy().tobytes() == want[p.name].tobytes(), p.name
+        assert s == oracle.safe_checksum(want[p.name]), p.name
+
+
+def test_resident_launches_of_one_plan_on_two_streams_do_not_share_tables(gpu_engine, oracle, tmp_path):
+    """Double-buffered use: the same plan launched asynchronously into buffer set A on one stream and,
+    right away, into set B on another.  The second call rewrites the plan's pointer tables; the first
+    launch must still land wholly in A."""
+    layout, tp, ep, shards, ck_kw = tiny_layouts()["llama_tp4"]
+    synth.write_checkpoint(layout.checkpoint(), str(tmp_path), n_shards=shards, seed=42)
+    rv = layout.rank_view(tp_size=tp, tp_rank=3)
+    want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=3)
+    ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=3)
+    staged = _stage_files(ck)
+    sets = [gpu_engine.allocate(plan, fill=0x5A + k) for k in range(4)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    with torch.cuda.stream(streams[0]):
+        torch.cuda._sleep(50_000_000)  # keeps the first launch pending while the second call runs on the host
+    for k, dst in enumerate(sets):
+        gpu_engine.execute_resident(plan, staged, dst, stream=streams[k % 2].cuda_stream)
+    torch.cuda.synchronize()
+    for k, dst in enumerate(sets):
+        for p, d in zip(plan.params, dst):
+            assert d.cpu().numpy().tobytes() == want[p.name].tobytes(), (k, p.name)
+    assert gpu_engine.checksums(plan) == [oracle.safe_checksum(want[p.name]) for p in plan.params]
+
+
 def test_empty_and_scalar_tensors(gpu_engine, gpu_engine_band, oracle, tmp_path, mxp):
     """Zero-element tensors, 0-dim tensors and odd byte counts through the whole path."""
     from safetensors.torch import save_file

@@ -124,11 +124,11 @@ def test_truncated_shard_fails_the_strategy_and_the_chain_recovers(tmp_path, mon
     monkeypatch.setenv("MXP_SLOT_MIB", "1")
     real_execute = E.PlacementEngine.execute
 
-    def execute_after_truncation(eng, plan, dst):
+    def execute_after_truncation(eng, plan, dst, **kw):
         size = os.path.getsize(info["files"][-1])
         with open(info["files"][-1], "r+b") as f:
             f.truncate(size // 2)
-        return real_execute(eng, plan, dst)
+        return real_execute(eng, plan, dst, **kw)
 
     monkeypatch.setattr(E.PlacementEngine, "execute", execute_after_truncation)
     model = ToyModel(rv)
