@@ -133,31 +133,53 @@ static void parse_file(mxp_ckpt& ck, const std::string& path, const std::vector<
       if (d.type != Json::Int || d.i < 0)
         throw Error(MXP_ERR_FORMAT, path + ": bad shape for tensor '" + kv.first + "'");
       t.shape.push_back(d.i);
-      numel *= (uint64_t)d.i;
+      // a product that wraps must not pass for a small tensor
+      if (__builtin_mul_overflow(numel, (uint64_t)d.i, &numel))
+        throw Error(MXP_ERR_FORMAT, path + ": the shape of tensor '" + kv.first + "' overflows 64 bits");
     }
     const int64_t b = jo->arr[0].i, e = jo->arr[1].i;
     if (b < 0 || e < b) throw Error(MXP_ERR_FORMAT, path + ": bad data_offsets for '" + kv.first + "'");
     t.file_index = file_index;
     t.file_offset = data_start + (uint64_t)b;
     t.nbytes = (uint64_t)(e - b);
-    if (t.nbytes != numel * (uint64_t)dtype_size(t.dtype))
+    uint64_t need_bytes = 0;
+    if (__builtin_mul_overflow(numel, (uint64_t)dtype_size(t.dtype), &need_bytes))
+      throw Error(MXP_ERR_FORMAT, path + ": the size of tensor '" + kv.first + "' overflows 64 bits");
+    if (t.nbytes != need_bytes)
       throw Error(MXP_ERR_FORMAT, path + ": tensor '" + kv.first + "' has " + std::to_string(t.nbytes) +
-                                      " bytes but its shape and dtype need " +
-                                      std::to_string(numel * (uint64_t)dtype_size(t.dtype)));
+                                      " bytes but its shape and dtype need " + std::to_string(need_bytes));
     if (t.file_offset + t.nbytes > file_size)
       throw Error(MXP_ERR_IO, path + ": tensor '" + kv.first + "' extends past the end of the file");
     recs.push_back(std::move(t));
   }
-  if (wanted) {
-    std::unordered_map<std::string, int> want;
-    for (const auto& w : *wanted) want.emplace(w, 1);
-    std::vector<TensorRec> keep;
-    for (auto& r : recs)
-      if (want.count(r.name)) keep.push_back(std::move(r));
-    recs.swap(keep);
-  }
   std::stable_sort(recs.begin(), recs.end(),
                    [](const TensorRec& a, const TensorRec& b) { return a.file_offset < b.file_offset; });
+  // Two tensors may not share bytes (the format lays them out back to back); empty ones have none.
+  {
+    const TensorRec* prev = nullptr;
+    for (const auto& r : recs) {
+      if (r.nbytes == 0) continue;
+      if (prev && r.file_offset < prev->file_offset + prev->nbytes)
+        throw Error(MXP_ERR_FORMAT, path + ": tensors '" + prev->name + "' and '" + r.name + "' overlap in the file");
+      prev = &r;
+    }
+  }
+  if (wanted) {
+    // Every name the index assigns to this shard must be in its header: the reference's per-file
+    // loop looks each one up and fails on a missing key (gds_loader.py:297-313).
+    std::unordered_map<std::string, int> want;
+    for (const auto& w : *wanted) want.emplace(w, 0);
+    std::vector<TensorRec> keep;
+    for (auto& r : recs) {
+      auto it = want.find(r.name);
+      if (it == want.end()) continue;
+      it->second = 1;
+      keep.push_back(std::move(r));
+    }
+    for (const auto& w : *wanted)
+      if (!want[w]) throw Error(MXP_ERR_FORMAT, "tensor '" + w + "' is assigned to " + path + " by the index but is not in its header");
+    recs.swap(keep);
+  }
   FileRec fr;
   fr.path = path;
   fr.size = file_size;

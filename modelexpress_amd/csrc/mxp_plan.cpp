@@ -656,9 +656,11 @@ int64_t mxp_plan_add_param(mxp_plan* plan, const char* name, int32_t dtype, int3
     for (int d = 0; d < ndim; ++d) {
       if (shape[d] < 0) throw Error(MXP_ERR_ARG, "negative dimension");
       p.shape.push_back(shape[d]);
-      n *= (uint64_t)shape[d];
+      if (__builtin_mul_overflow(n, (uint64_t)shape[d], &n)) throw Error(MXP_ERR_ARG, std::string("the shape of parameter ") + name + " overflows 64 bits");
     }
-    p.nbytes = n * (uint64_t)dtype_size(dtype);
+    // below 2^62 bytes every product of a subset of the extents with the element size fits a signed 64-bit value too
+    if (__builtin_mul_overflow(n, (uint64_t)dtype_size(dtype), &p.nbytes) || p.nbytes >= (1ull << 62))
+      throw Error(MXP_ERR_ARG, std::string("the size of parameter ") + name + " overflows");
     idx = (int64_t)plan->params.size();
     plan->param_by_name.emplace(p.name, idx);
     plan->params.push_back(std::move(p));

@@ -74,3 +74,67 @@ def test_truncations_and_bit_flips_of_a_good_file(tmp_path, cut, flip, bit):
     blob[flip % len(blob)] ^= 1 << bit
     p.write_bytes(bytes(blob[: max(0, len(blob) - cut)]))
     _check(p)
+
+
+def _write(path, header: dict, blob: int):
+    raw = json.dumps(header).encode()
+    path.write_bytes(struct.pack("<Q", len(raw)) + raw + bytes(blob))
+
+
+def test_shape_products_that_wrap_are_rejected(tmp_path):
+    """[2^32, 2^32] multiplies to 0 mod 2^64: it must not pass for an empty tensor."""
+    p = tmp_path / "model.safetensors"
+    _write(p, {"w": {"dtype": "U8", "shape": [1 << 32, 1 << 32], "data_offsets": [0, 0]}}, 16)
+    with pytest.raises(MxpError) as e:
+        Checkpoint(str(p))
+    assert e.value.code == ERR_FORMAT and "overflows" in e.value.message
+    _write(p, {"w": {"dtype": "F64", "shape": [1 << 61], "data_offsets": [0, 0]}}, 16)  # numel fits, bytes do not
+    with pytest.raises(MxpError) as e:
+        Checkpoint(str(p))
+    assert e.value.code == ERR_FORMAT and "overflows" in e.value.message
+
+
+def test_parameter_sizes_that_wrap_are_rejected(tmp_path):
+    from modelexpress_amd._lib import ERR_ARG
+    from modelexpress_amd.engine import PlacementPlan
+
+    p = tmp_path / "model.safetensors"
+    _write(p, {"w": {"dtype": "U8", "shape": [4], "data_offsets": [0, 4]}}, 4)
+    with Checkpoint(str(p)) as ck:
+        for shape in ((1 << 32, 1 << 32), (1 << 62,)):
+            with pytest.raises(MxpError) as e:
+                PlacementPlan(ck, [_Spec("w", "U8", shape)])
+            assert e.value.code == ERR_ARG and "overflows" in e.value.message
+
+
+class _Spec:
+    """A parameter row whose byte count Python does not pre-compute."""
+
+    def __init__(self, name, dtype, shape):
+        self.name, self.dtype, self.shape = name, dtype, shape
+
+
+def test_overlapping_tensors_are_rejected(tmp_path):
+    p = tmp_path / "model.safetensors"
+    _write(p, {"a": {"dtype": "U8", "shape": [8], "data_offsets": [0, 8]},
+               "b": {"dtype": "U8", "shape": [8], "data_offsets": [4, 12]}}, 12)
+    with pytest.raises(MxpError) as e:
+        Checkpoint(str(p))
+    assert e.value.code == ERR_FORMAT and "overlap" in e.value.message
+    # empty tensors share an offset with their neighbour without sharing bytes
+    _write(p, {"a": {"dtype": "U8", "shape": [8], "data_offsets": [0, 8]},
+               "e": {"dtype": "F32", "shape": [0, 4], "data_offsets": [4, 4]},
+               "b": {"dtype": "U8", "shape": [4], "data_offsets": [8, 12]}}, 12)
+    with Checkpoint(str(p)) as ck:
+        assert len(ck) == 3
+
+
+def test_index_names_missing_from_their_shard_fail_the_open(tmp_path):
+    """gds_loader.py:297-313 looks every indexed name up in its shard's header: a missing one is an
+    error there (KeyError), not a silently shorter checkpoint."""
+    _write(tmp_path / "s0.safetensors", {"a": {"dtype": "U8", "shape": [4], "data_offsets": [0, 4]}}, 4)
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(
+        {"weight_map": {"a": "s0.safetensors", "ghost": "s0.safetensors"}}))
+    with pytest.raises(MxpError) as e:
+        Checkpoint(str(tmp_path))
+    assert e.value.code == ERR_FORMAT and "ghost" in e.value.message
