@@ -19,7 +19,7 @@ from pathlib import Path
 HEADER = Path(__file__).with_name("mxp.h")
 
 SCALARS = {"int": "c_int", "int32_t": "i32", "int64_t": "i64", "uint8_t": "u8", "uint16_t": "u16", "uint32_t": "u32",
-           "uint64_t": "u64", "double": "f64", "char": "c_char", "void": "c_void", "size_t": "usize"}
+           "uint64_t": "u64", "double": "f64", "float": "f32", "char": "c_char", "void": "c_void", "size_t": "usize"}
 
 
 def strip_comments(text: str) -> str:

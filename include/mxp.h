@@ -292,6 +292,15 @@ int mxp_execute_after(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs,
 int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* file_dev_ptrs,
                          void* const* dst_ptrs, void* stream, mxp_exec_stats* stats);
 
+/* Launch timing for measurements.  Switched on, every asynchronous mxp_execute_resident (stats ==
+ * NULL) records a HIP-event pair around its placement kernel on the launch stream and does NOT
+ * synchronise, so a timed loop of K launches yields both its wall time and the K kernel
+ * durations.  mxp_engine_launch_times waits for the launches and writes the durations (ms) of the
+ * most recent min(capacity, recorded, 256) of them, oldest first.  Switching on or off restarts
+ * the count.  No counterpart in the reference. */
+int mxp_engine_set_launch_timing(mxp_engine* engine, int32_t on);
+int mxp_engine_launch_times(mxp_engine* engine, float* out_ms, int32_t capacity, int32_t* n_out);
+
 /* Checksums accumulated by the last execute, one per parameter (tensor_utils.py:27-44
  * over the parameter's row-major bytes).  Synchronises the engine first. */
 int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_t n);

@@ -145,6 +145,8 @@ SIGNATURES = {
     "mxp_execute": (C.c_int, [_P, _P, _PP, C.POINTER(ExecStats)]),
     "mxp_execute_after": (C.c_int, [_P, _P, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_execute_resident": (C.c_int, [_P, _P, _PP, _PP, _P, C.POINTER(ExecStats)]),
+    "mxp_engine_set_launch_timing": (C.c_int, [_P, C.c_int32]),
+    "mxp_engine_launch_times": (C.c_int, [_P, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
     "mxp_plan_checksums": (C.c_int, [_P, _P, _U32P, C.c_int64]),
     "mxp_checksum32": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_checksum32_static": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),

@@ -186,11 +186,17 @@ struct mxp_engine {
   DevBuf<TransposeItem> items_dev;
   hipEvent_t items_busy = nullptr;
   bool items_recorded = false;
+  // launch timing (mxp_engine_set_launch_timing): event pairs around the placement kernel of the
+  // last kTimingRing resident launches, recorded without synchronising
+  std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_ring;
+  bool timing_on = false;
+  uint64_t timing_count = 0;
   // mxp_checksum32_static: this GPU's scratch array and a pinned mirror of it, both set up at create
   unsigned char* static_dev = nullptr;
   unsigned char* static_host = nullptr;  // pinned
 
   ~mxp_engine() {
+    for (auto& pr : timing_ring) { (void)hipEventDestroy(pr.first); (void)hipEventDestroy(pr.second); }
     if (static_host) (void)hipHostFree(static_host);
     if (arena_busy) (void)hipEventDestroy(arena_busy);
     if (caller_ev) (void)hipEventDestroy(caller_ev);
@@ -388,7 +394,15 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
           }
         }
         uint64_t lead = 0, need = 0;
-        if (L->direct_io) {
+        if (L->direct_io && p.rows > 1) {
+          // packed rows: each row is read as whole blocks into the reader's own buffer and only
+          // its bytes are copied into the slot, so the slot layout is that of buffered packing
+          for (uint64_t r = 0; r < p.rows; ++r) {
+            const uint64_t o0 = p.file_off + r * p.file_pitch;
+            L->file_bytes += align_up(o0 + p.nbytes, blk) - o0 / blk * blk;
+          }
+          L->file_bytes -= p.nbytes * p.rows;  // added back below with the slot bytes
+        } else if (L->direct_io) {
           const uint64_t a0 = p.file_off / blk * blk, a1 = align_up(p.file_off + p.nbytes, blk);
           lead = p.file_off - a0;
           need = lead + p.nbytes;
@@ -613,12 +627,12 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     if (o.streams <= 0) o.streams = 4;
     if (o.tile_bytes == 0) o.tile_bytes = kPlaceThreads * kPlaceBatch * 16;
     if (o.nan_bits == 0) o.nan_bits = 0x7FC0;
-    // Packing strided rows on the host issues one read per row: right for the page cache,
-    // wrong for direct I/O, where whole row bands are staged and gathered on the device.
+    // Packing strided rows on the host issues one read per row: right for the page cache.  Under
+    // direct I/O every row read is widened to whole 4 KiB blocks, so whole row bands staged and
+    // gathered on the device are the default there; packing stays available (it reads less when
+    // rows are far apart: 4 KiB per 1 KiB row of an 8 KiB pitch instead of 8 KiB).
     if (o.pack_strided_on_host == 0) o.pack_strided_on_host = o.use_o_direct ? 2 : 1;
     if (o.pack_strided_on_host > 2) throw Error(MXP_ERR_ARG, "pack_strided_on_host must be 0, 1 or 2");
-    if (o.use_o_direct && o.pack_strided_on_host == 1)
-      throw Error(MXP_ERR_ARG, "direct I/O reads whole blocks; it cannot be combined with per-row host packing");
     if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
     if (o.tile_bytes < 1024 || o.tile_bytes > (uint32_t)(kPlaceThreads * kPlaceBatch * 16))
       throw Error(MXP_ERR_ARG, "tile_bytes must be in [1 KiB, 128 KiB]");
@@ -753,7 +767,13 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
         for (const auto& r : ch.ranges)
           for (uint64_t row = 0; row < r.rows; ++row) {
             uint8_t* into = sl.host + r.slot_off + row * r.nbytes;
-            if (direct_buf) {
+            if (direct_buf && r.rows > 1) {
+              const uint64_t o0 = r.file_off + row * r.file_pitch, a0 = o0 / 4096 * 4096;
+              const uint64_t a1 = align_up(o0 + r.nbytes, 4096);
+              pread_full(fds[r.file], static_cast<uint8_t*>(direct_buf), a1 - a0, a0, ck.files[r.file].path,
+                         o0 - a0 + r.nbytes);
+              std::memcpy(into, static_cast<uint8_t*>(direct_buf) + (o0 - a0), r.nbytes);
+            } else if (direct_buf) {
               pread_full(fds[r.file], static_cast<uint8_t*>(direct_buf), r.nbytes, r.file_off + row * r.file_pitch,
                          ck.files[r.file].path, r.need);
               std::memcpy(into, direct_buf, r.need ? r.need : r.nbytes);
@@ -836,13 +856,20 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
   HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, stream));
   L.digests_valid = e.fused_digests;
   if (e.fused_digests) HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(L.digest_sums.p), 10 * pl.params.size(), 0u, stream));
+  const bool ring_timed = e.timing_on && !stats && !is_capturing(stream);
+  const auto& pair = e.timing_ring.empty() ? std::pair<hipEvent_t, hipEvent_t>() : e.timing_ring[e.timing_count % e.timing_ring.size()];
   if (stats) HIP_OK(hipEventRecord(e.ev_a, stream));
+  if (ring_timed) HIP_OK(hipEventRecord(pair.first, stream));
   if (e.fused_digests)
     HIP_OK(launch_place_digest(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
                                L.dst_sizes.p, L.digest_sums.p, e.opt.nan_bits, stream));
   else
     HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
                         e.opt.nan_bits, stream));
+  if (ring_timed) {
+    HIP_OK(hipEventRecord(pair.second, stream));
+    ++e.timing_count;
+  }
   mark_launch(L, stream);
   if (stats) {
     HIP_OK(hipEventRecord(e.ev_b, stream));
@@ -910,6 +937,41 @@ int mxp_engine_set_fused_digests(mxp_engine* engine, int32_t on) {
   return guard([&] {
     if (!engine) throw Error(MXP_ERR_ARG, "mxp_engine_set_fused_digests: null engine");
     engine->fused_digests = on != 0;
+  });
+}
+
+int mxp_engine_set_launch_timing(mxp_engine* engine, int32_t on) {
+  return guard([&] {
+    if (!engine) throw Error(MXP_ERR_ARG, "mxp_engine_set_launch_timing: null engine");
+    constexpr size_t kTimingRing = 256;
+    HIP_OK(hipSetDevice(engine->opt.device));
+    if (on && engine->timing_ring.empty()) {
+      engine->timing_ring.reserve(kTimingRing);
+      for (size_t k = 0; k < kTimingRing; ++k) {
+        hipEvent_t a = nullptr, b = nullptr;
+        HIP_OK(hipEventCreate(&a));
+        if (hipEventCreate(&b) != hipSuccess) { (void)hipEventDestroy(a); throw Error(MXP_ERR_DEVICE, "hipEventCreate failed"); }
+        engine->timing_ring.emplace_back(a, b);
+      }
+    }
+    engine->timing_on = on != 0;
+    engine->timing_count = 0;
+  });
+}
+
+int mxp_engine_launch_times(mxp_engine* engine, float* out_ms, int32_t capacity, int32_t* n_out) {
+  return guard([&] {
+    if (!engine || !n_out || capacity < 0 || (capacity && !out_ms)) throw Error(MXP_ERR_ARG, "mxp_engine_launch_times: bad argument");
+    mxp_engine& e = *engine;
+    HIP_OK(hipSetDevice(e.opt.device));
+    const uint64_t have = std::min<uint64_t>(e.timing_count, e.timing_ring.size());
+    const uint64_t n = std::min<uint64_t>(have, (uint64_t)capacity);
+    for (uint64_t k = 0; k < n; ++k) {
+      const auto& pr = e.timing_ring[(e.timing_count - n + k) % e.timing_ring.size()];
+      HIP_OK(hipEventSynchronize(pr.second));
+      HIP_OK(hipEventElapsedTime(&out_ms[k], pr.first, pr.second));
+    }
+    *n_out = (int32_t)n;
   });
 }
 

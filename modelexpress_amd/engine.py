@@ -280,6 +280,17 @@ class PlacementEngine:
                                              C.byref(stats) if timed else None))
         return stats.as_dict() if timed else None
 
+    def set_launch_timing(self, on: bool = True) -> None:
+        """Asynchronous resident launches record an event pair around their placement kernel (no synchronisation)."""
+        L.check(L.lib().mxp_engine_set_launch_timing(self._h, 1 if on else 0))
+
+    def launch_times(self, n: int = 256) -> list[float]:
+        """Kernel durations (ms) of the most recent ``n`` timed resident launches, oldest first; waits for them."""
+        out = (C.c_float * max(1, n))()
+        got = C.c_int32()
+        L.check(L.lib().mxp_engine_launch_times(self._h, out, n, C.byref(got)))
+        return [float(out[i]) for i in range(got.value)]
+
     def set_fused_digests(self, on: bool = True) -> None:
         """Placements also accumulate the ``tensor_digest`` sums of every parameter inside the placement kernel."""
         L.check(L.lib().mxp_engine_set_fused_digests(self._h, 1 if on else 0))

@@ -112,8 +112,12 @@ def run_faithful_sample(ckpt_dir: str, names: list, tp_size: int, tp_rank: int, 
     flattened tensor (the 1-D case, the only one in which the reference returns a value).
     Returns bytes processed and seconds; used only to report how the literal formulation
     compares with the one-pass C form."""
+    import warnings
+
     import torch
 
+    # the memory-mapped checkpoint is read-only and only ever read here
+    warnings.filterwarnings("ignore", message="The given NumPy array is not writable")
     torch.set_num_threads(threads)
     weights = dict(O.load_checkpoint(ckpt_dir, mmap=True))
     placed = 0

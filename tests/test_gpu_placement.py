@@ -55,15 +55,17 @@ def test_direct_io_ranges_match_oracle(name, oracle, tmp_path, mxp):
     rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=tp_rank % ep, param_dtype=param_dtype)
     want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
     ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
-    eng = PlacementEngine(0, ring_slots=3, slot_bytes=1 << 17, reader_threads=2, streams=2, use_o_direct=True)
-    dst = eng.allocate(plan, fill=0x11)
-    eng.execute(plan, dst)
-    for p, d, s in zip(plan.params, dst, eng.checksums(plan)):
-        assert d.cpu().numpy().tobytes() == want[p.name].tobytes(), p.name
-        assert s == oracle.safe_checksum(want[p.name]), p.name
-    with pytest.raises(mxp.MxpError, match="direct I/O"):
-        PlacementEngine(0, use_o_direct=True, pack_strided_on_host=True)
-    eng.close()
+    # default under direct I/O: whole row bands, gathered on the device; then strided rows packed by the readers
+    for pack in (None, True):
+        eng = PlacementEngine(0, ring_slots=3, slot_bytes=1 << 17, reader_threads=2, streams=2, use_o_direct=True,
+                              pack_strided_on_host=pack)
+        dst = eng.allocate(plan, fill=0x11)
+        stats = eng.execute(plan, dst)
+        for p, d, s in zip(plan.params, dst, eng.checksums(plan)):
+            assert d.cpu().numpy().tobytes() == want[p.name].tobytes(), (pack, p.name)
+            assert s == oracle.safe_checksum(want[p.name]), (pack, p.name)
+        assert stats["file_bytes"] >= stats["placed_bytes"]  # whole blocks are read
+        eng.close()
 
 
 def test_megatron_interleaved_qkv_refit_on_device(gpu_engine, gpu_engine_band, oracle, tmp_path, mxp):
