@@ -149,6 +149,39 @@ def _timed_resident(eng, plan, staged, dst, steps: int, warmup: int) -> dict:
     return {"wall_s": wall, "ms_per_step": wall / steps * 1e3, "kernel_ms": k_ms}
 
 
+def _segment_classes(eng, ck, plan, rv, staged, dst, tp, rank, cast, steps, warmup) -> dict:
+    """Sub-plans over the parameters of one kind each (the other tensors are skipped), launched and timed
+    like the whole step.  A class is named after the parameter it writes; its writes share one shape."""
+    from modelexpress_amd.engine import PlacementPlan
+
+    def kind(name: str) -> str:
+        for key in ("qkv_proj", "o_proj", "gate_up_proj", "down_proj", "embed_tokens", "lm_head", "w13", "w2", "wte", "wpe"):
+            if key in name:
+                return key
+        return "other (norms, biases, scales, small matrices)"
+
+    groups: dict = {}
+    for i, p in enumerate(rv.params):
+        groups.setdefault(kind(p.name), []).append(i)
+    res = {}
+    for label, idx in groups.items():
+        sub = PlacementPlan(ck, [rv.params[i] for i in idx], tp_size=tp, tp_rank=rank,
+                            stacked_params_mapping=rv.stacked_params_mapping, expert_mapping=rv.expert_mapping,
+                            allow_cast=cast, allow_unmapped=True)
+        writes = sub.writes()
+        totals = sub.totals()
+        t = _timed_resident(eng, sub, staged, [dst[i] for i in idx], steps, warmup)
+        k = sum(t["kernel_ms"]) / len(t["kernel_ms"])
+        w0 = writes[0]
+        res[label] = {"buffers": len(idx), "writes": len(writes), "placed_bytes": totals["placed_bytes"],
+                      "typical_write": {"rows": w0.rows, "row_bytes": w0.row_bytes, "src_pitch": w0.src_pitch, "dst_pitch": w0.dst_pitch},
+                      "kernel_ms_avg": round(k, 4), "kernel_ms_min": round(min(t["kernel_ms"]), 4),
+                      "gbps_algorithmic": round(totals["kernel_algorithmic_bytes"] / (k * 1e-3) / 1e9, 1),
+                      "frac_of_hbm_peak": round(totals["kernel_algorithmic_bytes"] / (k * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)}
+        sub.close()
+    return res
+
+
 def _fs_type(path: str) -> str:
     """File-system type of the mount that holds ``path`` (longest matching mount point)."""
     best, kind = "", "unknown"
@@ -243,6 +276,9 @@ def main() -> int:
                          "bypassing the page cache")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run one plain 1 GiB device copy (a kernel of known traffic, for scaling profiler counters)")
+    ap.add_argument("--classes", action="store_true",
+                    help="also time each class of segments of the workload as a launch of its own (contiguous row "
+                         "blocks, strided column slices, vocabulary slices ...): the breakdown of the step time")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the block of the other four configurations that the default run appends")
     ap.add_argument("--seed", type=int, default=20240229)
@@ -329,6 +365,10 @@ def main() -> int:
                                 "step; the end-to-end rate from files (PCIe-bound) is roofline.e2e"},
             "roofline": roofline,
         }
+
+        # ---- the step broken down by class of segment, each class a launch of its own ----
+        if args.classes:
+            out["segment_classes"] = _segment_classes(eng, ck, plan, rv, staged, dst, tp, rank, cast, args.steps, args.warmup)
 
         # ---- the read-only operators over the finished buffers (1 x bytes each) ----
         sizes = [p.nbytes for p in plan.params]

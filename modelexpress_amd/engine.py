@@ -223,6 +223,7 @@ class PlacementEngine:
         self._h = C.c_void_p()
         L.check(L.lib().mxp_engine_create(C.byref(opts), C.byref(self._h)))
         self.device = device
+        self.nan_bits = nan_bits or 0x7FC0  # the bf16 image this engine gives every fp32 / fp16 NaN
 
     def close(self) -> None:
         if self._h:

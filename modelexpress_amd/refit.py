@@ -22,6 +22,7 @@ that waives the "untouched until verified" guarantee and is therefore explicit.
 
 from __future__ import annotations
 
+import contextlib
 import json
 import logging
 from dataclasses import dataclass, field
@@ -76,9 +77,6 @@ class StagedWeights:
     digests: list
     stats: dict
     in_place: bool
-
-
-import contextlib
 
 
 def _null():
@@ -169,6 +167,9 @@ class HipRefitAdapter:
         lay = self.layout
         self.timing = RefitTimingRecorder(backend="hip_placement", version=inputs.version_id, tp_rank=lay.tp_rank,
                                           tp_size=lay.tp_size, cold=self._plans_built == 0)
+        # the NaN image of the casts is platform-defined upstream (torch's device kernels give 0x7FC0, its
+        # AVX-512 CPU kernels 0xFFFF): the record says which one this cycle wrote
+        self.timing.extra["cast_nan_bits"] = f"0x{self.engine.nan_bits:04x}"
         with self.timing.span("transfer_planning"):
             ck = Checkpoint(inputs.checkpoint_path)
             plan = PlacementPlan(ck, lay.params, tp_size=lay.tp_size, tp_rank=lay.tp_rank,

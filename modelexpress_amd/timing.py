@@ -32,6 +32,7 @@ class RefitTimingRecorder:
                  cold: bool | None = None, clock=time.perf_counter):
         self.backend, self.version, self.tp_rank, self.tp_size, self.cold = backend, version, tp_rank, tp_size, cold
         self.bytes = 0
+        self.extra: dict[str, Any] = {}  # further facts of the cycle, emitted with the record
         self._clock = clock
         self._started = clock()
         self._stages = {s: {"duration_s": 0.0, "count": 0, "statuses": []} for s in REFIT_TIMING_STAGES}
@@ -65,7 +66,7 @@ class RefitTimingRecorder:
         return {
             "backend": self.backend, "version": self.version, "tp_rank": self.tp_rank, "tp_size": self.tp_size,
             "cold_warm": None if self.cold is None else ("cold" if self.cold else "warm"), "bytes": self.bytes,
-            "total_s": round(total, 6),
+            "total_s": round(total, 6), **self.extra,
             "stages": {s: {"duration_s": round(v["duration_s"], 6), "count": v["count"], "statuses": v["statuses"]}
                        for s, v in self._stages.items() if v["count"]},
         }

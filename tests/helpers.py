@@ -9,11 +9,15 @@ from modelexpress_amd import models
 from modelexpress_amd.engine import Checkpoint, PlacementPlan
 
 
-def oracle_place(oracle, ckpt_dir: str, rv, *, tp_size=1, tp_rank=0, allow_cast=False, nan_bits=0x7FC0,
-                 strict_params=True):
-    """The oracle's parameter buffers for one rank: ``{name: OTensor}``."""
-    weights = oracle.load_checkpoint(ckpt_dir)
-    params = {p.name: oracle.OTensor.zeros(p.shape, p.dtype) for p in rv.params}
+def oracle_place(oracle, ckpt_dir: str | None, rv, *, tp_size=1, tp_rank=0, allow_cast=False, nan_bits=0x7FC0,
+                 strict_params=True, weights=None, only_params=None):
+    """The oracle's parameter buffers for one rank: ``{name: OTensor}``.  ``weights`` (a list of
+    ``(name, OTensor)``) stands in for the checkpoint directory; ``only_params`` restricts the rank's
+    parameter table to those names (the weights given must then be the ones that write into them)."""
+    if weights is None:
+        weights = oracle.load_checkpoint(ckpt_dir)
+    wanted = [p for p in rv.params if only_params is None or p.name in only_params]
+    params = {p.name: oracle.OTensor.zeros(p.shape, p.dtype) for p in wanted}
     skip = tuple(rv.skip_prefixes)
     weights = [(n, t) for n, t in weights if not n.startswith(skip)] if skip else weights
     local_of = {}

@@ -1,5 +1,8 @@
-"""Full-size checks (benchmark configuration 2: Llama-3-8B, one TP=8 rank slice, 16 GB
-staged in HBM) through properties that do not need the oracle to process 16 GB:
+"""Full-size checks of the benchmark configurations (2: Llama-3-8B, one TP=8 rank slice, 16 GB staged
+in HBM; 3: the same rank refitted from a 32 GB fp32 checkpoint with the real 1e-6 edge-case density;
+4: one Mixtral-8x7B layer's expert stack at its real shapes; 5: the dense and MoE layers of a
+DeepSeek-V3 rank share at their real shapes, fp8 weights with their 128x128 scale tiles) through
+properties that do not need the oracle to process the whole checkpoint:
 
 * the checkpoint is generated on the device by the seeded generator, which produces the
   same bytes as the host generator, so any single tensor can be regenerated on the host
@@ -80,6 +83,131 @@ def test_llama3_8b_rank_slice_full_size(oracle, oracle_c, tmp_path, mxp):
     eng.execute_resident(plan, staged, dst)
     assert eng.checksums(plan) == fused
     assert all(torch.equal(a, b) for a, b in zip(before, dst[:8]))
+    eng.close()
+
+
+def _check_params_against_oracle(oracle, oracle_c, plan, rv, dst, fused, by_name, names, *, tp, rank, cast=False):
+    """Regenerates on the host every checkpoint tensor that writes into the parameters ``names``, runs the
+    oracle's loader over them (slice, fuse, stack, cast) and compares bytes and checksums.  Returns the
+    regenerated source tensors ``{name: uint8 array of shape + (element size,)}``."""
+    from helpers import oracle_place
+
+    sources = sorted({w.tensor for w in plan.writes() if w.param in names})
+    host = {n: _host_tensor(by_name[n], SEED) for n in sources}
+    weights = [(n, oracle.OTensor(host[n], by_name[n].dtype)) for n in sources]
+    want = oracle_place(oracle, None, rv, tp_size=tp, tp_rank=rank, allow_cast=cast, weights=weights, only_params=set(names))
+    idx = {p.name: i for i, p in enumerate(plan.params)}
+    for name in names:
+        got = dst[idx[name]].cpu().numpy()
+        assert got.tobytes() == want[name].tobytes(), name
+        assert fused[idx[name]] == oracle_c.checksum32(np.frombuffer(want[name].tobytes(), dtype=np.uint8)), name
+    return host
+
+
+def _all_checksums_alone(eng, dst) -> list:
+    out = []
+    for i in range(0, len(dst), 1024):
+        out += eng.checksum32(dst[i:i + 1024])
+    return out
+
+
+def test_llama3_8b_refit_cast_full_size(oracle, oracle_c, tmp_path, mxp):
+    """Configuration 3: the resident rank slice refitted from a 32 GB fp32 checkpoint whose values carry
+    denormals, infinities and NaNs at 1e-6 density each: slice + round-to-nearest-even cast + checksums in
+    one launch (fsdp/adapter.py:203-206, refit/reshard/receiver.py:964-971)."""
+    layout = models.Llama()
+    tensors = layout.checkpoint(dtype="F32", edge_cases=models.NORMAL_EDGE)
+    by_name = {t.name: t for t in tensors}
+    synth.write_headers_only(tensors, str(tmp_path), n_shards=8)
+    ck = Checkpoint(str(tmp_path))
+    assert sum(t.nbytes for t in ck.tensors()) == 32_121_044_992
+    rv = layout.rank_view(tp_size=TP, tp_rank=RANK, param_dtype="BF16")
+    plan = PlacementPlan(ck, rv.params, tp_size=TP, tp_rank=RANK, stacked_params_mapping=rv.stacked_params_mapping,
+                         allow_cast=True)
+    totals = plan.totals()
+    assert totals["placed_bytes"] == 2_008_031_232 and totals["kernel_algorithmic_bytes"] == 3 * 2_008_031_232
+    eng = PlacementEngine(0)
+    staged = synth.stage_on_device(ck, tensors, seed=SEED)
+    dst = eng.allocate(plan, fill=0x5A)
+    eng.execute_resident(plan, staged, dst)
+    fused = eng.checksums(plan)
+    assert fused == _all_checksums_alone(eng, dst)  # 195 buffers, two independent device passes
+    layer = "model.layers.9."
+    names = [layer + "self_attn.qkv_proj.weight", layer + "self_attn.o_proj.weight", layer + "mlp.down_proj.weight",
+             "model.norm.weight"]
+    host = _check_params_against_oracle(oracle, oracle_c, plan, rv, dst, fused, by_name, names, tp=TP, rank=RANK, cast=True)
+    # the real edge-case density: at 1e-6 each, ~100 M regenerated elements hold every class
+    u = np.concatenate([h.reshape(-1).view("<u4") for h in host.values()])
+    mag = u & 0x7FFFFFFF
+    counts = {"nan": int((mag > 0x7F800000).sum()), "inf": int((mag == 0x7F800000).sum()),
+              "denormal": int(((mag != 0) & (mag < 0x00800000)).sum())}
+    assert all(5 <= c <= 2000 for c in counts.values()), (counts, u.size)
+    # refit again over the live buffers: same bytes
+    eng.execute_resident(plan, staged, dst)
+    assert eng.checksums(plan) == fused
+    eng.close()
+
+
+def test_mixtral_layer_expert_stack_real_shapes(oracle, oracle_c, tmp_path, mxp):
+    """Configuration 4, one layer at its real shapes: eight experts' w1 / w3 [14336, 4096] fused into
+    w13 [8, 28672, 4096], w2 [4096, 14336] stacked into [8, 4096, 14336] (installer.py:695-754)."""
+    layout = models.Mixtral(layers=1)
+    tensors = layout.checkpoint()
+    by_name = {t.name: t for t in tensors}
+    synth.write_headers_only(tensors, str(tmp_path), n_shards=2)
+    ck = Checkpoint(str(tmp_path))
+    rv = layout.rank_view()
+    plan = PlacementPlan(ck, rv.params, stacked_params_mapping=rv.stacked_params_mapping, expert_mapping=rv.expert_mapping)
+    shapes = {p.name: tuple(p.shape) for p in plan.params}
+    pre = "model.layers.0.block_sparse_moe.experts."
+    assert shapes[pre + "w13_weight"] == (8, 28672, 4096) and shapes[pre + "w2_weight"] == (8, 4096, 14336)
+    eng = PlacementEngine(0)
+    staged = synth.stage_on_device(ck, tensors, seed=SEED)
+    dst = eng.allocate(plan, fill=0x33)
+    eng.execute_resident(plan, staged, dst)
+    fused = eng.checksums(plan)
+    assert fused == _all_checksums_alone(eng, dst)
+    _check_params_against_oracle(oracle, oracle_c, plan, rv, dst, fused, by_name,
+                                 [pre + "w13_weight", pre + "w2_weight", "model.layers.0.self_attn.qkv_proj.weight"],
+                                 tp=1, rank=0)
+    eng.close()
+
+
+def test_deepseek_v3_layers_real_shapes(oracle, oracle_c, tmp_path, mxp):
+    """Configuration 5 at real shapes (three dense layers and one MoE layer of 256 routed experts, TP=8 /
+    EP=8): fp8 weights with their fp32 128x128 scale tiles.  o_proj is sliced on K, so its scale tiles are
+    a strided column slice ([56, 128] -> [56, 16]: rows of 64 bytes); q_b_proj / kv_b_proj on rows; the
+    rank's 32 local experts are stacked with their scale tiles (installer.py:80-83,292-339,695-754)."""
+    tp = ep = 8
+    rank = 5
+    layout = models.DeepSeekV3(layers=4, dense_layers=3)
+    tensors = layout.checkpoint()
+    by_name = {t.name: t for t in tensors}
+    synth.write_headers_only(tensors, str(tmp_path), n_shards=6)
+    ck = Checkpoint(str(tmp_path))
+    rv = layout.rank_view(tp_size=tp, tp_rank=rank, ep_size=ep, ep_rank=rank)
+    plan = PlacementPlan(ck, rv.params, tp_size=tp, tp_rank=rank, stacked_params_mapping=rv.stacked_params_mapping,
+                         expert_mapping=rv.expert_mapping)
+    shapes = {p.name: tuple(p.shape) for p in plan.params}
+    a, m = "model.layers.1.self_attn.", "model.layers.3.mlp."
+    assert shapes[a + "o_proj.weight"] == (7168, 2048) and shapes[a + "o_proj.weight_scale_inv"] == (56, 16)
+    assert shapes[m + "experts.w13_weight"] == (32, 4096, 7168) and shapes[m + "experts.w13_weight_scale_inv"] == (32, 32, 56)
+    assert shapes[m + "experts.w2_weight_scale_inv"] == (32, 56, 16)
+    scale_write = [w for w in plan.writes() if w.param == a + "o_proj.weight_scale_inv"]
+    assert len(scale_write) == 1 and (scale_write[0].rows, scale_write[0].row_bytes, scale_write[0].src_pitch) == (56, 64, 512)
+    eng = PlacementEngine(0)
+    staged = synth.stage_on_device(ck, tensors, seed=SEED)
+    dst = eng.allocate(plan, fill=0x44)
+    eng.execute_resident(plan, staged, dst)
+    fused = eng.checksums(plan)
+    assert fused == _all_checksums_alone(eng, dst)
+    names = [a + "o_proj.weight", a + "o_proj.weight_scale_inv", a + "q_b_proj.weight", a + "q_b_proj.weight_scale_inv",
+             a + "kv_b_proj.weight", a + "kv_b_proj.weight_scale_inv", "model.layers.2.mlp.down_proj.weight",
+             "model.layers.2.mlp.down_proj.weight_scale_inv", "model.layers.2.mlp.gate_up_proj.weight_scale_inv",
+             m + "experts.w13_weight", m + "experts.w13_weight_scale_inv", m + "experts.w2_weight",
+             m + "experts.w2_weight_scale_inv", m + "shared_experts.gate_up_proj.weight",
+             m + "shared_experts.down_proj.weight_scale_inv"]
+    _check_params_against_oracle(oracle, oracle_c, plan, rv, dst, fused, by_name, names, tp=tp, rank=rank)
     eng.close()
 
 

@@ -153,6 +153,65 @@ def test_cast_nan_image_is_a_parameter(mxp, oracle):
     eng.close()
 
 
+_TORCH = {"F32": (torch.float32, np.uint32), "BF16": (torch.bfloat16, np.uint16), "F16": (torch.float16, np.uint16),
+          "F8_E4M3": (torch.float8_e4m3fn, np.uint8)}
+
+
+@pytest.mark.parametrize("src_dtype,dst_dtype", [("F32", "BF16"), ("BF16", "F32"), ("F16", "F32"), ("F32", "F16"),
+                                                 ("F8_E4M3", "BF16"), ("F16", "BF16"), ("BF16", "F16")])
+def test_default_conversions_equal_torch_on_this_device(gpu_engine, src_dtype, dst_dtype):
+    """What the reference runs for a dtype-converting copy is ``recv.copy_(staging)`` on the DEVICE
+    (refit/reshard/receiver.py:964-971, fsdp/adapter.py:203-206), so the images this library produces
+    with default options - NaNs of every sign and payload included - are compared bit for bit with
+    ``torch.Tensor.to`` run on this very GPU.  (torch's CPU kernels may disagree about NaNs with the
+    device ones: fp32 -> bf16 gives 0xFFFF on AVX-512 hosts and 0x7FC0 on the device.)"""
+    rng = np.random.default_rng(21)
+    t_src, np_src = _TORCH[src_dtype]
+    t_dst, np_dst = _TORCH[dst_dtype]
+    bits = np.dtype(np_src).itemsize * 8
+    if bits == 32:
+        nan_exp = np.uint32(0x7F800000)
+        payload = rng.integers(1, 1 << 23, 4096, dtype=np.uint64).astype(np.uint32)
+        sign = (rng.integers(0, 2, 4096, dtype=np.uint64).astype(np.uint32) << 31)
+        nans = nan_exp | payload | sign
+        special = np.array([0x7FC00000, 0xFFC00000, 0x7F800001, 0xFF800001, 0x7FFFFFFF, 0xFFFFFFFF, 0x7F800000, 0xFF800000,
+                            0x00000001, 0x807FFFFF, 0x7F7FFFFF, 0x3F808000, 0x3F818000, 0x477FE000, 0x477FF000, 0x33000000],
+                           dtype=np.uint32)
+        src = np.concatenate([special, nans, rng.integers(0, 1 << 32, 1 << 16, dtype=np.uint64).astype(np.uint32)])
+    elif bits == 16:
+        src = np.arange(1 << 16, dtype=np.uint16)  # every pattern, every NaN among them
+    else:
+        src = np.arange(256, dtype=np.uint8)
+    dev_src = torch.from_numpy(src.copy()).cuda()
+    want = dev_src.view(t_src).to(t_dst).contiguous().view(torch.uint8).cpu().numpy().view(np_dst)
+    out = torch.zeros(src.size * np.dtype(np_dst).itemsize, dtype=torch.uint8, device="cuda")
+    gpu_engine.cast(dev_src.view(torch.uint8), out, src.size, src_dtype, dst_dtype, checksum=False)
+    got = out.cpu().numpy().view(np_dst)
+    bad = np.flatnonzero(got != want)
+    assert bad.size == 0, [(hex(int(src[i])), hex(int(got[i])), hex(int(want[i]))) for i in bad[:8]]
+
+
+def test_nan_image_of_the_host_can_be_probed_and_asked_for(mxp):
+    """A caller that wants the CPU path's bytes instead (torch CPU maps every fp32 NaN to one image that
+    depends on the host's vector ISA) probes that image and passes it as ``nan_bits``."""
+    from modelexpress_amd.engine import PlacementEngine
+
+    probed = int(torch.tensor([float("nan")]).to(torch.bfloat16).view(torch.int16).item()) & 0xFFFF
+    assert (probed & 0x7FFF) > 0x7F80
+    rng = np.random.default_rng(22)
+    nans = (np.uint32(0x7F800000) | rng.integers(1, 1 << 23, 2048, dtype=np.uint64).astype(np.uint32)
+            | (rng.integers(0, 2, 2048, dtype=np.uint64).astype(np.uint32) << 31))
+    src = np.concatenate([nans, rng.integers(0, 1 << 32, 1 << 14, dtype=np.uint64).astype(np.uint32)])
+    want = torch.from_numpy(src.view(np.float32).copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    if not np.all(want[:2048] == probed):
+        pytest.skip("torch CPU on this host does not map every NaN to one image")
+    eng = PlacementEngine(0, nan_bits=probed)
+    out = torch.zeros(src.size * 2, dtype=torch.uint8, device="cuda")
+    eng.cast_f32_bf16(_dev(src), out, src.size)
+    assert np.array_equal(out.cpu().numpy().view(np.uint16), want)
+    eng.close()
+
+
 @pytest.mark.parametrize("rows,row_bytes,src_pitch,dst_pitch,src_off", [
     (4096, 1024, 8192, 1024, 1024 * 3),      # o_proj TP=8 column slice
     (512, 3584, 28672, 3584, 3584 * 5),      # down_proj TP=8 column slice

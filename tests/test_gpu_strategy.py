@@ -255,6 +255,7 @@ def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
     rec = ad.timing.as_dict()
     assert rec["backend"] == "hip_placement" and rec["version"] == "v1" and rec["bytes"] == sum(p.nbytes for p in rv.params)
     assert {"transfer_planning", "wire_transfer", "receive_sync", "installation"} <= set(rec["stages"])
+    assert rec["cast_nan_bits"] == "0x7fc0"  # the image the casts of this cycle wrote (torch's device image)
     assert ad.timing.emit().startswith("MX_REFIT_TIMING {")
     ad.release_staged_weight(staged)
     ad.close()
