@@ -292,6 +292,15 @@ int mxp_execute_after(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs,
 int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* file_dev_ptrs,
                          void* const* dst_ptrs, void* stream, mxp_exec_stats* stats);
 
+/* Final-address placement (on by default).  During mxp_execute a piece that is contiguous in the
+ * file and in its parameter buffer and is not converted is copied by hipMemcpyAsync from the pinned
+ * slot straight to its final address - the reference's own loader reads each tensor into its own
+ * device buffer (gds_loader.py:284-331) - and the kernel only reads it back for the checksum (and
+ * the digest sums); strided slices, conversions and pieces under `min_bytes` still go through the
+ * bounce slot and the placement kernel.  min_bytes: 0 = the default (64 KiB), a negative value =
+ * off (every byte takes the bounce slot).  Results are identical either way. */
+int mxp_engine_set_direct_placement(mxp_engine* engine, int64_t min_bytes);
+
 /* Launch timing for measurements.  Switched on, every asynchronous mxp_execute_resident (stats ==
  * NULL) records a HIP-event pair around its placement kernel on the launch stream and does NOT
  * synchronise, so a timed loop of K launches yields both its wall time and the K kernel
@@ -334,6 +343,21 @@ int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* 
  * `stream` is idle, like mxp_checksum32. */
 int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
                           uint32_t* out, void* stream);
+/* mxp_checksum32 / mxp_digest over a FIXED set of device buffers, lowered once: a refit loop
+ * verifies the same buffers every step, and the reference keeps its descriptor lists for that
+ * reason (refit/reshard/receiver.py:787-801; the verify loop is
+ * modelexpress_rl/inference/nixl_staged_transfer.py:529-549).  _create lowers the buffers, uploads
+ * the descriptor tables and allocates the result block; a run is then one kernel launch and one
+ * small copy back (no descriptor build, no upload, no allocation), and waits only for that copy.
+ * The addresses and sizes are the ones given at create; when a buffer moves, build a new plan.
+ * One run of a plan at a time. */
+typedef struct mxp_verify_plan mxp_verify_plan;
+int mxp_verify_plan_create(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
+                           mxp_verify_plan** out);
+int mxp_verify_plan_checksums(mxp_engine* engine, mxp_verify_plan* plan, uint32_t* out, void* stream);
+/* `scalars` as for mxp_digest (7 u64 per buffer), or NULL. */
+int mxp_verify_plan_digests(mxp_engine* engine, mxp_verify_plan* plan, uint8_t* out16, uint64_t* scalars, void* stream);
+void mxp_verify_plan_destroy(mxp_verify_plan* plan);
 /* tensor_digest (refit/reshard/verify.py:79-155) of n device buffers: 16 bytes each
  * (blake2b-128 over the little-endian u64 scalars).  `scalars`, if not NULL, receives
  * 7 u64 per tensor: n, sum_rows, sum_rows_weighted, sum_tail, sum_tail_weighted,

@@ -145,11 +145,16 @@ SIGNATURES = {
     "mxp_execute": (C.c_int, [_P, _P, _PP, C.POINTER(ExecStats)]),
     "mxp_execute_after": (C.c_int, [_P, _P, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_execute_resident": (C.c_int, [_P, _P, _PP, _PP, _P, C.POINTER(ExecStats)]),
+    "mxp_engine_set_direct_placement": (C.c_int, [_P, C.c_int64]),
     "mxp_engine_set_launch_timing": (C.c_int, [_P, C.c_int32]),
     "mxp_engine_launch_times": (C.c_int, [_P, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
     "mxp_plan_checksums": (C.c_int, [_P, _P, _U32P, C.c_int64]),
     "mxp_checksum32": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_checksum32_static": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
+    "mxp_verify_plan_create": (C.c_int, [_P, _PP, _U64P, C.c_int64, C.POINTER(C.c_void_p)]),
+    "mxp_verify_plan_checksums": (C.c_int, [_P, _P, _U32P, _P]),
+    "mxp_verify_plan_digests": (C.c_int, [_P, _P, C.POINTER(C.c_uint8), _U64P, _P]),
+    "mxp_verify_plan_destroy": (None, [_P]),
     "mxp_digest": (C.c_int, [_P, _PP, _U64P, C.c_int64, C.POINTER(C.c_uint8), _U64P, _P]),
     "mxp_cast_f32_bf16": (C.c_int, [_P, _P, _P, C.c_uint64, _U32P, _P]),
     "mxp_cast": (C.c_int, [_P, _P, _P, C.c_uint64, C.c_int32, _U32P, _P]),

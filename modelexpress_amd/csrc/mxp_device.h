@@ -69,6 +69,10 @@ struct alignas(16) Seg {
 };
 static_assert(sizeof(Seg) == 80, "Seg layout is part of the host<->device contract");
 
+// `src_buf` of a checksum-only segment that reads the destination buffer `dst_buf` itself (bytes a
+// host-to-device copy placed there) instead of a source buffer.
+constexpr uint32_t kSrcIsDestination = 0xFFFFFFFFu;
+
 struct WorkItem {
   uint32_t seg;
   uint32_t tile;

@@ -90,6 +90,9 @@ uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
 
+// Pieces below this size take the bounce slot by default: a copy call of their own would cost more than it saves.
+constexpr uint64_t kDirectMinBytes = 64 * 1024;
+
 template <typename T>
 struct DevBuf {
   T* p = nullptr;
@@ -128,6 +131,7 @@ struct mxp_plan::Lowered {
   uint64_t slot_bytes = 0;
   uint32_t tile_bytes = 0;
   bool host_pack = false;
+  uint64_t direct_min = 0;
   int reader_threads = 0;  // the chunk-size ramp depends on it
   bool direct_io = false;
   // resident tables: source buffer index = shard file index
@@ -178,6 +182,8 @@ struct mxp_engine {
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
   hipEvent_t caller_ev = nullptr;   // what the caller had queued when an ingest started
   bool fused_digests = false;       // placements also accumulate the tensor_digest sums (mxp_engine_set_fused_digests)
+  uint64_t direct_min = kDirectMinBytes;  // ingest copies contiguous pieces of at least this size straight to their
+                                          // final address; 0 = none (mxp_engine_set_direct_placement)
   hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
   bool arena_recorded = false;
   // descriptor table of batched transposes: same protocol as the arena, its own event
@@ -225,6 +231,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   const bool host_pack = eng.opt.pack_strided_on_host == 1;
   if (pl.lowered && pl.lowered->slot_bytes == eng.opt.slot_bytes && pl.lowered->tile_bytes == eng.opt.tile_bytes &&
       pl.lowered->host_pack == host_pack && pl.lowered->direct_io == (eng.opt.use_o_direct != 0) &&
+      pl.lowered->direct_min == eng.direct_min &&
       pl.lowered->reader_threads == eng.opt.reader_threads)
     return;
   if (pl.lowered) { free_lowered(pl.lowered); pl.lowered = nullptr; }
@@ -232,6 +239,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   L->slot_bytes = eng.opt.slot_bytes;
   L->tile_bytes = eng.opt.tile_bytes;
   L->host_pack = host_pack;
+  L->direct_min = eng.direct_min;
   L->direct_io = eng.opt.use_o_direct != 0;
   L->reader_threads = eng.opt.reader_threads;
   // Direct I/O reads whole 4 KiB blocks at 4 KiB offsets into 4 KiB aligned memory: every
@@ -347,7 +355,8 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       if (cur.ranges.empty()) return;
       cur.seg_count = (uint32_t)segs.size() - cur.seg_begin;
       cur.work_count = (uint32_t)work.size() - cur.work_begin;
-      L->h2d_bytes += cur.used_bytes;
+      for (const auto& d : cur.direct) L->h2d_bytes += d.nbytes;
+      for (const auto& r : cur.bounce_runs) L->h2d_bytes += r.second;
       L->chunks.push_back(cur);
       cur = Chunk();
     };
@@ -424,7 +433,31 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
         L->file_bytes += in_slot;
         p.box.src_off = at + lead;
         const size_t w0 = work.size();
-        lower_box(p.box, lo, segs, work);
+        // A piece that is contiguous on both sides and not converted needs no kernel to move it: the
+        // host-to-device copy lands it at its final address (as the reference's loader reads a tensor
+        // straight into its own device buffer, gds_loader.py:284-331) and the kernel only reads it
+        // back for the checksum.  Everything else goes through the bounce slot.
+        const uint64_t piece_dst = p.box.rows * p.box.row_bytes;
+        const bool abutting = p.box.rows == 1 || (p.box.src_pitch == op_src_bytes(p.box.op, p.box.row_bytes) &&
+                                                  p.box.dst_pitch == p.box.row_bytes);
+        if (L->direct_min && p.box.op == kOpCopy && abutting && piece_dst >= L->direct_min) {
+          cur.direct.push_back(DirectCopy{at + lead, p.box.dst_off, piece_dst, p.box.dst_buf});
+          BoxCopy c;
+          c.src_buf = kSrcIsDestination;
+          c.dst_buf = p.box.dst_buf;
+          c.src_off = c.dst_off = p.box.dst_off;
+          c.row_bytes = piece_dst;
+          c.op = kOpChecksumOnly;
+          c.csum_slot = p.box.csum_slot;
+          lower_box(c, lo, segs, work);
+        } else {
+          const uint64_t lo_off = at, hi_off = at + in_slot;
+          if (!cur.bounce_runs.empty() && lo_off - (cur.bounce_runs.back().first + cur.bounce_runs.back().second) < 4096)
+            cur.bounce_runs.back().second = hi_off - cur.bounce_runs.back().first;  // a small gap is cheaper than another copy
+          else
+            cur.bounce_runs.emplace_back(lo_off, hi_off - lo_off);
+          lower_box(p.box, lo, segs, work);
+        }
         // work items index segments relative to the chunk's first segment
         for (size_t k = w0; k < work.size(); ++k) work[k].seg -= cur.seg_begin;
         if (!have_rest) break;
@@ -783,8 +816,12 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
           }
         read_s[tid] += now_s() - t0;
         hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
-        HIP_OK(hipMemcpyAsync(sl.dev, sl.host, ch.used_bytes, hipMemcpyHostToDevice, st));
         mutated.store(1);
+        for (const auto& r : ch.bounce_runs)
+          HIP_OK(hipMemcpyAsync(sl.dev + r.first, sl.host + r.first, r.second, hipMemcpyHostToDevice, st));
+        for (const auto& d : ch.direct)
+          HIP_OK(hipMemcpyAsync(static_cast<uint8_t*>(dst_ptrs[d.param]) + d.dst_off, sl.host + d.slot_off, d.nbytes,
+                                hipMemcpyHostToDevice, st));
         if (digests)
           HIP_OK(launch_place_digest(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
                                      e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, L.dst_sizes.p, L.digest_sums.p,
@@ -937,6 +974,14 @@ int mxp_engine_set_fused_digests(mxp_engine* engine, int32_t on) {
   return guard([&] {
     if (!engine) throw Error(MXP_ERR_ARG, "mxp_engine_set_fused_digests: null engine");
     engine->fused_digests = on != 0;
+  });
+}
+
+int mxp_engine_set_direct_placement(mxp_engine* engine, int64_t min_bytes) {
+  return guard([&] {
+    if (!engine) throw Error(MXP_ERR_ARG, "mxp_engine_set_direct_placement: null engine");
+    // a plan is lowered again when it next runs on this engine
+    engine->direct_min = min_bytes < 0 ? 0 : min_bytes == 0 ? kDirectMinBytes : (uint64_t)min_bytes;
   });
 }
 
@@ -1546,6 +1591,146 @@ struct mxp_view_plan {
   DevBuf<TransposeItem> items;
   uint64_t bytes = 0;  // destination bytes one run writes
 };
+
+// A fixed set of device buffers lowered once for repeated verification (mxp_verify_plan_create):
+// descriptor tables, accumulators and a pinned result block of its own, so a run neither builds
+// nor uploads anything.
+struct mxp_verify_plan {
+  int device = 0;
+  int64_t n = 0;
+  std::vector<uint64_t> nbytes;
+  DevBuf<uint8_t> tables;  // [segments][work items][source pointers][checksums][digest jobs][digest sums]
+  size_t o_work = 0, o_src = 0, o_sums = 0, o_jobs = 0, o_dsums = 0;
+  uint32_t n_work = 0, n_blocks = 0;
+  uint8_t* host = nullptr;  // pinned: [checksums][digest sums]
+  hipEvent_t done = nullptr;     // results have reached `host`
+  hipEvent_t cleared = nullptr;  // the accumulators are zero again
+  bool cleared_rec = false;
+  ~mxp_verify_plan() {
+    if (host) (void)hipHostFree(host);
+    if (done) (void)hipEventDestroy(done);
+    if (cleared) (void)hipEventDestroy(cleared);
+  }
+};
+
+int mxp_verify_plan_create(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
+                           mxp_verify_plan** out) {
+  return guard([&] {
+    if (!out) throw Error(MXP_ERR_ARG, "mxp_verify_plan_create: null out");
+    *out = nullptr;
+    if (!engine || n < 0 || (n && (!ptrs || !nbytes))) throw Error(MXP_ERR_ARG, "mxp_verify_plan_create: bad argument");
+    auto vp = std::make_unique<mxp_verify_plan>();
+    vp->device = engine->opt.device;
+    vp->n = n;
+    HIP_OK(hipSetDevice(vp->device));
+    LowerOptions lo;
+    lo.tile_bytes = engine->opt.tile_bytes;
+    std::vector<Seg> segs;
+    std::vector<WorkItem> work;
+    std::vector<const void*> srcs;
+    std::vector<DigestJob> jobs((size_t)n);
+    uint64_t blocks = 0;
+    for (int64_t k = 0; k < n; ++k) {
+      if (nbytes[k] && !ptrs[k]) throw Error(MXP_ERR_ARG, "mxp_verify_plan_create: null pointer");
+      vp->nbytes.push_back(nbytes[k]);
+      const void* base;
+      uint64_t off;
+      split_ptr(ptrs[k], base, off);
+      srcs.push_back(base);
+      BoxCopy b;
+      b.src_buf = (uint32_t)k;
+      b.src_off = off;
+      b.row_bytes = nbytes[k];
+      b.op = kOpChecksumOnly;
+      b.csum_slot = (uint32_t)k;
+      lower_box(b, lo, segs, work);
+      jobs[k].ptr = static_cast<const uint8_t*>(ptrs[k]);
+      jobs[k].nbytes = nbytes[k];
+      jobs[k].out_slot = (uint64_t)k * 5;
+      jobs[k].first_block = blocks;
+      const uint64_t rows = (nbytes[k] / 4) / kDigestRowWords;
+      blocks += rows ? (rows + kDigestRowsPerBlock - 1) / kDigestRowsPerBlock : 1;
+    }
+    if (work.size() > 0x7FFFFFFFull || blocks > 0x7FFFFFFFull) throw Error(MXP_ERR_ARG, "mxp_verify_plan_create: batch too large for one launch");
+    vp->n_work = (uint32_t)work.size();
+    vp->n_blocks = (uint32_t)blocks;
+    vp->o_work = align_up(segs.size() * sizeof(Seg), 256);
+    vp->o_src = align_up(vp->o_work + work.size() * sizeof(WorkItem), 256);
+    vp->o_sums = align_up(vp->o_src + srcs.size() * sizeof(void*), 256);
+    vp->o_jobs = align_up(vp->o_sums + (size_t)n * 4, 256);
+    vp->o_dsums = align_up(vp->o_jobs + jobs.size() * sizeof(DigestJob), 256);
+    std::vector<uint8_t> host(align_up(vp->o_dsums + (size_t)n * 40, 256) + 256, 0);  // accumulators start at zero
+    if (!segs.empty()) std::memcpy(host.data(), segs.data(), segs.size() * sizeof(Seg));
+    if (!work.empty()) std::memcpy(host.data() + vp->o_work, work.data(), work.size() * sizeof(WorkItem));
+    if (!srcs.empty()) std::memcpy(host.data() + vp->o_src, srcs.data(), srcs.size() * sizeof(void*));
+    if (!jobs.empty()) std::memcpy(host.data() + vp->o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
+    vp->tables.upload(host.data(), host.size());
+    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&vp->host), (size_t)(n ? n : 1) * 44 + 16, hipHostMallocDefault));
+    HIP_OK(hipEventCreateWithFlags(&vp->done, hipEventDisableTiming));
+    HIP_OK(hipEventCreateWithFlags(&vp->cleared, hipEventDisableTiming));
+    *out = vp.release();
+  });
+}
+
+int mxp_verify_plan_checksums(mxp_engine* engine, mxp_verify_plan* plan, uint32_t* out, void* stream_v) {
+  return guard([&] {
+    if (!engine || !plan || (plan->n && !out)) throw Error(MXP_ERR_ARG, "mxp_verify_plan_checksums: null argument");
+    if (plan->device != engine->opt.device) throw Error(MXP_ERR_ARG, "mxp_verify_plan_checksums: the plan was built for another device");
+    if (plan->n == 0) return;
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    HIP_OK(hipSetDevice(plan->device));
+    uint8_t* d = plan->tables.p;
+    uint32_t* sums = reinterpret_cast<uint32_t*>(d + plan->o_sums);
+    if (plan->cleared_rec) HIP_OK(hipStreamWaitEvent(stream, plan->cleared, 0));  // a run on another stream than the last
+    HIP_OK(launch_place(reinterpret_cast<const Seg*>(d), reinterpret_cast<const WorkItem*>(d + plan->o_work), plan->n_work,
+                        reinterpret_cast<const void* const*>(d + plan->o_src), nullptr, sums, engine->opt.nan_bits, stream, true));
+    HIP_OK(hipMemcpyAsync(plan->host, sums, (size_t)plan->n * 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipEventRecord(plan->done, stream));
+    // the accumulators are cleared for the next run behind the result copy, off the caller's path
+    HIP_OK(launch_fill_u32(sums, (uint64_t)plan->n, 0u, stream));
+    HIP_OK(hipEventRecord(plan->cleared, stream));
+    plan->cleared_rec = true;
+    HIP_OK(hipEventSynchronize(plan->done));
+    std::memcpy(out, plan->host, (size_t)plan->n * 4);
+  });
+}
+
+int mxp_verify_plan_digests(mxp_engine* engine, mxp_verify_plan* plan, uint8_t* out16, uint64_t* scalars, void* stream_v) {
+  return guard([&] {
+    if (!engine || !plan || (plan->n && !out16)) throw Error(MXP_ERR_ARG, "mxp_verify_plan_digests: null argument");
+    if (plan->device != engine->opt.device) throw Error(MXP_ERR_ARG, "mxp_verify_plan_digests: the plan was built for another device");
+    if (plan->n == 0) return;
+    hipStream_t stream = static_cast<hipStream_t>(stream_v);
+    HIP_OK(hipSetDevice(plan->device));
+    uint8_t* d = plan->tables.p;
+    unsigned long long* dsums = reinterpret_cast<unsigned long long*>(d + plan->o_dsums);
+    if (plan->cleared_rec) HIP_OK(hipStreamWaitEvent(stream, plan->cleared, 0));
+    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(d + plan->o_jobs), (uint32_t)plan->n, plan->n_blocks, dsums, stream));
+    uint8_t* h = plan->host + (size_t)plan->n * 4;  // 8-byte aligned: n * 4 with n * 40 behind it needs n even or a pad
+    h = reinterpret_cast<uint8_t*>((reinterpret_cast<uintptr_t>(h) + 7u) & ~(uintptr_t)7u);
+    HIP_OK(hipMemcpyAsync(h, dsums, (size_t)plan->n * 40, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipEventRecord(plan->done, stream));
+    HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(dsums), (uint64_t)plan->n * 10, 0u, stream));
+    HIP_OK(hipEventRecord(plan->cleared, stream));
+    plan->cleared_rec = true;
+    HIP_OK(hipEventSynchronize(plan->done));
+    const uint64_t* sums = reinterpret_cast<const uint64_t*>(h);
+    for (int64_t k = 0; k < plan->n; ++k) {
+      const uint64_t nb = plan->nbytes[(size_t)k];
+      const uint64_t sc[7] = {nb, sums[5 * k], sums[5 * k + 1], sums[5 * k + 2], sums[5 * k + 3], sums[5 * k + 4], nb % 4};
+      if (scalars) std::memcpy(scalars + 7 * k, sc, sizeof sc);
+      const int rc = mxp_digest_from_scalars(sc, out16 + 16 * k);
+      if (rc != MXP_OK) throw Error(rc, mxp_last_error());
+    }
+  });
+}
+
+void mxp_verify_plan_destroy(mxp_verify_plan* plan) {
+  if (!plan) return;
+  (void)hipSetDevice(plan->device);
+  (void)hipDeviceSynchronize();
+  delete plan;
+}
 
 int mxp_permute_copy(mxp_engine* engine, const void* src, void* dst, int32_t ndim, const int64_t* shape,
                      const int64_t* src_strides, const int32_t* perm, int32_t elem_size, uint32_t* checksum,

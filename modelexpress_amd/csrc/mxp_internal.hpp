@@ -98,9 +98,17 @@ struct FileRange {
   uint64_t rows = 1, file_pitch = 0;
   uint64_t need = 0;  // bytes that must exist (a direct-I/O range is rounded up past them); 0 = all
 };
+// A contiguous, unconverted piece of a chunk that is copied from the pinned slot straight to its
+// final place in a parameter buffer.
+struct DirectCopy {
+  uint64_t slot_off, dst_off, nbytes;
+  uint32_t param;
+};
 struct Chunk {
   std::vector<FileRange> ranges;
-  uint64_t used_bytes = 0;   // bytes of the slot that cross PCIe
+  std::vector<DirectCopy> direct;                           // pinned slot -> parameter buffer
+  std::vector<std::pair<uint64_t, uint64_t>> bounce_runs;   // (slot offset, bytes): pinned slot -> bounce slot
+  uint64_t used_bytes = 0;   // bytes of the slot in use
   uint32_t seg_begin = 0, seg_count = 0;    // into the ingest segment table
   uint32_t work_begin = 0, work_count = 0;  // into the ingest work table
 };

@@ -12,68 +12,12 @@
 //  digest_kernel  int32-word row sums for the blake2b-hashed tensor digest
 //                 (reads each byte once)
 #include "mxp_device.h"
+#include "mxp_checksum.h"
 #include "mxp_convert.h"
 #include <atomic>
 #include <type_traits>
 
 namespace mxp {
-
-// ---------------------------------------------------------------------------
-// Checksum algebra.  The per-tensor fingerprint is
-//     sum_i  byte[i] * ((i * 2654435761 + 1) mod 2^32)   mod 2^32
-// (reference: modelexpress/tensor_utils.py:27-44).  For a group of bytes starting at
-// position i with local offsets j:
-//     sum_j b_j * ((i + j) K + 1) = K * (i * S0 + S1) + S0,   S0 = sum b_j, S1 = sum j b_j
-// so three wrapping 32-bit accumulators P = sum i*S0, R = sum S1, Q = sum S0 are kept
-// per lane and folded once at the end as K * (P + R) + Q.  S0 and S1 come from the
-// unsigned 8-bit dot-product instruction, four bytes at a time.
-// ---------------------------------------------------------------------------
-struct Csum {
-  uint32_t P = 0, Q = 0, R = 0;
-  __device__ __forceinline__ void add16(const uint4& x, uint32_t i) {
-    uint32_t s0 = __builtin_amdgcn_udot4(x.x, 0x01010101u, 0u, false);
-    s0 = __builtin_amdgcn_udot4(x.y, 0x01010101u, s0, false);
-    s0 = __builtin_amdgcn_udot4(x.z, 0x01010101u, s0, false);
-    s0 = __builtin_amdgcn_udot4(x.w, 0x01010101u, s0, false);
-    R = __builtin_amdgcn_udot4(x.x, 0x03020100u, R, false);
-    R = __builtin_amdgcn_udot4(x.y, 0x07060504u, R, false);
-    R = __builtin_amdgcn_udot4(x.z, 0x0b0a0908u, R, false);
-    R = __builtin_amdgcn_udot4(x.w, 0x0f0e0d0cu, R, false);
-    Q += s0;
-    P += i * s0;
-  }
-  __device__ __forceinline__ void add8(uint32_t lo, uint32_t hi, uint32_t i) {
-    uint32_t s0 = __builtin_amdgcn_udot4(lo, 0x01010101u, 0u, false);
-    s0 = __builtin_amdgcn_udot4(hi, 0x01010101u, s0, false);
-    R = __builtin_amdgcn_udot4(lo, 0x03020100u, R, false);
-    R = __builtin_amdgcn_udot4(hi, 0x07060504u, R, false);
-    Q += s0;
-    P += i * s0;
-  }
-  // Up to four bytes packed little-endian in x (missing bytes zero).
-  __device__ __forceinline__ void add4(uint32_t x, uint32_t i) {
-    uint32_t s0 = __builtin_amdgcn_udot4(x, 0x01010101u, 0u, false);
-    R = __builtin_amdgcn_udot4(x, 0x03020100u, R, false);
-    Q += s0;
-    P += i * s0;
-  }
-  // One unit of UNIT <= 4 bytes (the narrow paths).
-  template <int UNIT>
-  __device__ __forceinline__ void addn(uint32_t x, uint32_t i) { add4(x, i); }
-  __device__ __forceinline__ uint32_t fold() const { return kKnuth * (P + R) + Q; }
-};
-
-__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
-  return v;
-}
-
-__device__ __forceinline__ unsigned long long wave_sum_u64(unsigned long long v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
-  return v;
-}
 
 // Checksum plus the tensor_digest sums of the bytes being stored (reference:
 // modelexpress/refit/reshard/verify.py:112-150), for launches that verify what they place
@@ -406,8 +350,8 @@ __device__ __forceinline__ void place_body(
   const uint32_t r0 = w.tile * s.rows_per_tile;
   const uint32_t nrows = min(s.rows - r0, s.rows_per_tile);
   const uint32_t n_units = nrows * s.units_per_row;
-  const uint8_t* src =
-      static_cast<const uint8_t*>(src_bases[s.src_buf]) + s.src_off + (uint64_t)r0 * s.src_pitch;
+  const void* src_base = s.src_buf == kSrcIsDestination ? dst_bases[s.dst_buf] : src_bases[s.src_buf];
+  const uint8_t* src = static_cast<const uint8_t*>(src_base) + s.src_off + (uint64_t)r0 * s.src_pitch;
   uint8_t* dst = nullptr;
   if (s.op != kOpChecksumOnly)
     dst = static_cast<uint8_t*>(dst_bases[s.dst_buf]) + s.dst_off + (uint64_t)r0 * s.dst_pitch;
@@ -449,6 +393,7 @@ __device__ __forceinline__ void place_body(
     case kOpCastBf16F16 * 32u + 2u: run_tile<kOpCastBf16F16, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 16u: run_tile<kOpChecksumOnly, 16>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 4u: run_tile<kOpChecksumOnly, 4>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
+    case kOpChecksumOnly * 32u + 2u: run_tile<kOpChecksumOnly, 2>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     case kOpChecksumOnly * 32u + 1u: run_tile<kOpChecksumOnly, 1>(s, src, dst, csum_base, n_units, nan_bits, cs); break;
     default: break;  // the host validates (op, unit) before upload
   }

@@ -45,17 +45,12 @@
 // 384 bytes lifts 16384 x 16384 to 6.0 TB/s: the loss is in how the strided source lines fall
 // on the memory channels, which a caller controls and this kernel does not.
 #include "mxp_device.h"
+#include "mxp_checksum.h"
 #include "mxp_convert.h"
 
 namespace mxp {
 
 namespace {
-
-__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_down(v, o, 64);
-  return v;
-}
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 ld16_nt(const uint8_t* p) {
@@ -67,28 +62,6 @@ __device__ __forceinline__ void st16_nt(uint8_t* p, const uint4& v) {
   t.x = v.x; t.y = v.y; t.z = v.z; t.w = v.w;
   __builtin_nontemporal_store(t, reinterpret_cast<u32x4*>(p));
 }
-
-// Same checksum algebra as place_kernel (see mxp_kernels.hip).
-struct Csum {
-  uint32_t P = 0, Q = 0, R = 0;
-  __device__ __forceinline__ void add16(const uint4& x, uint32_t i) {
-    uint32_t s0 = __builtin_amdgcn_udot4(x.x, 0x01010101u, 0u, false);
-    s0 = __builtin_amdgcn_udot4(x.y, 0x01010101u, s0, false);
-    s0 = __builtin_amdgcn_udot4(x.z, 0x01010101u, s0, false);
-    s0 = __builtin_amdgcn_udot4(x.w, 0x01010101u, s0, false);
-    R = __builtin_amdgcn_udot4(x.x, 0x03020100u, R, false);
-    R = __builtin_amdgcn_udot4(x.y, 0x07060504u, R, false);
-    R = __builtin_amdgcn_udot4(x.z, 0x0b0a0908u, R, false);
-    R = __builtin_amdgcn_udot4(x.w, 0x0f0e0d0cu, R, false);
-    Q += s0;
-    P += i * s0;
-  }
-  __device__ __forceinline__ void add_byte(uint32_t b, uint32_t i) {
-    Q += b;
-    P += i * b;
-  }
-  __device__ __forceinline__ uint32_t fold() const { return kKnuth * (P + R) + Q; }
-};
 
 constexpr int kWaves = kTransposeWaves;
 constexpr int kThreads = kWaves * 64;

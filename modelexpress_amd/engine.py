@@ -281,6 +281,11 @@ class PlacementEngine:
                                              C.byref(stats) if timed else None))
         return stats.as_dict() if timed else None
 
+    def set_direct_placement(self, min_bytes: int = 0) -> None:
+        """Ingest copies contiguous unconverted pieces of at least ``min_bytes`` straight to their final address
+        (0 = the default, 64 KiB); a negative value sends every byte through the bounce slot and the kernel."""
+        L.check(L.lib().mxp_engine_set_direct_placement(self._h, int(min_bytes)))
+
     def set_launch_timing(self, on: bool = True) -> None:
         """Asynchronous resident launches record an event pair around their placement kernel (no synchronisation)."""
         L.check(L.lib().mxp_engine_set_launch_timing(self._h, 1 if on else 0))
@@ -326,6 +331,10 @@ class PlacementEngine:
         L.check(L.lib().mxp_checksum32_static(self._h, _ptr_array([_addr(t) for t in buffers]),
                                               (C.c_uint64 * max(1, n))(*sizes), n, out, C.c_void_p(stream)))
         return [format(out[i], "08x") for i in range(n)]
+
+    def verify_plan(self, buffers: Sequence, nbytes: Sequence[int] | None = None) -> "VerifyPlan":
+        """``buffers`` lowered once for repeated ``checksums()`` / ``digests()`` passes."""
+        return VerifyPlan(self, buffers, nbytes)
 
     def digest(self, buffers: Sequence, nbytes: Sequence[int] | None = None, *, stream: int = 0,
                with_scalars: bool = False):
@@ -490,6 +499,43 @@ class PlacementEngine:
         out = C.c_double()
         L.check(L.lib().mxp_measure_h2d(self._h, nbytes, repeats, C.byref(out)))
         return float(out.value)
+
+
+class VerifyPlan:
+    """Handle of ``mxp_verify_plan``: a fixed set of device buffers lowered once for repeated ``checksum32`` /
+    ``tensor_digest`` passes; a run is one launch and one small copy back."""
+
+    def __init__(self, engine: "PlacementEngine", buffers: Sequence, nbytes: Sequence[int] | None = None):
+        self._engine = engine
+        self.n = len(buffers)
+        sizes = [_nbytes(t) for t in buffers] if nbytes is None else list(nbytes)
+        self._keep = list(buffers)  # the plan holds raw addresses: keep the tensors alive with it
+        self._h = C.c_void_p()
+        L.check(L.lib().mxp_verify_plan_create(engine._h, _ptr_array([_addr(t) for t in buffers]),
+                                               (C.c_uint64 * max(1, self.n))(*sizes), self.n, C.byref(self._h)))
+        self._sums = (C.c_uint32 * max(1, self.n))()
+        self._dig = (C.c_uint8 * (16 * max(1, self.n)))()
+
+    def checksums(self, *, stream: int = 0) -> list[str]:
+        L.check(L.lib().mxp_verify_plan_checksums(self._engine._h, self._h, self._sums, C.c_void_p(stream)))
+        return [format(self._sums[i], "08x") for i in range(self.n)]
+
+    def digests(self, *, stream: int = 0) -> list[str]:
+        L.check(L.lib().mxp_verify_plan_digests(self._engine._h, self._h, self._dig, None, C.c_void_p(stream)))
+        raw = bytes(self._dig)
+        return [raw[16 * i: 16 * i + 16].hex() for i in range(self.n)]
+
+    def close(self) -> None:
+        if self._h:
+            L.lib().mxp_verify_plan_destroy(self._h)
+            self._h = C.c_void_p()
+            self._keep = []
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:  # noqa: BLE001
+            pass
 
 
 class ViewPlan:

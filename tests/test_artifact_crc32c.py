@@ -3,10 +3,22 @@
 
 import zlib
 
+import pytest
+
 from modelexpress_amd.artifact_manifest import build_checksums, crc32c
 
 
 def test_pinned_vectors(mxp):
+    _pinned_vectors()
+
+
+@pytest.mark.gpu
+def test_pinned_vectors_on_the_gpu_box(mxp):
+    """The same literals where the GPU tests run: the host there takes the SSE4.2 ``crc32`` path."""
+    _pinned_vectors()
+
+
+def _pinned_vectors():
     assert crc32c(b"xyz") == "25236885"
     assert crc32c(b"abcd") == "92c80a31"
     assert crc32c(b"ef") == "6bb2dff5"

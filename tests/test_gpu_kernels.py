@@ -53,6 +53,36 @@ def test_digest_matches_oracle(gpu_engine, oracle, oracle_c):
         assert h == oracle.tensor_digest_bytes(b.tobytes()), b.size
 
 
+def test_verify_plan_repeats_match_one_shot_calls(gpu_engine, oracle, oracle_c):
+    """Buffers lowered once (the reference caches its descriptor lists, refit/reshard/receiver.py:787-801):
+    every run must give what the one-shot calls and the oracle give, also after the bytes changed and
+    on another stream; the accumulators a run leaves behind must not leak into the next."""
+    rng = np.random.default_rng(15)
+    sizes = [0, 1, 3, 16, 4097, 65536 + 4096 * 3 + 9, 17 * 4096 + 2, (1 << 21) + 5]
+    bufs = [rng.integers(0, 256, n, dtype=np.uint8) for n in sizes]
+    base = torch.from_numpy(np.concatenate([np.zeros(3, np.uint8)] + bufs)).cuda()  # views at odd offsets
+    dev, pos = [], 3
+    for b in bufs:
+        dev.append(base[pos: pos + b.size])
+        pos += b.size
+    plan = gpu_engine.verify_plan(dev)
+    side = torch.cuda.Stream()
+    for rep in range(3):
+        want_c = [oracle_c.checksum32(b) for b in bufs]
+        want_d = [oracle.tensor_digest_bytes(b.tobytes()) for b in bufs]
+        stream = side.cuda_stream if rep == 1 else 0
+        torch.cuda.synchronize()
+        assert plan.checksums(stream=stream) == want_c == gpu_engine.checksum32(dev)
+        assert plan.digests(stream=stream) == want_d == gpu_engine.digest(dev)
+        for b, d in zip(bufs, dev):  # new bytes at the same addresses
+            if b.size:
+                b[b.size // 2] ^= 0x5A
+                d[b.size // 2] ^= 0x5A
+    plan.close()
+    empty = gpu_engine.verify_plan([])
+    assert empty.checksums() == [] and empty.digests() == []
+
+
 def test_digest_reference_invariants_on_device(gpu_engine, oracle):
     a = np.arange(8192, dtype=np.int32)
     b = a.copy()

@@ -25,15 +25,21 @@ def test_families_match_oracle(name, gpu_engine, gpu_engine_band, oracle, tmp_pa
         rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=ep_rank, param_dtype=param_dtype)
         want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
         ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
-        for mode in ("ingest", "ingest_band", "resident"):
+        # ingest: contiguous pieces of every size copied straight to their final address; ingest_bounce: every
+        # byte through the bounce slot and the kernel; ingest_band: 64 KiB slots, row bands gathered on the device
+        for mode in ("ingest", "ingest_bounce", "ingest_band", "resident"):
             eng = gpu_engine_band if mode == "ingest_band" else gpu_engine
             dst = eng.allocate(plan, fill=0xAB)
             if mode == "resident":
                 eng.execute_resident(plan, _stage_files(ck), dst)
             else:
-                stats = eng.execute(plan, dst)
+                eng.set_direct_placement({"ingest": 1, "ingest_bounce": -1}.get(mode, 0))
+                try:
+                    stats = eng.execute(plan, dst)
+                finally:
+                    eng.set_direct_placement(0)
                 assert stats["placed_bytes"] == sum(p.nbytes for p in plan.params)
-                if mode == "ingest":  # packed on the host: nothing but placed bytes (times the cast factor) is read
+                if mode != "ingest_band":  # packed on the host: nothing but placed bytes (times the cast factor) is read
                     assert stats["file_bytes"] == sum(p.nbytes for p in plan.params) * ratio
             sums = eng.checksums(plan)
             for p, d, s in zip(plan.params, dst, sums):
