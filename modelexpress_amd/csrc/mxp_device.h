@@ -95,9 +95,12 @@ constexpr uint32_t kDigestRowWords = 1024;   // 4 KiB rows
 constexpr uint32_t kDigestRowsPerBlock = 32; // 128 KiB per workgroup, two rows per wavefront
 
 // ---- launch wrappers (mxp_kernels.hip) -------------------------------------
+// `zero_dev` / `zero_words`: 32-bit words the launch also clears (its first workgroup does), e.g. the
+// accumulators of the launch after it; they must not overlap anything this launch reads or adds to.
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
-                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only = false);
+                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only = false,
+                        uint32_t* zero_dev = nullptr, uint32_t zero_words = 0);
 // launch_place that also accumulates the tensor_digest sums of the bytes it stores: five 64-bit
 // words per destination buffer (whole-row sum, row-weighted sum, tail sum, tail-weighted sum,
 // ragged-byte sum), added to `digest_sums_dev` (cleared by the caller); `dst_sizes_dev[b]` is
@@ -105,7 +108,7 @@ hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t 
 hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                                const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev,
                                const unsigned long long* dst_sizes_dev, unsigned long long* digest_sums_dev,
-                               uint16_t nan_bits, hipStream_t stream);
+                               uint16_t nan_bits, hipStream_t stream, uint32_t* zero_dev = nullptr, uint32_t zero_words = 0);
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
                          unsigned long long* out_dev, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);

@@ -146,9 +146,17 @@ struct mxp_plan::Lowered {
   // per execute
   DevBuf<void*> dst_bases;
   DevBuf<const void*> src_bases;
-  DevBuf<uint32_t> sums;
+  // Accumulators, two sets: a launch adds to one set and clears the other one on its way, so the
+  // next launch finds zeros without a clearing launch of its own.  One set = [checksum per parameter]
+  // [five 64-bit digest sums per parameter].  `clean[s]` = the host knows set s holds zeros.
+  DevBuf<uint32_t> acc;
+  size_t acc_stride = 0, acc_digest_off = 0, acc_words = 0;  // in 32-bit words
+  int cur = 0;
+  bool clean[2] = {false, false};
+  bool single_set = false;  // a launch of this plan was captured into a graph: set 0 only from then on
+  uint32_t* sums(int set) { return acc.p + (size_t)set * acc_stride; }
+  unsigned long long* digest_sums(int set) { return reinterpret_cast<unsigned long long*>(acc.p + (size_t)set * acc_stride + acc_digest_off); }
   DevBuf<unsigned long long> dst_sizes;    // byte size of every parameter (fused digests)
-  DevBuf<unsigned long long> digest_sums;  // five sums per parameter, accumulated by place_digest_kernel
   bool digests_valid = false;              // the last execute accumulated them
   std::vector<void*> dst_host;        // what dst_bases currently holds
   std::vector<const void*> src_host;  // what src_bases currently holds
@@ -472,7 +480,15 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   }
   L->dst_bases.reserve(pl.params.size() ? pl.params.size() : 1);
   L->src_bases.reserve(ck.files.size() ? ck.files.size() : 1);
-  L->sums.reserve(pl.params.size() ? pl.params.size() : 1);
+  {
+    const size_t n = pl.params.size();
+    L->acc_digest_off = align_up(n ? n : 1, 2);        // the 64-bit sums sit on an 8-byte boundary
+    L->acc_words = L->acc_digest_off + 10 * (n ? n : 1);
+    L->acc_stride = align_up(L->acc_words, 64);
+    L->acc.reserve(2 * L->acc_stride);
+    HIP_OK(hipMemset(L->acc.p, 0, 2 * L->acc_stride * sizeof(uint32_t)));
+    L->clean[0] = L->clean[1] = true;
+  }
   L->tab_cap = pl.params.size() + ck.files.size() + 1;
   HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&L->tab_host), L->tab_cap * sizeof(void*), hipHostMallocDefault));
   HIP_OK(hipEventCreateWithFlags(&L->upload_done, hipEventDisableTiming));
@@ -481,7 +497,6 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
     std::vector<unsigned long long> sizes;
     for (const auto& p : pl.params) sizes.push_back(p.nbytes);
     L->dst_sizes.upload(sizes.data(), sizes.size());
-    L->digest_sums.reserve(pl.params.size() ? 5 * pl.params.size() : 1);
   }
   pl.lowered = L.release();
   pl.lowered_free = free_lowered;
@@ -756,10 +771,12 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
   HIP_OK(hipEventRecord(e.caller_ev, caller_stream));
   for (auto st : e.streams) HIP_OK(hipStreamWaitEvent(st, e.caller_ev, 0));
   upload_tables(L, pl, dst_ptrs, nullptr, 0, e.streams[0]);
-  HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, e.streams[0]));
   const bool digests = e.fused_digests;
   L.digests_valid = false;
-  if (digests) HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(L.digest_sums.p), 10 * pl.params.size(), 0u, e.streams[0]));
+  if (!L.clean[L.cur]) HIP_OK(launch_fill_u32(L.sums(L.cur), L.acc_words, 0u, e.streams[0]));
+  L.clean[L.cur] = false;
+  uint32_t* const sums_dev = L.sums(L.cur);
+  unsigned long long* const dsums_dev = L.digest_sums(L.cur);
   HIP_OK(hipStreamSynchronize(e.streams[0]));
   for (auto& s : e.slots) s->submitted = 0;
 
@@ -824,11 +841,11 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
                                 hipMemcpyHostToDevice, st));
         if (digests)
           HIP_OK(launch_place_digest(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
-                                     e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, L.dst_sizes.p, L.digest_sums.p,
+                                     e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, sums_dev, L.dst_sizes.p, dsums_dev,
                                      e.opt.nan_bits, st));
         else
           HIP_OK(launch_place(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
-                              e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, L.sums.p, e.opt.nan_bits, st));
+                              e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, sums_dev, e.opt.nan_bits, st));
         HIP_OK(hipEventRecord(sl.done, st));
         {
           std::lock_guard<std::mutex> lk(sl.mu);
@@ -890,19 +907,36 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
   auto& L = *pl.lowered;
   if (stats) std::memset(stats, 0, sizeof *stats);
   upload_tables(L, pl, dst_ptrs, file_dev_ptrs, ck.files.size(), stream);
-  HIP_OK(launch_fill_u32(L.sums.p, pl.params.size(), 0u, stream));
   L.digests_valid = e.fused_digests;
-  if (e.fused_digests) HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(L.digest_sums.p), 10 * pl.params.size(), 0u, stream));
-  const bool ring_timed = e.timing_on && !stats && !is_capturing(stream);
+  // Accumulators: a launch adds to one set and clears the other for the launch after it; only a set
+  // the host does not know to be zero gets a clearing launch first.  A captured launch is replayed
+  // with fixed arguments at times the host does not see, so from the first capture on the plan keeps
+  // to set 0 and every launch clears it itself: what mxp_plan_checksums reads is then always the
+  // set the last launch or replay wrote.
+  const bool capturing = is_capturing(stream);
+  if (capturing) L.single_set = true;
+  const bool alternate = !L.single_set && L.res_n_work != 0;
+  const int set = alternate ? (L.cur ^ 1) : 0;
+  if (!alternate || !L.clean[set]) HIP_OK(launch_fill_u32(L.sums(set), L.acc_words, 0u, stream));
+  uint32_t* zero_ptr = nullptr;
+  uint32_t zero_n = 0;
+  if (alternate) {
+    zero_ptr = L.sums(set ^ 1);
+    zero_n = (uint32_t)L.acc_words;
+  }
+  const bool ring_timed = e.timing_on && !stats && !capturing;
   const auto& pair = e.timing_ring.empty() ? std::pair<hipEvent_t, hipEvent_t>() : e.timing_ring[e.timing_count % e.timing_ring.size()];
   if (stats) HIP_OK(hipEventRecord(e.ev_a, stream));
   if (ring_timed) HIP_OK(hipEventRecord(pair.first, stream));
   if (e.fused_digests)
-    HIP_OK(launch_place_digest(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
-                               L.dst_sizes.p, L.digest_sums.p, e.opt.nan_bits, stream));
+    HIP_OK(launch_place_digest(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums(set),
+                               L.dst_sizes.p, L.digest_sums(set), e.opt.nan_bits, stream, zero_ptr, zero_n));
   else
-    HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums.p,
-                        e.opt.nan_bits, stream));
+    HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums(set),
+                        e.opt.nan_bits, stream, false, zero_ptr, zero_n));
+  L.cur = set;
+  L.clean[set] = false;
+  L.clean[set ^ 1] = zero_n != 0;
   if (ring_timed) {
     HIP_OK(hipEventRecord(pair.second, stream));
     ++e.timing_count;
@@ -966,7 +1000,7 @@ int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_
     if (n != (int64_t)plan->params.size()) throw Error(MXP_ERR_ARG, "mxp_plan_checksums: n must equal the parameter count");
     HIP_OK(hipSetDevice(engine->opt.device));
     HIP_OK(hipDeviceSynchronize());
-    if (n) HIP_OK(hipMemcpy(out, plan->lowered->sums.p, (size_t)n * 4, hipMemcpyDeviceToHost));
+    if (n) HIP_OK(hipMemcpy(out, plan->lowered->sums(plan->lowered->cur), (size_t)n * 4, hipMemcpyDeviceToHost));
   });
 }
 
@@ -1029,7 +1063,7 @@ int mxp_plan_digests(mxp_engine* engine, mxp_plan* plan, uint8_t* out16, int64_t
     HIP_OK(hipSetDevice(engine->opt.device));
     HIP_OK(hipDeviceSynchronize());
     std::vector<unsigned long long> sums(5 * (size_t)n);
-    if (n) HIP_OK(hipMemcpy(sums.data(), plan->lowered->digest_sums.p, sums.size() * 8, hipMemcpyDeviceToHost));
+    if (n) HIP_OK(hipMemcpy(sums.data(), plan->lowered->digest_sums(plan->lowered->cur), sums.size() * 8, hipMemcpyDeviceToHost));
     for (int64_t i = 0; i < n; ++i) {
       const auto& p = plan->params[(size_t)i];
       if (p.bytes_written != p.nbytes)

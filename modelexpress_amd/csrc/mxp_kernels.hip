@@ -344,7 +344,11 @@ __device__ __forceinline__ void place_body(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
     uint32_t* __restrict__ sums, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes = nullptr,
-    unsigned long long* __restrict__ digest_sums = nullptr) {
+    unsigned long long* __restrict__ digest_sums = nullptr, uint32_t* __restrict__ zero = nullptr, uint32_t zero_words = 0) {
+  // Housekeeping for the launch after this one: its accumulators are cleared here, so it needs no
+  // clearing launch of its own.
+  if (blockIdx.x == 0)
+    for (uint32_t i = threadIdx.x; i < zero_words; i += kPlaceThreads) zero[i] = 0u;
   const WorkItem w = work[blockIdx.x];
   const Seg s = segs[w.seg];
   const uint32_t r0 = w.tile * s.rows_per_tile;
@@ -441,8 +445,8 @@ __device__ __forceinline__ void place_body(
 __global__ __launch_bounds__(kPlaceThreads) void place_kernel(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
-    uint32_t* __restrict__ sums, uint32_t nan_bits) {
-  place_body<false>(segs, work, src_bases, dst_bases, sums, nan_bits);
+    uint32_t* __restrict__ sums, uint32_t nan_bits, uint32_t* __restrict__ zero, uint32_t zero_words) {
+  place_body<false>(segs, work, src_bases, dst_bases, sums, nan_bits, nullptr, nullptr, zero, zero_words);
 }
 
 // place_kernel that also accumulates the tensor_digest sums of every destination buffer
@@ -451,8 +455,8 @@ __global__ __launch_bounds__(kPlaceThreads) void place_digest_kernel(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
     uint32_t* __restrict__ sums, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes,
-    unsigned long long* __restrict__ digest_sums) {
-  place_body<false, true>(segs, work, src_bases, dst_bases, sums, nan_bits, dst_sizes, digest_sums);
+    unsigned long long* __restrict__ digest_sums, uint32_t* __restrict__ zero, uint32_t zero_words) {
+  place_body<false, true>(segs, work, src_bases, dst_bases, sums, nan_bits, dst_sizes, digest_sums, zero, zero_words);
 }
 
 // Read-only variant for batches made of checksum-only segments.
@@ -488,7 +492,8 @@ hipError_t configure_place_kernels() {
 
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
-                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only) {
+                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only,
+                        uint32_t* zero_dev, uint32_t zero_words) {
   if (n_work == 0) return hipSuccess;
   if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
   const uint32_t lds_place = kOnePerCu, lds_csum = kOnePerCu;
@@ -498,18 +503,18 @@ hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t 
     return hipGetLastError();
   }
   hipLaunchKernelGGL(place_kernel, dim3(n_work), dim3(kPlaceThreads), lds_place, stream, segs_dev,
-                     work_dev, src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits);
+                     work_dev, src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits, zero_dev, zero_words);
   return hipGetLastError();
 }
 
 hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                                const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev,
                                const unsigned long long* dst_sizes_dev, unsigned long long* digest_sums_dev,
-                               uint16_t nan_bits, hipStream_t stream) {
+                               uint16_t nan_bits, hipStream_t stream, uint32_t* zero_dev, uint32_t zero_words) {
   if (n_work == 0) return hipSuccess;
   if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
   hipLaunchKernelGGL(place_digest_kernel, dim3(n_work), dim3(kPlaceThreads), kOnePerCu, stream, segs_dev, work_dev,
-                     src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits, dst_sizes_dev, digest_sums_dev);
+                     src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits, dst_sizes_dev, digest_sums_dev, zero_dev, zero_words);
   return hipGetLastError();
 }
 
