@@ -94,24 +94,67 @@ constexpr int kDigestThreads = 1024;
 constexpr uint32_t kDigestRowWords = 1024;   // 4 KiB rows
 constexpr uint32_t kDigestRowsPerBlock = 32; // 128 KiB per workgroup, two rows per wavefront
 
+// Accumulator fan.  Every workgroup ends with one atomic add per accumulator it feeds, and adds to
+// one address are applied one after the other by the memory side: a launch whose workgroups all
+// feed one checksum measured a tenth slower than the same launch without the add.  So each
+// accumulator array is kept in `lanes()` copies, `pitch` elements apart (a 32-bit checksum is one
+// element, a tensor_digest slot is five 64-bit elements), workgroup b adds to copy b & mask, and
+// whoever reads the results adds the copies up (fold_fan): sums mod 2^32 / 2^64 commute.
+// mask == 0 is the plain layout, one copy.
+constexpr uint32_t kFanLanes = 64;
+struct Fan {
+  uint32_t mask = 0, pitch = 0;
+  uint32_t lanes() const { return mask + 1; }
+};
+// Fan for `n_slots` accumulators: copies a multiple of 256 bytes apart, so that the copies of one
+// accumulator fall into different cache lines; tables too large to be worth copying stay plain.
+inline Fan make_fan(uint64_t n_slots) {
+  Fan f;
+  if (n_slots > 16384) {
+    f.pitch = (uint32_t)n_slots;
+    return f;
+  }
+  f.mask = kFanLanes - 1;
+  f.pitch = (uint32_t)((n_slots ? n_slots : 1) + 63) / 64 * 64;
+  return f;
+}
+// Elements (of either kind) the fanned array of `per_slot`-element accumulators holds.
+inline uint64_t fan_elems(const Fan& f, uint32_t per_slot = 1) { return (uint64_t)f.lanes() * f.pitch * per_slot; }
+// out[k] = sum over the copies of element k, k < n (n <= pitch * per_slot).
+template <typename T>
+inline void fold_fan(const T* fanned, const Fan& f, uint32_t per_slot, uint64_t n, T* out) {
+  for (uint64_t k = 0; k < n; ++k) out[k] = 0;
+  for (uint32_t l = 0; l < f.lanes(); ++l) {
+    const T* lane = fanned + (uint64_t)l * f.pitch * per_slot;
+    for (uint64_t k = 0; k < n; ++k) out[k] += lane[k];
+  }
+}
+
 // ---- launch wrappers (mxp_kernels.hip) -------------------------------------
-// `zero_dev` / `zero_words`: 32-bit words the launch also clears (its first workgroup does), e.g. the
-// accumulators of the launch after it; they must not overlap anything this launch reads or adds to.
+// `sums_dev` is fanned by `fan`.  `zero_dev` / `zero_words`: 32-bit words the launch also clears
+// (spread over its workgroups), e.g. the accumulators of the launch after it; they must not overlap
+// anything this launch reads or adds to.
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
-                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only = false,
+                        uint32_t* sums_dev, Fan fan, uint16_t nan_bits, hipStream_t stream, bool checksum_only = false,
                         uint32_t* zero_dev = nullptr, uint32_t zero_words = 0);
 // launch_place that also accumulates the tensor_digest sums of the bytes it stores: five 64-bit
 // words per destination buffer (whole-row sum, row-weighted sum, tail sum, tail-weighted sum,
-// ragged-byte sum), added to `digest_sums_dev` (cleared by the caller); `dst_sizes_dev[b]` is
-// the byte size of destination buffer b, segment offsets are offsets inside their buffer.
+// ragged-byte sum), added to `digest_sums_dev` (cleared by the caller, fanned by `fan` with five
+// elements per slot); `dst_sizes_dev[b]` is the byte size of destination buffer b, segment offsets
+// are offsets inside their buffer.
 hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
-                               const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev,
+                               const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev, Fan fan,
                                const unsigned long long* dst_sizes_dev, unsigned long long* digest_sums_dev,
                                uint16_t nan_bits, hipStream_t stream, uint32_t* zero_dev = nullptr, uint32_t zero_words = 0);
+// `out_dev` is fanned by `fan` with five 64-bit elements per slot (DigestJob::out_slot counts elements).
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
-                         unsigned long long* out_dev, hipStream_t stream);
+                         unsigned long long* out_dev, Fan fan, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);
+// Device-side fold_fan: out_dev[k] = sum over the copies of element k, k < n; with `clear` the
+// elements read are left at zero.  T is uint32_t or unsigned long long.
+template <typename T>
+hipError_t launch_fold_fan(T* fanned_dev, Fan fan, uint32_t per_slot, uint64_t n, T* out_dev, bool clear, hipStream_t stream);
 
 // Batched 2-D transpose (mxp_permute.hip).  "i" = the destination's innermost dimension,
 // "j" = the source's innermost dimension; strides are in elements.
@@ -157,8 +200,9 @@ struct alignas(16) TransposeItem {
 hipError_t configure_place_kernels();
 // `elem_size` is the source element; `op` is kOpCopy or a conversion whose source element it is
 // (dj, batch_dstride and the checksum positions then count destination elements / bytes).
+// `sum_out` (may be null) is one checksum accumulator fanned by `fan`.
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size, uint32_t op,
-                            uint32_t nan_bits, uint32_t* sum_out, hipStream_t stream);
+                            uint32_t nan_bits, uint32_t* sum_out, Fan fan, hipStream_t stream);
 // `n_items` transposes of one (elem_size, op, waves) in a launch of `total_tiles` workgroups; the
 // host checks each descriptor as launch_transpose would (transpose_desc_ok).
 hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_items, uint64_t total_tiles, uint32_t waves,

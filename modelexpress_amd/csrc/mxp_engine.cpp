@@ -148,11 +148,16 @@ struct mxp_plan::Lowered {
   DevBuf<const void*> src_bases;
   // Accumulators, two sets: a launch adds to one set and clears the other one on its way, so the
   // next launch finds zeros without a clearing launch of its own.  One set = [checksum per parameter]
-  // [five 64-bit digest sums per parameter].  `clean[s]` = the host knows set s holds zeros.
+  // [five 64-bit digest sums per parameter], both fanned by `fan`.  `clean[s]` = the host knows set s
+  // holds zeros; `digest_used[s]` = a launch has added digest sums to set s since it was last
+  // cleared (otherwise only the checksums need clearing).
   DevBuf<uint32_t> acc;
+  Fan fan;
   size_t acc_stride = 0, acc_digest_off = 0, acc_words = 0;  // in 32-bit words
   int cur = 0;
   bool clean[2] = {false, false};
+  bool digest_used[2] = {false, false};
+  size_t dirty_words(int set) const { return digest_used[set] ? acc_words : acc_digest_off; }
   bool single_set = false;  // a launch of this plan was captured into a graph: set 0 only from then on
   uint32_t* sums(int set) { return acc.p + (size_t)set * acc_stride; }
   unsigned long long* digest_sums(int set) { return reinterpret_cast<unsigned long long*>(acc.p + (size_t)set * acc_stride + acc_digest_off); }
@@ -482,8 +487,9 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
   L->src_bases.reserve(ck.files.size() ? ck.files.size() : 1);
   {
     const size_t n = pl.params.size();
-    L->acc_digest_off = align_up(n ? n : 1, 2);        // the 64-bit sums sit on an 8-byte boundary
-    L->acc_words = L->acc_digest_off + 10 * (n ? n : 1);
+    L->fan = make_fan(n);
+    L->acc_digest_off = align_up(fan_elems(L->fan), 2);  // the 64-bit sums sit on an 8-byte boundary
+    L->acc_words = L->acc_digest_off + 2 * fan_elems(L->fan, 5);
     L->acc_stride = align_up(L->acc_words, 64);
     L->acc.reserve(2 * L->acc_stride);
     HIP_OK(hipMemset(L->acc.p, 0, 2 * L->acc_stride * sizeof(uint32_t)));
@@ -609,7 +615,7 @@ void ensure_desc(mxp_engine& e, size_t bytes) {
 }
 
 // Runs a batch of boxes whose sources / destinations are raw device pointers.
-// Layout of the descriptor arena: [segs][work][src ptrs][dst ptrs][sums].
+// Layout of the descriptor arena: [segs][work][src ptrs][dst ptrs][checksums, fanned][checksums, folded].
 void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vector<const void*>& srcs,
                const std::vector<void*>& dsts, uint32_t n_sums, uint32_t* sums_out, hipStream_t stream) {
   LowerOptions lo;
@@ -622,26 +628,30 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
   const size_t o_src = align_up(o_work + work.size() * sizeof(WorkItem), 256);
   const size_t o_dst = align_up(o_src + srcs.size() * sizeof(void*), 256);
   const size_t o_sum = align_up(o_dst + dsts.size() * sizeof(void*), 256);
-  const size_t total = align_up(o_sum + (size_t)n_sums * 4, 256);
+  // [checksums, fanned][checksums, folded] follow the uploaded tables; both are written on the device only
+  const Fan fan = sums_out ? make_fan(n_sums) : Fan{};
+  const size_t o_out = align_up(o_sum + (sums_out ? fan_elems(fan) * 4 : 0), 256);
+  const size_t total = align_up(o_out + (size_t)n_sums * 4, 256);
   acquire_arena(e);
   ensure_desc(e, total);
-  std::memset(e.desc_host, 0, total);
   if (!segs.empty()) std::memcpy(e.desc_host + o_segs, segs.data(), segs.size() * sizeof(Seg));
   if (!work.empty()) std::memcpy(e.desc_host + o_work, work.data(), work.size() * sizeof(WorkItem));
   if (!srcs.empty()) std::memcpy(e.desc_host + o_src, srcs.data(), srcs.size() * sizeof(void*));
   if (!dsts.empty()) std::memcpy(e.desc_host + o_dst, dsts.data(), dsts.size() * sizeof(void*));
-  HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, total, hipMemcpyHostToDevice, stream));
+  HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, o_sum, hipMemcpyHostToDevice, stream));
   uint8_t* d = e.desc_dev.p;
+  uint32_t* const fanned = reinterpret_cast<uint32_t*>(d + o_sum);
+  if (sums_out) HIP_OK(launch_fill_u32(fanned, fan_elems(fan), 0u, stream));
   bool checksum_only = !boxes.empty();
   for (const auto& b : boxes) checksum_only = checksum_only && b.op == kOpChecksumOnly;
   HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + o_segs), reinterpret_cast<const WorkItem*>(d + o_work),
                       (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + o_src),
-                      reinterpret_cast<void* const*>(d + o_dst), reinterpret_cast<uint32_t*>(d + o_sum),
-                      e.opt.nan_bits, stream, checksum_only));
+                      reinterpret_cast<void* const*>(d + o_dst), fanned, fan, e.opt.nan_bits, stream, checksum_only));
   if (sums_out && n_sums) {
-    HIP_OK(hipMemcpyAsync(e.desc_host + o_sum, d + o_sum, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(launch_fold_fan(fanned, fan, 1, (uint64_t)n_sums, reinterpret_cast<uint32_t*>(d + o_out), false, stream));
+    HIP_OK(hipMemcpyAsync(e.desc_host + o_out, d + o_out, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
-    std::memcpy(sums_out, e.desc_host + o_sum, (size_t)n_sums * 4);
+    std::memcpy(sums_out, e.desc_host + o_out, (size_t)n_sums * 4);
   }
   release_arena(e, stream);
 }
@@ -773,8 +783,9 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
   upload_tables(L, pl, dst_ptrs, nullptr, 0, e.streams[0]);
   const bool digests = e.fused_digests;
   L.digests_valid = false;
-  if (!L.clean[L.cur]) HIP_OK(launch_fill_u32(L.sums(L.cur), L.acc_words, 0u, e.streams[0]));
+  if (!L.clean[L.cur]) HIP_OK(launch_fill_u32(L.sums(L.cur), L.dirty_words(L.cur), 0u, e.streams[0]));
   L.clean[L.cur] = false;
+  L.digest_used[L.cur] = digests;
   uint32_t* const sums_dev = L.sums(L.cur);
   unsigned long long* const dsums_dev = L.digest_sums(L.cur);
   HIP_OK(hipStreamSynchronize(e.streams[0]));
@@ -841,11 +852,11 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
                                 hipMemcpyHostToDevice, st));
         if (digests)
           HIP_OK(launch_place_digest(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
-                                     e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, sums_dev, L.dst_sizes.p, dsums_dev,
+                                     e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, sums_dev, L.fan, L.dst_sizes.p, dsums_dev,
                                      e.opt.nan_bits, st));
         else
           HIP_OK(launch_place(L.ing_segs.p + ch.seg_begin, L.ing_work.p + ch.work_begin, ch.work_count,
-                              e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, sums_dev, e.opt.nan_bits, st));
+                              e.slot_ptrs.p + (c % n_slots), L.dst_bases.p, sums_dev, L.fan, e.opt.nan_bits, st));
         HIP_OK(hipEventRecord(sl.done, st));
         {
           std::lock_guard<std::mutex> lk(sl.mu);
@@ -917,22 +928,26 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
   if (capturing) L.single_set = true;
   const bool alternate = !L.single_set && L.res_n_work != 0;
   const int set = alternate ? (L.cur ^ 1) : 0;
-  if (!alternate || !L.clean[set]) HIP_OK(launch_fill_u32(L.sums(set), L.acc_words, 0u, stream));
+  // (a captured clearing launch runs before every replay: it covers what this launch adds to as well)
+  if (!alternate || !L.clean[set])
+    HIP_OK(launch_fill_u32(L.sums(set), L.digest_used[set] || e.fused_digests ? L.acc_words : L.acc_digest_off, 0u, stream));
   uint32_t* zero_ptr = nullptr;
   uint32_t zero_n = 0;
   if (alternate) {
     zero_ptr = L.sums(set ^ 1);
-    zero_n = (uint32_t)L.acc_words;
+    zero_n = (uint32_t)L.dirty_words(set ^ 1);
+    L.digest_used[set ^ 1] = false;
   }
+  L.digest_used[set] = e.fused_digests;
   const bool ring_timed = e.timing_on && !stats && !capturing;
   const auto& pair = e.timing_ring.empty() ? std::pair<hipEvent_t, hipEvent_t>() : e.timing_ring[e.timing_count % e.timing_ring.size()];
   if (stats) HIP_OK(hipEventRecord(e.ev_a, stream));
   if (ring_timed) HIP_OK(hipEventRecord(pair.first, stream));
   if (e.fused_digests)
-    HIP_OK(launch_place_digest(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums(set),
+    HIP_OK(launch_place_digest(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums(set), L.fan,
                                L.dst_sizes.p, L.digest_sums(set), e.opt.nan_bits, stream, zero_ptr, zero_n));
   else
-    HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums(set),
+    HIP_OK(launch_place(L.res_segs.p, L.res_work.p, L.res_n_work, L.src_bases.p, L.dst_bases.p, L.sums(set), L.fan,
                         e.opt.nan_bits, stream, false, zero_ptr, zero_n));
   L.cur = set;
   L.clean[set] = false;
@@ -1000,7 +1015,10 @@ int mxp_plan_checksums(mxp_engine* engine, mxp_plan* plan, uint32_t* out, int64_
     if (n != (int64_t)plan->params.size()) throw Error(MXP_ERR_ARG, "mxp_plan_checksums: n must equal the parameter count");
     HIP_OK(hipSetDevice(engine->opt.device));
     HIP_OK(hipDeviceSynchronize());
-    if (n) HIP_OK(hipMemcpy(out, plan->lowered->sums(plan->lowered->cur), (size_t)n * 4, hipMemcpyDeviceToHost));
+    auto& L = *plan->lowered;
+    std::vector<uint32_t> fanned(fan_elems(L.fan));
+    HIP_OK(hipMemcpy(fanned.data(), L.sums(L.cur), fanned.size() * 4, hipMemcpyDeviceToHost));
+    fold_fan(fanned.data(), L.fan, 1, (uint64_t)n, out);
   });
 }
 
@@ -1062,8 +1080,10 @@ int mxp_plan_digests(mxp_engine* engine, mxp_plan* plan, uint8_t* out16, int64_t
     if (n != (int64_t)plan->params.size()) throw Error(MXP_ERR_ARG, "mxp_plan_digests: n must equal the parameter count");
     HIP_OK(hipSetDevice(engine->opt.device));
     HIP_OK(hipDeviceSynchronize());
-    std::vector<unsigned long long> sums(5 * (size_t)n);
-    if (n) HIP_OK(hipMemcpy(sums.data(), plan->lowered->digest_sums(plan->lowered->cur), sums.size() * 8, hipMemcpyDeviceToHost));
+    auto& L = *plan->lowered;
+    std::vector<unsigned long long> fanned(fan_elems(L.fan, 5)), sums(5 * (size_t)n + 1);
+    HIP_OK(hipMemcpy(fanned.data(), L.digest_sums(L.cur), fanned.size() * 8, hipMemcpyDeviceToHost));
+    fold_fan(fanned.data(), L.fan, 5, 5 * (uint64_t)n, sums.data());
     for (int64_t i = 0; i < n; ++i) {
       const auto& p = plan->params[(size_t)i];
       if (p.bytes_written != p.nbytes)
@@ -1162,7 +1182,7 @@ int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uin
     HIP_OK(hipMemcpyAsync(d + kStaticOffPtrs, h + kStaticOffPtrs, kStaticOffSums - kStaticOffPtrs + (size_t)n * 4, hipMemcpyHostToDevice, stream));
     HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + kStaticOffSegs), reinterpret_cast<const WorkItem*>(d + kStaticOffWork),
                         (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + kStaticOffPtrs), nullptr,
-                        reinterpret_cast<uint32_t*>(d + kStaticOffSums), e.opt.nan_bits, stream, true));
+                        reinterpret_cast<uint32_t*>(d + kStaticOffSums), Fan{}, e.opt.nan_bits, stream, true));  // one copy: the scratch is full
     HIP_OK(hipMemcpyAsync(h + kStaticOffSums, d + kStaticOffSums, (size_t)n * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
     std::memcpy(out, sums, (size_t)n * 4);
@@ -1465,17 +1485,18 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
 
 void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hipStream_t stream) {
   uint32_t* sum_dev = nullptr;
+  const Fan fan = make_fan(1);
   if (checksum) {
     acquire_arena(e);
-    ensure_desc(e, 256);
+    ensure_desc(e, fan_elems(fan) * 4);
     sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
-    HIP_OK(launch_fill_u32(sum_dev, 1, 0u, stream));
+    HIP_OK(launch_fill_u32(sum_dev, fan_elems(fan), 0u, stream));
   }
-  HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, e.opt.nan_bits, sum_dev, stream));
+  HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, e.opt.nan_bits, sum_dev, fan, stream));
   if (checksum) {
-    HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, fan_elems(fan) * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
-    std::memcpy(checksum, e.desc_host, 4);
+    fold_fan(reinterpret_cast<const uint32_t*>(e.desc_host), fan, 1, 1, checksum);
     release_arena(e, stream);
   }
 }
@@ -1633,16 +1654,19 @@ struct mxp_verify_plan {
   int device = 0;
   int64_t n = 0;
   std::vector<uint64_t> nbytes;
-  DevBuf<uint8_t> tables;  // [segments][work items][source pointers][checksums][digest jobs][digest sums]
+  // [segments][work items][source pointers][checksums, fanned][digest jobs][digest sums, fanned]
+  DevBuf<uint8_t> tables;
+  Fan fan;
   size_t o_work = 0, o_src = 0, o_sums = 0, o_jobs = 0, o_dsums = 0;
   uint32_t n_work = 0, n_blocks = 0;
-  uint8_t* host = nullptr;  // pinned: [checksums][digest sums]
-  hipEvent_t done = nullptr;     // results have reached `host`
-  hipEvent_t cleared = nullptr;  // the accumulators are zero again
+  // pinned: [checksums][digest sums]; the kernel that adds the fanned copies up stores its results
+  // here directly (`host_dev` is the device's address of the block), so no copy follows it
+  uint8_t* host = nullptr;
+  uint8_t* host_dev = nullptr;
+  hipEvent_t cleared = nullptr;  // the results are in `host` and the accumulators are zero again
   bool cleared_rec = false;
   ~mxp_verify_plan() {
     if (host) (void)hipHostFree(host);
-    if (done) (void)hipEventDestroy(done);
     if (cleared) (void)hipEventDestroy(cleared);
   }
 };
@@ -1691,16 +1715,17 @@ int mxp_verify_plan_create(mxp_engine* engine, const void* const* ptrs, const ui
     vp->o_work = align_up(segs.size() * sizeof(Seg), 256);
     vp->o_src = align_up(vp->o_work + work.size() * sizeof(WorkItem), 256);
     vp->o_sums = align_up(vp->o_src + srcs.size() * sizeof(void*), 256);
-    vp->o_jobs = align_up(vp->o_sums + (size_t)n * 4, 256);
+    vp->fan = make_fan((uint64_t)n);
+    vp->o_jobs = align_up(vp->o_sums + fan_elems(vp->fan) * 4, 256);
     vp->o_dsums = align_up(vp->o_jobs + jobs.size() * sizeof(DigestJob), 256);
-    std::vector<uint8_t> host(align_up(vp->o_dsums + (size_t)n * 40, 256) + 256, 0);  // accumulators start at zero
+    std::vector<uint8_t> host(align_up(vp->o_dsums + fan_elems(vp->fan, 5) * 8, 256), 0);  // accumulators start at zero
     if (!segs.empty()) std::memcpy(host.data(), segs.data(), segs.size() * sizeof(Seg));
     if (!work.empty()) std::memcpy(host.data() + vp->o_work, work.data(), work.size() * sizeof(WorkItem));
     if (!srcs.empty()) std::memcpy(host.data() + vp->o_src, srcs.data(), srcs.size() * sizeof(void*));
     if (!jobs.empty()) std::memcpy(host.data() + vp->o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
     vp->tables.upload(host.data(), host.size());
     HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&vp->host), (size_t)(n ? n : 1) * 44 + 16, hipHostMallocDefault));
-    HIP_OK(hipEventCreateWithFlags(&vp->done, hipEventDisableTiming));
+    HIP_OK(hipHostGetDevicePointer(reinterpret_cast<void**>(&vp->host_dev), vp->host, 0));
     HIP_OK(hipEventCreateWithFlags(&vp->cleared, hipEventDisableTiming));
     *out = vp.release();
   });
@@ -1717,14 +1742,13 @@ int mxp_verify_plan_checksums(mxp_engine* engine, mxp_verify_plan* plan, uint32_
     uint32_t* sums = reinterpret_cast<uint32_t*>(d + plan->o_sums);
     if (plan->cleared_rec) HIP_OK(hipStreamWaitEvent(stream, plan->cleared, 0));  // a run on another stream than the last
     HIP_OK(launch_place(reinterpret_cast<const Seg*>(d), reinterpret_cast<const WorkItem*>(d + plan->o_work), plan->n_work,
-                        reinterpret_cast<const void* const*>(d + plan->o_src), nullptr, sums, engine->opt.nan_bits, stream, true));
-    HIP_OK(hipMemcpyAsync(plan->host, sums, (size_t)plan->n * 4, hipMemcpyDeviceToHost, stream));
-    HIP_OK(hipEventRecord(plan->done, stream));
-    // the accumulators are cleared for the next run behind the result copy, off the caller's path
-    HIP_OK(launch_fill_u32(sums, (uint64_t)plan->n, 0u, stream));
+                        reinterpret_cast<const void* const*>(d + plan->o_src), nullptr, sums, plan->fan, engine->opt.nan_bits, stream,
+                        true));
+    // the copies are added up on the device, which leaves them cleared for the next run
+    HIP_OK(launch_fold_fan(sums, plan->fan, 1, (uint64_t)plan->n, reinterpret_cast<uint32_t*>(plan->host_dev), true, stream));
     HIP_OK(hipEventRecord(plan->cleared, stream));
     plan->cleared_rec = true;
-    HIP_OK(hipEventSynchronize(plan->done));
+    HIP_OK(hipEventSynchronize(plan->cleared));
     std::memcpy(out, plan->host, (size_t)plan->n * 4);
   });
 }
@@ -1739,15 +1763,15 @@ int mxp_verify_plan_digests(mxp_engine* engine, mxp_verify_plan* plan, uint8_t* 
     uint8_t* d = plan->tables.p;
     unsigned long long* dsums = reinterpret_cast<unsigned long long*>(d + plan->o_dsums);
     if (plan->cleared_rec) HIP_OK(hipStreamWaitEvent(stream, plan->cleared, 0));
-    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(d + plan->o_jobs), (uint32_t)plan->n, plan->n_blocks, dsums, stream));
-    uint8_t* h = plan->host + (size_t)plan->n * 4;  // 8-byte aligned: n * 4 with n * 40 behind it needs n even or a pad
-    h = reinterpret_cast<uint8_t*>((reinterpret_cast<uintptr_t>(h) + 7u) & ~(uintptr_t)7u);
-    HIP_OK(hipMemcpyAsync(h, dsums, (size_t)plan->n * 40, hipMemcpyDeviceToHost, stream));
-    HIP_OK(hipEventRecord(plan->done, stream));
-    HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(dsums), (uint64_t)plan->n * 10, 0u, stream));
+    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(d + plan->o_jobs), (uint32_t)plan->n, plan->n_blocks, dsums, plan->fan,
+                         stream));
+    const size_t h_off = align_up((size_t)plan->n * 4, 8);  // the 64-bit sums follow the checksums
+    const uint8_t* h = plan->host + h_off;
+    HIP_OK(launch_fold_fan(dsums, plan->fan, 5, 5 * (uint64_t)plan->n, reinterpret_cast<unsigned long long*>(plan->host_dev + h_off), true,
+                           stream));
     HIP_OK(hipEventRecord(plan->cleared, stream));
     plan->cleared_rec = true;
-    HIP_OK(hipEventSynchronize(plan->done));
+    HIP_OK(hipEventSynchronize(plan->cleared));
     const uint64_t* sums = reinterpret_cast<const uint64_t*>(h);
     for (int64_t k = 0; k < plan->n; ++k) {
       const uint64_t nb = plan->nbytes[(size_t)k];
@@ -1878,10 +1902,10 @@ int mxp_view_plan_run(mxp_engine* engine, mxp_view_plan* plan, void* stream_v) {
       uint8_t* d = plan->tables.p;
       HIP_OK(launch_place(reinterpret_cast<const Seg*>(d), reinterpret_cast<const WorkItem*>(d + plan->o_work), plan->n_work,
                           reinterpret_cast<const void* const*>(d + plan->o_src), reinterpret_cast<void* const*>(d + plan->o_dst),
-                          nullptr, engine->opt.nan_bits, stream));
+                          nullptr, Fan{}, engine->opt.nan_bits, stream));
     }
     for (const auto& t : plan->singles)
-      HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, engine->opt.nan_bits, nullptr, stream));
+      HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, engine->opt.nan_bits, nullptr, Fan{}, stream));
     for (const auto& g : plan->groups)
       HIP_OK(launch_transpose_batch(plan->items.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
                                     engine->opt.nan_bits, stream));
@@ -1980,15 +2004,19 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
     }
     if (blocks > 0x7FFFFFFFull) throw Error(MXP_ERR_ARG, "mxp_digest: batch too large for one launch");
     const size_t o_jobs = 0;
-    const size_t o_out = align_up(jobs.size() * sizeof(DigestJob), 256);
+    // [jobs][digest sums, fanned][digest sums, folded]: only the jobs are uploaded
+    const Fan fan = make_fan((uint64_t)n);
+    const size_t o_fan = align_up(jobs.size() * sizeof(DigestJob), 256);
+    const size_t o_out = align_up(o_fan + fan_elems(fan, 5) * 8, 256);
     const size_t total = o_out + (size_t)n * 5 * 8;
     acquire_arena(e);
     ensure_desc(e, total);
-    std::memset(e.desc_host, 0, total);
     std::memcpy(e.desc_host + o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
-    HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, total, hipMemcpyHostToDevice, stream));
-    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(e.desc_dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks,
-                         reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_out), stream));
+    HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, jobs.size() * sizeof(DigestJob), hipMemcpyHostToDevice, stream));
+    unsigned long long* const fanned = reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_fan);
+    HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(fanned), 2 * fan_elems(fan, 5), 0u, stream));
+    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(e.desc_dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks, fanned, fan, stream));
+    HIP_OK(launch_fold_fan(fanned, fan, 5, 5 * (uint64_t)n, reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_out), false, stream));
     HIP_OK(hipMemcpyAsync(e.desc_host + o_out, e.desc_dev.p + o_out, (size_t)n * 5 * 8, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
     release_arena(e, stream);

@@ -343,12 +343,13 @@ template <bool CHECKSUM_ONLY, bool DIGEST = false>
 __device__ __forceinline__ void place_body(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
-    uint32_t* __restrict__ sums, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes = nullptr,
+    uint32_t* __restrict__ sums, Fan fan, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes = nullptr,
     unsigned long long* __restrict__ digest_sums = nullptr, uint32_t* __restrict__ zero = nullptr, uint32_t zero_words = 0) {
-  // Housekeeping for the launch after this one: its accumulators are cleared here, so it needs no
-  // clearing launch of its own.
-  if (blockIdx.x == 0)
-    for (uint32_t i = threadIdx.x; i < zero_words; i += kPlaceThreads) zero[i] = 0u;
+  // Housekeeping for the launch after this one: its accumulators are cleared here, a slice per
+  // workgroup, so it needs no clearing launch of its own.
+  for (uint64_t i = (uint64_t)blockIdx.x * kPlaceThreads + threadIdx.x; i < zero_words; i += (uint64_t)gridDim.x * kPlaceThreads) zero[i] = 0u;
+  // This workgroup's copy of the accumulators.
+  const uint32_t lane_first = (blockIdx.x & fan.mask) * fan.pitch;
   const WorkItem w = work[blockIdx.x];
   const Seg s = segs[w.seg];
   const uint32_t r0 = w.tile * s.rows_per_tile;
@@ -420,12 +421,12 @@ __device__ __forceinline__ void place_body(
       unsigned long long t = 0;
 #pragma unroll
       for (int k = 0; k < kPlaceThreads / 64; ++k) t += dpart[k][threadIdx.x];
-      if (t) atomicAdd(&digest_sums[5ull * s.dst_buf + threadIdx.x], t);
+      if (t) atomicAdd(&digest_sums[5ull * (lane_first + s.dst_buf) + threadIdx.x], t);
     } else if (threadIdx.x == 64 && s.csum_slot != 0xFFFFFFFFu) {
       uint32_t t = 0;
 #pragma unroll
       for (int k = 0; k < kPlaceThreads / 64; ++k) t += part[k];
-      atomicAdd(&sums[s.csum_slot], t);
+      atomicAdd(&sums[lane_first + s.csum_slot], t);
     }
   } else if (s.csum_slot != 0xFFFFFFFFu) {
     __shared__ uint32_t part[kPlaceThreads / 64];
@@ -436,7 +437,7 @@ __device__ __forceinline__ void place_body(
       uint32_t t = 0;
 #pragma unroll
       for (int k = 0; k < kPlaceThreads / 64; ++k) t += part[k];
-      atomicAdd(&sums[s.csum_slot], t);
+      atomicAdd(&sums[lane_first + s.csum_slot], t);
     }
   }
 }
@@ -445,8 +446,8 @@ __device__ __forceinline__ void place_body(
 __global__ __launch_bounds__(kPlaceThreads) void place_kernel(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
-    uint32_t* __restrict__ sums, uint32_t nan_bits, uint32_t* __restrict__ zero, uint32_t zero_words) {
-  place_body<false>(segs, work, src_bases, dst_bases, sums, nan_bits, nullptr, nullptr, zero, zero_words);
+    uint32_t* __restrict__ sums, Fan fan, uint32_t nan_bits, uint32_t* __restrict__ zero, uint32_t zero_words) {
+  place_body<false>(segs, work, src_bases, dst_bases, sums, fan, nan_bits, nullptr, nullptr, zero, zero_words);
 }
 
 // place_kernel that also accumulates the tensor_digest sums of every destination buffer
@@ -454,23 +455,26 @@ __global__ __launch_bounds__(kPlaceThreads) void place_kernel(
 __global__ __launch_bounds__(kPlaceThreads) void place_digest_kernel(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
     const void* const* __restrict__ src_bases, void* const* __restrict__ dst_bases,
-    uint32_t* __restrict__ sums, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes,
+    uint32_t* __restrict__ sums, Fan fan, uint32_t nan_bits, const unsigned long long* __restrict__ dst_sizes,
     unsigned long long* __restrict__ digest_sums, uint32_t* __restrict__ zero, uint32_t zero_words) {
-  place_body<false, true>(segs, work, src_bases, dst_bases, sums, nan_bits, dst_sizes, digest_sums, zero, zero_words);
+  place_body<false, true>(segs, work, src_bases, dst_bases, sums, fan, nan_bits, dst_sizes, digest_sums, zero, zero_words);
 }
 
 // Read-only variant for batches made of checksum-only segments.
 __global__ __launch_bounds__(kPlaceThreads) void checksum_kernel(
     const Seg* __restrict__ segs, const WorkItem* __restrict__ work,
-    const void* const* __restrict__ src_bases, uint32_t* __restrict__ sums) {
-  place_body<true>(segs, work, src_bases, nullptr, sums, 0u);
+    const void* const* __restrict__ src_bases, uint32_t* __restrict__ sums, Fan fan) {
+  place_body<true>(segs, work, src_bases, nullptr, sums, fan, 0u);
 }
 
 // One workgroup per compute unit: a unit then alternates between one 128 KiB read burst and
-// one 128 KiB write burst instead of mixing the two.  Two resident workgroups measured 4-10%
+// one 128 KiB write burst instead of mixing the two.  Two resident workgroups measured 3-5%
 // slower on every configuration.  The limit is imposed with an otherwise unused dynamic LDS
 // allocation of more than half a unit's LDS, which needs the attribute below once per device.
+// A launch that only reads (checksum_kernel) is the other way round: two resident workgroups, one
+// loading while the other adds up, read a tenth faster than one.
 constexpr uint32_t kOnePerCu = 96 * 1024;
+constexpr uint32_t kTwoPerCu = 48 * 1024;
 
 hipError_t configure_place_kernels() {
   static std::atomic<uint64_t> configured{0};  // bit per device
@@ -492,29 +496,29 @@ hipError_t configure_place_kernels() {
 
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
-                        uint32_t* sums_dev, uint16_t nan_bits, hipStream_t stream, bool checksum_only,
+                        uint32_t* sums_dev, Fan fan, uint16_t nan_bits, hipStream_t stream, bool checksum_only,
                         uint32_t* zero_dev, uint32_t zero_words) {
   if (n_work == 0) return hipSuccess;
   if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
-  const uint32_t lds_place = kOnePerCu, lds_csum = kOnePerCu;
+  const uint32_t lds_place = kOnePerCu, lds_csum = kTwoPerCu;
   if (checksum_only) {
     hipLaunchKernelGGL(checksum_kernel, dim3(n_work), dim3(kPlaceThreads), lds_csum, stream, segs_dev, work_dev,
-                       src_bases_dev, sums_dev);
+                       src_bases_dev, sums_dev, fan);
     return hipGetLastError();
   }
   hipLaunchKernelGGL(place_kernel, dim3(n_work), dim3(kPlaceThreads), lds_place, stream, segs_dev,
-                     work_dev, src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits, zero_dev, zero_words);
+                     work_dev, src_bases_dev, dst_bases_dev, sums_dev, fan, (uint32_t)nan_bits, zero_dev, zero_words);
   return hipGetLastError();
 }
 
 hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
-                               const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev,
+                               const void* const* src_bases_dev, void* const* dst_bases_dev, uint32_t* sums_dev, Fan fan,
                                const unsigned long long* dst_sizes_dev, unsigned long long* digest_sums_dev,
                                uint16_t nan_bits, hipStream_t stream, uint32_t* zero_dev, uint32_t zero_words) {
   if (n_work == 0) return hipSuccess;
   if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
   hipLaunchKernelGGL(place_digest_kernel, dim3(n_work), dim3(kPlaceThreads), kOnePerCu, stream, segs_dev, work_dev,
-                     src_bases_dev, dst_bases_dev, sums_dev, (uint32_t)nan_bits, dst_sizes_dev, digest_sums_dev, zero_dev, zero_words);
+                     src_bases_dev, dst_bases_dev, sums_dev, fan, (uint32_t)nan_bits, dst_sizes_dev, digest_sums_dev, zero_dev, zero_words);
   return hipGetLastError();
 }
 
@@ -577,7 +581,7 @@ __device__ __forceinline__ void digest_rows(const uint8_t* __restrict__ p, uint6
 }
 
 __global__ __launch_bounds__(kDigestThreads) void digest_kernel(
-    const DigestJob* __restrict__ jobs, uint32_t n_jobs, unsigned long long* __restrict__ out) {
+    const DigestJob* __restrict__ jobs, uint32_t n_jobs, unsigned long long* __restrict__ out, Fan fan) {
   // Workgroup-uniform binary search for the job that owns this workgroup.
   uint32_t lo = 0, hi = n_jobs;
   while (hi - lo > 1) {
@@ -628,17 +632,53 @@ __global__ __launch_bounds__(kDigestThreads) void digest_kernel(
     unsigned long long t = 0;
 #pragma unroll
     for (int k = 0; k < kDigestThreads / 64; ++k) t += part[k][threadIdx.x];
-    if (t) atomicAdd(&out[j.out_slot + threadIdx.x], t);
+    if (t) atomicAdd(&out[5ull * ((blockIdx.x & fan.mask) * fan.pitch) + j.out_slot + threadIdx.x], t);
   }
 }
 
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
-                         unsigned long long* out_dev, hipStream_t stream) {
+                         unsigned long long* out_dev, Fan fan, hipStream_t stream) {
   if (n_jobs == 0 || n_blocks == 0) return hipSuccess;
   hipLaunchKernelGGL(digest_kernel, dim3(n_blocks), dim3(kDigestThreads), 0, stream, jobs_dev,
-                     n_jobs, out_dev);
+                     n_jobs, out_dev, fan);
   return hipGetLastError();
 }
+
+// out[k] = sum over the fan's copies of element k (k < n); with `clear`, the elements read are
+// left at zero for the next launch that adds to them.  One wavefront per element: lane l reads
+// copy l (a fan has at most 64 copies), so the loads of an element are all in flight at once.
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) { return wave_sum_u32(v); }
+__device__ __forceinline__ unsigned long long wave_sum(unsigned long long v) { return wave_sum_u64(v); }
+
+template <typename T>
+__global__ __launch_bounds__(256) void fold_fan_kernel(T* __restrict__ fanned, Fan fan, uint32_t per_slot, uint64_t n,
+                                                       T* __restrict__ out, bool clear) {
+  static_assert(kFanLanes <= 64, "one lane of a wavefront per copy");
+  const uint64_t lane_elems = (uint64_t)fan.pitch * per_slot;
+  const uint32_t lane = threadIdx.x & 63u;
+  for (uint64_t k = blockIdx.x * 4ull + (threadIdx.x >> 6); k < n; k += (uint64_t)gridDim.x * 4ull) {
+    T v = 0;
+    if (lane <= fan.mask) {
+      T* p = fanned + lane * lane_elems + k;
+      v = *p;
+      if (clear) *p = 0;
+    }
+    v = wave_sum(v);
+    if (lane == 0) out[k] = v;
+  }
+}
+
+template <typename T>
+hipError_t launch_fold_fan(T* fanned, Fan fan, uint32_t per_slot, uint64_t n, T* out, bool clear, hipStream_t stream) {
+  if (n == 0) return hipSuccess;
+  const uint64_t blocks = (n + 3) / 4;
+  hipLaunchKernelGGL(fold_fan_kernel<T>, dim3((uint32_t)(blocks > 16384 ? 16384 : blocks)), dim3(256), 0, stream, fanned, fan,
+                     per_slot, n, out, clear);
+  return hipGetLastError();
+}
+template hipError_t launch_fold_fan<uint32_t>(uint32_t*, Fan, uint32_t, uint64_t, uint32_t*, bool, hipStream_t);
+template hipError_t launch_fold_fan<unsigned long long>(unsigned long long*, Fan, uint32_t, uint64_t, unsigned long long*, bool,
+                                                        hipStream_t);
 
 // Plain vector-store fill; used instead of a memset node so callers may capture it.
 __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, uint64_t n,

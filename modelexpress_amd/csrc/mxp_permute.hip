@@ -324,7 +324,7 @@ template <int ES, int OP>
 __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __restrict__ src,
                                                               uint8_t* __restrict__ dst,
                                                               const TransposeDesc d, uint32_t nan_bits,
-                                                              uint32_t* __restrict__ sum_out) {
+                                                              uint32_t* __restrict__ sum_out, Fan fan) {
   using S = Sub<ES, OP>;
   __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
 #pragma unroll
       for (int k = 0; k < kWaves; ++k)
         if ((uint32_t)k < d.waves) t += *reinterpret_cast<const uint32_t*>(lds + k * S::kLdsBytes);
-      atomicAdd(sum_out, t);
+      atomicAdd(&sum_out[(blockIdx.x & fan.mask) * fan.pitch], t);
     }
   }
 }
@@ -402,9 +402,10 @@ struct LaunchOne {
   const TransposeDesc& d;
   uint32_t nan_bits;
   uint32_t* sum_out;
+  Fan fan;
   template <int ES, int OP>
   void operator()() const {
-    hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, 0, stream, s, t, d, nan_bits, sum_out);
+    hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, 0, stream, s, t, d, nan_bits, sum_out, fan);
   }
 };
 
@@ -422,11 +423,11 @@ struct LaunchBatch {
 }  // namespace
 
 hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, int elem_size, uint32_t op,
-                            uint32_t nan_bits, uint32_t* sum_out, hipStream_t stream) {
+                            uint32_t nan_bits, uint32_t* sum_out, Fan fan, hipStream_t stream) {
   if (d.n_tiles == 0) return hipSuccess;
   if (!transpose_desc_ok(d)) return hipErrorInvalidValue;
   const LaunchOne one{dim3((uint32_t)d.n_tiles), dim3(d.waves * 64u), stream, static_cast<const uint8_t*>(src),
-                      static_cast<uint8_t*>(dst), d, nan_bits, sum_out};
+                      static_cast<uint8_t*>(dst), d, nan_bits, sum_out, fan};
   if (!with_instance(elem_size, op, one)) return hipErrorInvalidValue;
   return hipGetLastError();
 }
