@@ -157,6 +157,47 @@ def _timed_resident(eng, plan, staged, dst, steps: int, warmup: int) -> dict:
             "kernel_ms": single, "kernel_ms_avg": sum(single) / len(single)}
 
 
+def _pitch_probes(eng, reps: int = 10) -> dict:
+    """What the memory system does with the access shapes of the headline workload, one at a time, through the
+    library's own kernels (``mxp_copy_view`` without a checksum, about 1 GiB written per call): a contiguous
+    copy, the row gathers of the column slices from the checkpoint's power-of-two pitch, and the same
+    gathers from a pitch 256 bytes longer.  Reads alone and writes alone stand beside them."""
+    import torch
+    out = {}
+
+    def timed(fn):
+        fn()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(reps):
+            fn()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / reps
+
+    def entry(ms, moved, **kw):
+        return {**kw, "ms": round(ms, 4), "gbps": round(moved / ms / 1e6, 1), "frac_of_hbm_peak": round(moved / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+
+    for label, mats, rows, row_bytes, pitch in (
+            ("copy_contiguous", 1, 1, 1 << 30, 1 << 30),
+            ("gather_1KiB_rows_pitch_8192 (o_proj slice)", 256, 4096, 1024, 8192),
+            ("gather_1KiB_rows_pitch_8448", 256, 4096, 1024, 8448),
+            ("gather_3584B_rows_pitch_28672 (down_proj slice)", 73, 4096, 3584, 28672),
+            ("gather_3584B_rows_pitch_28928", 73, 4096, 3584, 28928)):
+        a = torch.empty(mats * rows * pitch, dtype=torch.uint8, device="cuda").random_(0, 256)
+        b = torch.empty(mats * rows * row_bytes, dtype=torch.uint8, device="cuda")
+        shape, strides = (mats * rows, row_bytes), (pitch, 1)
+        ms = timed(lambda: eng.copy_view(a, b, shape, 1, src_strides=strides, checksum=False))
+        out[label] = entry(ms, 2 * b.numel(), bytes_written=b.numel(), rows=mats * rows, row_bytes=row_bytes, src_pitch=pitch)
+        if label == "copy_contiguous":
+            vp = eng.verify_plan([b], [b.numel()])
+            out["read_only (checksum32 of 1 GiB, wall per call)"] = entry(timed(vp.checksums), b.numel())
+            vp.close()
+            out["write_only (torch fill_ of 1 GiB)"] = entry(timed(lambda: b.fill_(7)), b.numel())
+        del a, b
+    return out
+
+
 def _segment_classes(eng, ck, plan, rv, staged, dst, tp, rank, cast, steps, warmup) -> dict:
     """Sub-plans over the parameters of one kind each (the other tensors are skipped), launched and timed
     like the whole step.  A class is named after the parameter it writes; its writes share one shape."""
@@ -288,6 +329,9 @@ def main() -> int:
     ap.add_argument("--classes", action="store_true",
                     help="also time each class of segments of the workload as a launch of its own (contiguous row "
                          "blocks, strided column slices, vocabulary slices ...): the breakdown of the step time")
+    ap.add_argument("--probes", action="store_true",
+                    help="also time the workload's access shapes one by one (contiguous copy, the column slices' row "
+                         "gathers from the checkpoint's pitch and from a padded one, reads alone, writes alone)")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the block of the other four configurations that the default run appends")
     ap.add_argument("--seed", type=int, default=20240229)
@@ -381,6 +425,9 @@ def main() -> int:
         # ---- the step broken down by class of segment, each class a launch of its own ----
         if args.classes:
             out["segment_classes"] = _segment_classes(eng, ck, plan, rv, staged, dst, tp, rank, cast, args.steps, args.warmup)
+
+        if args.probes:
+            out["probes"] = _pitch_probes(eng)
 
         # ---- the read-only operators over the finished buffers (1 x bytes each) ----
         sizes = [p.nbytes for p in plan.params]
