@@ -88,6 +88,17 @@ double now_s() {
 }
 uint64_t align_up(uint64_t v, uint64_t a) { return (v + a - 1) / a * a; }
 
+// Waits for `ev` by polling for up to two milliseconds before it blocks: a blocking wait wakes up
+// tens of microseconds after the event, which a caller that waits for a 0.3 ms launch notices.
+hipError_t wait_event_promptly(hipEvent_t ev) {
+  const double t0 = now_s();
+  for (;;) {
+    const hipError_t r = hipEventQuery(ev);
+    if (r != hipErrorNotReady) return r;
+    if (now_s() - t0 > 2e-3) return hipEventSynchronize(ev);
+  }
+}
+
 }  // namespace
 
 // Pieces below this size take the bounce slot by default: a copy call of their own would cost more than it saves.
@@ -1748,7 +1759,7 @@ int mxp_verify_plan_checksums(mxp_engine* engine, mxp_verify_plan* plan, uint32_
     HIP_OK(launch_fold_fan(sums, plan->fan, 1, (uint64_t)plan->n, reinterpret_cast<uint32_t*>(plan->host_dev), true, stream));
     HIP_OK(hipEventRecord(plan->cleared, stream));
     plan->cleared_rec = true;
-    HIP_OK(hipEventSynchronize(plan->cleared));
+    HIP_OK(wait_event_promptly(plan->cleared));
     std::memcpy(out, plan->host, (size_t)plan->n * 4);
   });
 }
@@ -1771,7 +1782,7 @@ int mxp_verify_plan_digests(mxp_engine* engine, mxp_verify_plan* plan, uint8_t* 
                            stream));
     HIP_OK(hipEventRecord(plan->cleared, stream));
     plan->cleared_rec = true;
-    HIP_OK(hipEventSynchronize(plan->cleared));
+    HIP_OK(wait_event_promptly(plan->cleared));
     const uint64_t* sums = reinterpret_cast<const uint64_t*>(h);
     for (int64_t k = 0; k < plan->n; ++k) {
       const uint64_t nb = plan->nbytes[(size_t)k];

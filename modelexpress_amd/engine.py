@@ -516,13 +516,22 @@ class VerifyPlan:
         self._sums = (C.c_uint32 * max(1, self.n))()
         self._dig = (C.c_uint8 * (16 * max(1, self.n)))()
 
-    def checksums(self, *, stream: int = 0) -> list[str]:
+    def checksums_raw(self, *, stream: int = 0):
+        """One pass; the ``n`` checksums as the plan's own ``uint32`` ctypes array (rewritten by the next pass)."""
         L.check(L.lib().mxp_verify_plan_checksums(self._engine._h, self._h, self._sums, C.c_void_p(stream)))
-        return [format(self._sums[i], "08x") for i in range(self.n)]
+        return self._sums
+
+    def checksums(self, *, stream: int = 0) -> list[str]:
+        sums = self.checksums_raw(stream=stream)
+        return [format(sums[i], "08x") for i in range(self.n)]
+
+    def digests_raw(self, *, stream: int = 0):
+        """One pass; the ``n`` 16-byte digests as the plan's own ``uint8`` ctypes array (rewritten by the next pass)."""
+        L.check(L.lib().mxp_verify_plan_digests(self._engine._h, self._h, self._dig, None, C.c_void_p(stream)))
+        return self._dig
 
     def digests(self, *, stream: int = 0) -> list[str]:
-        L.check(L.lib().mxp_verify_plan_digests(self._engine._h, self._h, self._dig, None, C.c_void_p(stream)))
-        raw = bytes(self._dig)
+        raw = bytes(self.digests_raw(stream=stream))
         return [raw[16 * i: 16 * i + 16].hex() for i in range(self.n)]
 
     def close(self) -> None:
