@@ -653,11 +653,15 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
   uint8_t* d = e.desc_dev.p;
   uint32_t* const fanned = reinterpret_cast<uint32_t*>(d + o_sum);
   if (sums_out) HIP_OK(launch_fill_u32(fanned, fan_elems(fan), 0u, stream));
-  bool checksum_only = !boxes.empty();
-  for (const auto& b : boxes) checksum_only = checksum_only && b.op == kOpChecksumOnly;
+  bool checksum_only = !boxes.empty(), widening_only = !boxes.empty();
+  for (const auto& b : boxes) {
+    checksum_only = checksum_only && b.op == kOpChecksumOnly;
+    widening_only = widening_only && op_widens(b.op);
+  }
   HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + o_segs), reinterpret_cast<const WorkItem*>(d + o_work),
                       (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + o_src),
-                      reinterpret_cast<void* const*>(d + o_dst), fanned, fan, e.opt.nan_bits, stream, checksum_only));
+                      reinterpret_cast<void* const*>(d + o_dst), fanned, fan, e.opt.nan_bits, stream, checksum_only, nullptr, 0,
+                      widening_only));
   if (sums_out && n_sums) {
     HIP_OK(launch_fold_fan(fanned, fan, 1, (uint64_t)n_sums, reinterpret_cast<uint32_t*>(d + o_out), false, stream));
     HIP_OK(hipMemcpyAsync(e.desc_host + o_out, d + o_out, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));

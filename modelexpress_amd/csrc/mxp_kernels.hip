@@ -497,10 +497,10 @@ hipError_t configure_place_kernels() {
 hipError_t launch_place(const Seg* segs_dev, const WorkItem* work_dev, uint32_t n_work,
                         const void* const* src_bases_dev, void* const* dst_bases_dev,
                         uint32_t* sums_dev, Fan fan, uint16_t nan_bits, hipStream_t stream, bool checksum_only,
-                        uint32_t* zero_dev, uint32_t zero_words) {
+                        uint32_t* zero_dev, uint32_t zero_words, bool widening_only) {
   if (n_work == 0) return hipSuccess;
   if (hipError_t e = configure_place_kernels(); e != hipSuccess) return e;
-  const uint32_t lds_place = kOnePerCu, lds_csum = kTwoPerCu;
+  const uint32_t lds_place = widening_only ? kTwoPerCu : kOnePerCu, lds_csum = kTwoPerCu;
   if (checksum_only) {
     hipLaunchKernelGGL(checksum_kernel, dim3(n_work), dim3(kPlaceThreads), lds_csum, stream, segs_dev, work_dev,
                        src_bases_dev, sums_dev, fan);

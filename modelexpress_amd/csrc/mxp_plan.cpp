@@ -14,6 +14,7 @@
 #include <set>
 
 #include "mxp_internal.hpp"
+#include "mxp_overlap.hpp"
 
 namespace mxp {
 namespace {
@@ -391,6 +392,8 @@ struct Planner {
       got += vol;
       emit_writes(sh.tensor, kind, sv, dv);
     }
+    // (shards that overlap count twice here and are refused with the gaps: the reference reads shards with
+    // unordered transfers, so it defines no winner for them; transfer_plan.py:160-172 refuses them too)
     if (got != want)
       throw Error(MXP_ERR_COVERAGE, "virtual tensor '" + v.name + "': its shards cover " + std::to_string(got) +
                                         " of the " + std::to_string(want) + " elements this rank needs");
@@ -558,6 +561,8 @@ struct Planner {
       emit(it, kind, local, dest);
     }
 
+    resolve_overlaps();
+
     // ---- coverage (installer.py:219-251), extended to every parameter ----
     if (!unmapped.empty() && !(pl.flags & MXP_PLAN_ALLOW_UNMAPPED)) {
       std::string m = "placement coverage incomplete; refusing a partially-written model. unmapped checkpoint tensors=[";
@@ -580,37 +585,68 @@ struct Planner {
       if (uncovered.size() > 10) m += " ...";
       throw Error(MXP_ERR_COVERAGE, m + "]");
     }
-    check_disjoint();
   }
 
-  // Chunks execute on several streams, so two writes may land in either order: the
-  // reference's "later write wins" (receiver.py:939-955) cannot be honoured for
-  // overlapping destinations, and such a plan is refused instead.
-  void check_disjoint() const {
-    std::vector<std::vector<const WriteRec*>> per(pl.params.size());
-    for (const auto& w : pl.writes) per[w.param].push_back(&w);
+  // Later write wins.  The reference installs tensor after tensor on one stream, so where two
+  // writes of a parameter overlap the later one's bytes stay (installer.py:419-424; the staged
+  // re-slice keeps the captured order for overlapping destinations, receiver.py:939-955).  Here
+  // chunks run on several streams and a launch gives no order between its workgroups, so the
+  // order is settled at plan time instead: an earlier write gives up the bytes a later write of
+  // the same parameter covers, and what is left of it is re-expressed as pitched boxes.  Every
+  // destination byte then has exactly one writer, the fused checksums see the bytes that stay,
+  // and `bytes_written` is the exact size of the union.
+  void resolve_overlaps() {
+    std::vector<std::vector<size_t>> per(pl.params.size());
+    for (size_t i = 0; i < pl.writes.size(); ++i) per[pl.writes[i].param].push_back(i);
+    std::vector<char> touched(pl.params.size(), 0);
+    bool any = false;
+    for (size_t p = 0; p < per.size() && !any; ++p) {
+      // candidates by sorted spans, as cheap as the plain disjointness check
+      auto v = per[p];
+      std::sort(v.begin(), v.end(), [&](size_t a, size_t b) { return pl.writes[a].dst_offset < pl.writes[b].dst_offset; });
+      auto end = [&](size_t i) { const WriteRec& w = pl.writes[i]; return w.dst_offset + (w.rows - 1) * w.dst_pitch + w.row_bytes; };
+      for (size_t i = 0; i < v.size() && !any; ++i)
+        for (size_t j = i + 1; j < v.size() && pl.writes[v[j]].dst_offset < end(v[i]); ++j)
+          if (writes_may_overlap(pl.writes[v[i]], pl.writes[v[j]])) { any = true; break; }
+    }
+    if (!any) return;
+    // plan order = the order the reference would install in
+    std::vector<std::vector<WriteRec>> pieces(pl.writes.size());
+    for (size_t i = 0; i < pl.writes.size(); ++i) pieces[i].push_back(pl.writes[i]);
     for (size_t p = 0; p < per.size(); ++p) {
-      auto& v = per[p];
-      std::sort(v.begin(), v.end(), [](const WriteRec* a, const WriteRec* b) { return a->dst_offset < b->dst_offset; });
-      auto span_end = [](const WriteRec* w) { return w->dst_offset + (w->rows - 1) * w->dst_pitch + w->row_bytes; };
-      for (size_t i = 0; i < v.size(); ++i) {
-        const uint64_t end_i = span_end(v[i]);
-        for (size_t j = i + 1; j < v.size() && v[j]->dst_offset < end_i; ++j) {
-          const WriteRec *a = v[i], *b = v[j];
-          bool disjoint = false;
-          if (a->rows > 1 && b->rows > 1 && a->dst_pitch == b->dst_pitch) {
-            const uint64_t pitch = a->dst_pitch;
-            const uint64_t ca = a->dst_offset % pitch, cb = b->dst_offset % pitch;
-            if (ca + a->row_bytes <= pitch && cb + b->row_bytes <= pitch &&
-                (ca + a->row_bytes <= cb || cb + b->row_bytes <= ca))
-              disjoint = true;
+      const auto& idx = per[p];
+      for (size_t b = 1; b < idx.size(); ++b) {
+        const WriteRec& later = pl.writes[idx[b]];
+        for (size_t a = 0; a < b; ++a) {
+          std::vector<WriteRec> next;
+          bool changed = false;
+          for (const WriteRec& e : pieces[idx[a]]) {
+            if (!writes_may_overlap(e, later)) { next.push_back(e); continue; }
+            std::vector<WriteRec> left =
+                clip_write(e, later, dtype_size(ck.tensors[e.tensor].dtype), dtype_size(pl.params[e.param].dtype), pl.params[p].name);
+            changed = changed || left.size() != 1 || left[0].rows != e.rows || left[0].row_bytes != e.row_bytes;
+            next.insert(next.end(), left.begin(), left.end());
+            if (next.size() > (1u << 20)) throw Error(MXP_ERR_UNSUPPORTED, "overlapping writes of '" + pl.params[p].name + "' need too many boxes");
           }
-          if (!disjoint)
-            throw Error(MXP_ERR_UNSUPPORTED, "tensors '" + ck.tensors[a->tensor].name + "' and '" +
-                                                 ck.tensors[b->tensor].name + "' write overlapping bytes of '" +
-                                                 pl.params[p].name + "'");
+          if (changed) {
+            pieces[idx[a]].swap(next);
+            touched[p] = 1;
+          }
         }
       }
+    }
+    std::vector<WriteRec> all;
+    for (auto& v : pieces) all.insert(all.end(), v.begin(), v.end());
+    pl.writes.swap(all);
+    for (size_t p = 0; p < pl.params.size(); ++p) {
+      if (!touched[p]) continue;
+      pl.params[p].bytes_written = 0;
+      pl.params[p].n_writes = 0;
+    }
+    for (const auto& w : pl.writes) {
+      if (!touched[w.param]) continue;
+      pl.params[w.param].bytes_written += w.rows * w.row_bytes;
+      pl.params[w.param].n_writes += 1;
     }
   }
 };

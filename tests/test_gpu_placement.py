@@ -333,3 +333,45 @@ def test_random_models_on_the_device(seed, oracle, tmp_path, mxp):
             assert d.cpu().numpy().tobytes()[: p.nbytes] == want[p.name].tobytes(), (seed, mode, p.name)
             assert s == oracle.safe_checksum(want[p.name]) and g == oracle.tensor_digest(want[p.name]), (seed, mode, p.name)
     eng.close()
+
+
+@pytest.mark.parametrize("tp", [1, 2])
+def test_overlapping_writes_keep_the_later_tensor_on_device(tp, gpu_engine, gpu_engine_band, oracle, tmp_path):
+    """A checkpoint with gate_proj, up_proj and a premerged gate_up_proj: tensors installed one after the other
+    (engines/vllm/refit/installer.py:419-424) leave the later one's bytes.  The plan settles the order before any
+    byte moves, so every execution mode gives the serial result, and the fused checksums are those of the bytes
+    that stay."""
+    from safetensors.torch import save_file
+    from modelexpress_amd.engine import Checkpoint, ParamSpec, PlacementPlan
+
+    g = torch.Generator().manual_seed(11)
+    inter, hidden = 192, 96
+    tensors = {"mlp.gate_up_proj.weight": torch.randn(2 * inter, hidden, generator=g).to(torch.bfloat16),
+               "mlp.up_proj.weight": torch.randn(inter, hidden, generator=g).to(torch.bfloat16),
+               "mlp.gate_proj.weight": torch.randn(inter, hidden, generator=g).to(torch.bfloat16),
+               "mlp.down_proj.weight": torch.randn(hidden, inter, generator=g).to(torch.bfloat16)}
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    ck = Checkpoint(str(tmp_path))
+    ow = dict(oracle.load_checkpoint(str(tmp_path)))
+    order = [t.name for t in ck.tensors()]
+    for rank in range(tp):
+        specs = [ParamSpec("mlp.gate_up_proj.weight", "BF16", (2 * inter // tp, hidden)),
+                 ParamSpec("mlp.down_proj.weight", "BF16", (hidden, inter // tp))]
+        oparams = {p.name: oracle.OTensor.zeros(p.shape, p.dtype) for p in specs}
+        oracle.MdlOracle(oparams, tp, rank).load_weights([(n, ow[n]) for n in order])
+        plan = PlacementPlan(ck, specs, tp_size=tp, tp_rank=rank)
+        assert sum(q["bytes_written"] for q in plan.param_info()) == sum(p.nbytes for p in plan.params)
+        for mode in ("ingest", "ingest_bounce", "ingest_band", "resident"):
+            eng = gpu_engine_band if mode == "ingest_band" else gpu_engine
+            dst = eng.allocate(plan, fill=0xCD)
+            if mode == "resident":
+                eng.execute_resident(plan, _stage_files(ck), dst)
+            else:
+                eng.set_direct_placement({"ingest": 1, "ingest_bounce": -1}.get(mode, 0))
+                try:
+                    eng.execute(plan, dst)
+                finally:
+                    eng.set_direct_placement(0)
+            for p, d, s in zip(plan.params, dst, eng.checksums(plan)):
+                assert d.cpu().numpy().tobytes() == oparams[p.name].tobytes(), (tp, rank, mode, p.name)
+                assert s == oracle.safe_checksum(oparams[p.name]), (tp, rank, mode, p.name)

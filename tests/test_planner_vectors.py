@@ -298,3 +298,57 @@ def test_widening_and_half_conversions_are_planned(mxp, oracle, tmp_path):
     p16 = PlacementPlan(ck, [ParamSpec("a.weight", "F16", (4, 8)), ParamSpec("b.weight", "BF16", (4, 8))], allow_cast=True,
                         allow_unmapped=True)
     assert {x.tensor: (x.cast, x.row_bytes, x.src_pitch) for x in p16.writes()} == {"a.weight": (7, 64, 64), "b.weight": (6, 64, 64)}
+
+
+def _in_checkpoint_order(tmp_path, weights, tag):
+    """`weights` in the order the product iterates the file the third-party writer produces (the
+    oracle, like the reference's serial copy loop, installs in the order it is handed the tensors)."""
+    path = tmp_path / f"order_{tag}"
+    path.mkdir(exist_ok=True)
+    save_file({n: t.contiguous() for n, t in weights}, str(path / "model.safetensors"))
+    order = [t.name for t in Checkpoint(str(path)).tensors()]
+    by = dict(weights)
+    return [(n, by[n]) for n in order]
+
+
+@pytest.mark.parametrize("tp", [1, 2])
+def test_later_write_wins_where_two_tensors_meet_in_one_parameter(oracle, tmp_path, tp):
+    """engines/vllm/refit/installer.py:419-424 installs tensor after tensor, so the later tensor's bytes stay
+    where two of them map to the same bytes.  A checkpoint that holds gate_proj and up_proj AND a premerged
+    gate_up_proj: each half of the parameter keeps what the iteration met last; the product settles that
+    when it plans, so every destination byte still has one writer."""
+    merged = torch.arange(32, dtype=torch.int64).reshape(16, 2)
+    up = torch.arange(16, dtype=torch.int64).reshape(8, 2) + 1000
+    gate = torch.arange(16, dtype=torch.int64).reshape(8, 2) + 2000
+    local, half = 16 // tp, 8 // tp
+    weights = _in_checkpoint_order(tmp_path, [("mlp.gate_up_proj.weight", merged), ("mlp.up_proj.weight", up),
+                                              ("mlp.gate_proj.weight", gate)], f"m{tp}")
+    for rank in range(tp):
+        want, plan = _run_both(oracle, tmp_path, weights, {"mlp.gate_up_proj.weight": ("I64", (local, 2))},
+                               tp_size=tp, tp_rank=rank)
+        g_rows = u_rows = None
+        for name, _t in weights:  # replay of the serial loop, half by half
+            if name == "mlp.gate_up_proj.weight":
+                g_rows, u_rows = merged[rank * half:(rank + 1) * half], merged[8 + rank * half:8 + (rank + 1) * half]
+            elif name == "mlp.up_proj.weight":
+                u_rows = up[rank * half:(rank + 1) * half]
+            else:
+                g_rows = gate[rank * half:(rank + 1) * half]
+        assert want["mlp.gate_up_proj.weight"] == _bytes(torch.cat((g_rows, u_rows))), (tp, rank, [n for n, _ in weights])
+        info = {q["name"]: q for q in plan.param_info()}["mlp.gate_up_proj.weight"]
+        assert info["bytes_written"] == local * 2 * 8  # the size of the union, not the sum of the writes
+        spans = sorted((w.dst_offset, w.dst_offset + (w.rows - 1) * w.dst_pitch + w.row_bytes) for w in plan.writes())
+        assert all(a[1] <= b[0] for a, b in zip(spans, spans[1:]))  # what is left is disjoint
+        assert weights[-1][0] != "mlp.gate_up_proj.weight" and len(spans) < 2 + 2 * tp  # some write lost bytes
+
+
+def test_two_experts_mapped_to_one_slot_leave_the_later_one(oracle, tmp_path):
+    p = "model.layers.0.mlp."
+    e0 = torch.full((2, 2), 3.0).to(F8)
+    e1 = torch.full((2, 2), 5.0).to(F8)
+    weights = _in_checkpoint_order(tmp_path, [(p + "experts.0.down_proj.weight", e0), (p + "experts.1.down_proj.weight", e1)], "ex")
+    mapping = [(p + "experts.w2_", p + "experts.0.down_proj.", 0, "w2", 0), (p + "experts.w2_", p + "experts.1.down_proj.", 1, "w2", 0)]
+    want, plan = _run_both(oracle, tmp_path, weights, {p + "experts.w2_weight": ("F8_E4M3", (1, 2, 2))}, experts=mapping,
+                           expert_local=lambda _name, _gid: 0)
+    assert want[p + "experts.w2_weight"] == _bytes(dict(weights)[weights[-1][0]])
+    assert len(plan.writes()) == 1 and plan.writes()[0].tensor == weights[-1][0]
