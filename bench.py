@@ -46,10 +46,10 @@ sys.path.insert(0, str(ROOT))
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per place_kernel launch on the default workload, from the FETCH_SIZE and
 # WRITE_SIZE counter runs summarised in profiles/place_kernel_llama3_8b_tp8.txt (each
-# counter scaled by its reading for a plain 1 GiB device copy).  Counters cannot be read
+# counter scaled by its reading for plain device copies of known size).  Counters cannot be read
 # from inside this process, so the figure is carried here and reported only when the
 # workload is the profiled one.
-PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_097_800_000}
+PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_099_000_000}
 
 
 def _log(msg: str) -> None:
