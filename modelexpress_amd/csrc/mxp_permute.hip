@@ -45,6 +45,7 @@
 // 384 bytes lifts 16384 x 16384 to 6.0 TB/s: the loss is in how the strided source lines fall
 // on the memory channels, which a caller controls and this kernel does not.
 #include "mxp_device.h"
+#include <atomic>
 #include "mxp_checksum.h"
 #include "mxp_convert.h"
 
@@ -326,7 +327,7 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
                                                               const TransposeDesc d, uint32_t nan_bits,
                                                               uint32_t* __restrict__ sum_out, Fan fan) {
   using S = Sub<ES, OP>;
-  __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
+  extern __shared__ __align__(16) uint8_t lds[];  // S::kLdsBytes per wavefront of the workgroup
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   Csum cs;
   transpose_tile<ES, OP>(src, dst, d, blockIdx.x, nan_bits, lds, wave, cs);
@@ -352,8 +353,7 @@ __global__ __launch_bounds__(kThreads) void transpose_kernel(const uint8_t* __re
 template <int ES, int OP>
 __global__ __launch_bounds__(kThreads) void transpose_batch_kernel(const TransposeItem* __restrict__ items,
                                                                     uint32_t n_items, uint32_t nan_bits) {
-  using S = Sub<ES, OP>;
-  __shared__ __align__(16) uint8_t lds[kWaves * S::kLdsBytes];
+  extern __shared__ __align__(16) uint8_t lds[];  // Sub<ES, OP>::kLdsBytes per wavefront of the workgroup
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   uint32_t lo = 0, hi = n_items;  // the last item with first_tile <= blockIdx.x
   while (hi - lo > 1) {
@@ -394,6 +394,23 @@ bool with_instance(int elem_size, uint32_t op, F&& f) {
   }
 }
 
+// A workgroup's LDS is sized by the wavefronts it is launched with (a 2-wavefront workgroup that
+// reserved room for 8 left a compute unit with four resident wavefronts).  Above 64 KiB the
+// kernel instance needs the attribute once per device.
+template <typename K>
+hipError_t allow_lds(K kernel, uint32_t bytes) {
+  static std::atomic<uint64_t> allowed{0};  // per kernel instance: bit per device
+  if (bytes <= 64u * 1024u) return hipSuccess;
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (allowed.load(std::memory_order_acquire) & bit) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kWaves * 16 * 1024);
+  if (e == hipSuccess) allowed.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+
 struct LaunchOne {
   dim3 grid, block;
   hipStream_t stream;
@@ -403,9 +420,13 @@ struct LaunchOne {
   uint32_t nan_bits;
   uint32_t* sum_out;
   Fan fan;
+  mutable hipError_t err = hipSuccess;
   template <int ES, int OP>
   void operator()() const {
-    hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, 0, stream, s, t, d, nan_bits, sum_out, fan);
+    const uint32_t lds = (block.x / 64u) * Sub<ES, OP>::kLdsBytes;
+    err = allow_lds(transpose_kernel<ES, OP>, lds);
+    if (err != hipSuccess) return;
+    hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, lds, stream, s, t, d, nan_bits, sum_out, fan);
   }
 };
 
@@ -414,9 +435,13 @@ struct LaunchBatch {
   hipStream_t stream;
   const TransposeItem* items;
   uint32_t n_items, nan_bits;
+  mutable hipError_t err = hipSuccess;
   template <int ES, int OP>
   void operator()() const {
-    hipLaunchKernelGGL((transpose_batch_kernel<ES, OP>), grid, block, 0, stream, items, n_items, nan_bits);
+    const uint32_t lds = (block.x / 64u) * Sub<ES, OP>::kLdsBytes;
+    err = allow_lds(transpose_batch_kernel<ES, OP>, lds);
+    if (err != hipSuccess) return;
+    hipLaunchKernelGGL((transpose_batch_kernel<ES, OP>), grid, block, lds, stream, items, n_items, nan_bits);
   }
 };
 
@@ -429,6 +454,7 @@ hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, 
   const LaunchOne one{dim3((uint32_t)d.n_tiles), dim3(d.waves * 64u), stream, static_cast<const uint8_t*>(src),
                       static_cast<uint8_t*>(dst), d, nan_bits, sum_out, fan};
   if (!with_instance(elem_size, op, one)) return hipErrorInvalidValue;
+  if (one.err != hipSuccess) return one.err;
   return hipGetLastError();
 }
 
@@ -438,6 +464,7 @@ hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_ite
   if (total_tiles > 0x7FFFFFFFull || waves == 0 || waves > (uint32_t)kWaves || (waves & (waves - 1))) return hipErrorInvalidValue;
   const LaunchBatch many{dim3((uint32_t)total_tiles), dim3(waves * 64u), stream, items_dev, n_items, nan_bits};
   if (!with_instance(elem_size, op, many)) return hipErrorInvalidValue;
+  if (many.err != hipSuccess) return many.err;
   return hipGetLastError();
 }
 
