@@ -126,6 +126,9 @@ typedef struct mxp_plan mxp_plan;
 #define MXP_PLAN_ALLOW_UNMAPPED 0x2u      /* skip checkpoint tensors with no destination  */
 #define MXP_PLAN_ALLOW_UNCOVERED 0x4u     /* allow parameters no tensor writes            */
 #define MXP_PLAN_NO_FP8_BLOCK_CHECK 0x8u  /* do not require 128-aligned fp8 scale slicing */
+#define MXP_PLAN_NONLOCAL_EXPERTS_UNMAPPED 0x10u /* an expert that is not local to the rank counts as
+                                           * unmapped, as in the reference's loaderless mode
+                                           * (installer.py:708-710,219-251), instead of being skipped */
 
 int mxp_plan_create(const mxp_ckpt* ckpt, int32_t tp_size, int32_t tp_rank, uint32_t flags,
                     mxp_plan** out);
@@ -139,7 +142,9 @@ int64_t mxp_plan_add_param(mxp_plan* plan, const char* name, int32_t dtype, int3
 int mxp_plan_add_stacked(mxp_plan* plan, const char* fused_suffix, const char* member_suffix);
 /* One row of the model's get_expert_mapping(): shard is "w1", "w2" or "w3";
  * `local_expert_id` is the slot in the rank's stacked parameter, or -1 when the
- * expert is not local to this rank (such tensors are then skipped, not an error). */
+ * expert is not local to this rank: such tensors are then skipped, not an error (a rank is
+ * handed the whole checkpoint and there is no stock loader behind this one to hand them to),
+ * unless the plan was created with MXP_PLAN_NONLOCAL_EXPERTS_UNMAPPED. */
 int mxp_plan_add_expert(mxp_plan* plan, const char* param_prefix, const char* weight_prefix,
                         int32_t expert_id, const char* shard, int32_t local_expert_id);
 /* Skip checkpoint tensors whose name starts with `prefix` (e.g. other pipeline stages). */

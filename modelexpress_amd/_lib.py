@@ -33,6 +33,7 @@ PLAN_ALLOW_CAST_F32_BF16 = 0x1
 PLAN_ALLOW_UNMAPPED = 0x2
 PLAN_ALLOW_UNCOVERED = 0x4
 PLAN_NO_FP8_BLOCK_CHECK = 0x8
+PLAN_NONLOCAL_EXPERTS_UNMAPPED = 0x10
 
 WRITE_KINDS = ("direct", "fused", "expert", "premerged")
 

@@ -185,7 +185,7 @@ struct Planner {
       if (p < 0) return 0;
       const ParamRec& fp = pl.params[p];
       if (fp.shape.empty()) return 0;
-      if (e.local_id == -1) return 2;
+      if (e.local_id == -1) return (pl.flags & MXP_PLAN_NONLOCAL_EXPERTS_UNMAPPED) ? 0 : 2;
       if (e.local_id < 0 || e.local_id >= fp.shape[0]) return 0;
       const View slot = index0(full_view(fp.shape, p), e.local_id);
       if (e.shard == "w2") {

@@ -133,7 +133,8 @@ class PlacementPlan:
                  stacked_params_mapping: Sequence | None = None, expert_mapping: Sequence | None = None,
                  skip_prefixes: Sequence[str] = (), virtual_tensors: Sequence[VirtualTensor] = (),
                  allow_cast: bool = False, allow_unmapped: bool = False,
-                 allow_uncovered: bool = False, fp8_block_check: bool = True):
+                 allow_uncovered: bool = False, fp8_block_check: bool = True,
+                 nonlocal_experts_unmapped: bool = False):
         lib = L.lib()
         self.ckpt = ckpt
         flags = 0
@@ -141,6 +142,7 @@ class PlacementPlan:
         flags |= L.PLAN_ALLOW_UNMAPPED if allow_unmapped else 0
         flags |= L.PLAN_ALLOW_UNCOVERED if allow_uncovered else 0
         flags |= 0 if fp8_block_check else L.PLAN_NO_FP8_BLOCK_CHECK
+        flags |= L.PLAN_NONLOCAL_EXPERTS_UNMAPPED if nonlocal_experts_unmapped else 0
         self._h = C.c_void_p()
         L.check(lib.mxp_plan_create(ckpt._h, tp_size, tp_rank, flags, C.byref(self._h)))
         self.tp_size, self.tp_rank = tp_size, tp_rank

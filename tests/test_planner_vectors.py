@@ -352,3 +352,22 @@ def test_two_experts_mapped_to_one_slot_leave_the_later_one(oracle, tmp_path):
                            expert_local=lambda _name, _gid: 0)
     assert want[p + "experts.w2_weight"] == _bytes(dict(weights)[weights[-1][0]])
     assert len(plan.writes()) == 1 and plan.writes()[0].tensor == weights[-1][0]
+
+
+def test_expert_outside_the_rank_is_skipped_or_unmapped_on_request(tmp_path):
+    """installer.py:708-710: an expert whose local id is negative has no destination; the reference's loaderless
+    mode then refuses the load (installer.py:219-251), its normal mode hands the tensor to the stock loader.  The
+    product skips it by default (each rank reads the whole checkpoint) and offers the refusal as a plan flag."""
+    p = "model.layers.0.mlp."
+    e0 = torch.full((2, 2), 3.0).to(F8)
+    e1 = torch.full((2, 2), 5.0).to(F8)
+    save_file({p + "experts.0.down_proj.weight": e0, p + "experts.1.down_proj.weight": e1}, str(tmp_path / "model.safetensors"))
+    ck = Checkpoint(str(tmp_path))
+    mapping = [(p + "experts.w2_", p + "experts.0.down_proj.", 0, "w2", 0), (p + "experts.w2_", p + "experts.1.down_proj.", 1, "w2", -1)]
+    specs = [ParamSpec(p + "experts.w2_weight", "F8_E4M3", (1, 2, 2))]
+    plan = PlacementPlan(ck, specs, expert_mapping=mapping)
+    assert [w.tensor for w in plan.writes()] == [p + "experts.0.down_proj.weight"]
+    assert apply_plan_numpy(ck, plan)[p + "experts.w2_weight"].tobytes() == _bytes(e0)
+    with pytest.raises(MxpError, match="experts.1.down_proj.weight") as e:
+        PlacementPlan(ck, specs, expert_mapping=mapping, nonlocal_experts_unmapped=True)
+    assert e.value.code == ERR_COVERAGE
