@@ -329,6 +329,10 @@ def main() -> int:
     ap.add_argument("--classes", action="store_true",
                     help="also time each class of segments of the workload as a launch of its own (contiguous row "
                          "blocks, strided column slices, vocabulary slices ...): the breakdown of the step time")
+    ap.add_argument("--no-ops", action="store_true", help="skip the stand-alone operator measurements (ops)")
+    ap.add_argument("--direct-min", type=int, default=0,
+                    help="ingest leg: smallest contiguous piece copied straight to its final address, in bytes "
+                         "(0 = library default of 64 KiB, negative = every byte through the bounce slot and the kernel)")
     ap.add_argument("--probes", action="store_true",
                     help="also time the workload's access shapes one by one (contiguous copy, the column slices' row "
                          "gathers from the checkpoint's pitch and from a padded one, reads alone, writes alone)")
@@ -431,7 +435,7 @@ def main() -> int:
 
         # ---- the read-only operators over the finished buffers (1 x bytes each) ----
         sizes = [p.nbytes for p in plan.params]
-        if placed <= 8e9:
+        if placed <= 8e9 and not args.no_ops:
             ops = {}
             vplan = eng.verify_plan(dst, sizes)  # the buffers lowered once: a run is one launch and one small copy back
             # the plan's calls are timed as the C ABI returns them (a ctypes array); the one-shot calls include the
@@ -625,6 +629,8 @@ def main() -> int:
                 e2 = PlacementEngine(0, ring_slots=args.ring_slots, slot_bytes=args.slot_mib << 20,
                                      reader_threads=args.readers or host_threads, streams=4,
                                      tile_bytes=args.tile_kib * 1024, pack_strided_on_host=pack)
+                if args.direct_min:
+                    e2.set_direct_placement(args.direct_min)
                 best = None
                 for i in range(4):
                     st = e2.execute(plan, dst)
