@@ -437,7 +437,7 @@ def main() -> int:
         sizes = [p.nbytes for p in plan.params]
         if placed <= 8e9 and not args.no_ops:
             ops = {}
-            vplan = eng.verify_plan(dst, sizes)  # the buffers lowered once: a run is one launch and one small copy back
+            vplan = eng.verify_plan(dst, sizes)  # the buffers lowered once: a run is one launch, a small reduction and an event wait
             # the plan's calls are timed as the C ABI returns them (a ctypes array); the one-shot calls include the
             # wrapper's conversion of 195 results to hex strings
             for op_name, fn, one_shot in (("checksum32", vplan.checksums_raw, lambda: eng.checksum32(dst, sizes)),

@@ -352,8 +352,10 @@ int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uin
  * verifies the same buffers every step, and the reference keeps its descriptor lists for that
  * reason (refit/reshard/receiver.py:787-801; the verify loop is
  * modelexpress_rl/inference/nixl_staged_transfer.py:529-549).  _create lowers the buffers, uploads
- * the descriptor tables and allocates the result block; a run is then one kernel launch and one
- * small copy back (no descriptor build, no upload, no allocation), and waits only for that copy.
+ * the descriptor tables and allocates the pinned result block; a run is then one kernel launch
+ * plus a small one that adds up the accumulator copies, clears them and stores the totals into
+ * that block (no descriptor build, no upload, no allocation, no copy command), and waits for the
+ * event behind it.
  * The addresses and sizes are the ones given at create; when a buffer moves, build a new plan.
  * One run of a plan at a time. */
 typedef struct mxp_verify_plan mxp_verify_plan;

@@ -11,6 +11,8 @@
 //                 copy, 6 bytes per element for the cast)
 //  digest_kernel  int32-word row sums for the blake2b-hashed tensor digest
 //                 (reads each byte once)
+//  checksum_kernel the checksum alone over existing buffers (reads each byte once)
+//  fold_fan_kernel adds up the copies the accumulators are kept in (mxp_device.h: Fan)
 #include "mxp_device.h"
 #include "mxp_checksum.h"
 #include "mxp_convert.h"

@@ -505,7 +505,7 @@ class PlacementEngine:
 
 class VerifyPlan:
     """Handle of ``mxp_verify_plan``: a fixed set of device buffers lowered once for repeated ``checksum32`` /
-    ``tensor_digest`` passes; a run is one launch and one small copy back."""
+    ``tensor_digest`` passes; a run is one launch, a small reduction into pinned memory and an event wait."""
 
     def __init__(self, engine: "PlacementEngine", buffers: Sequence, nbytes: Sequence[int] | None = None):
         self._engine = engine
