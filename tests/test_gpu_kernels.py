@@ -83,6 +83,29 @@ def test_verify_plan_repeats_match_one_shot_calls(gpu_engine, oracle, oracle_c):
     assert empty.checksums() == [] and empty.digests() == []
 
 
+def test_batches_too_large_for_accumulator_copies_take_the_plain_layout(gpu_engine, oracle_c):
+    """Accumulators are kept in 64 copies up to 16,384 of them and in one copy beyond (csrc/mxp_device.h, make_fan):
+    both sides of that limit, through the one-shot calls and a verify plan, repeated; one large buffer among the
+    small ones gives many workgroups adding to one accumulator."""
+    rng = np.random.default_rng(23)
+    for n in (16384, 16385, 20000):
+        sizes = rng.integers(0, 200, n)
+        sizes[n // 2] = 3 * (1 << 20) + 7
+        data = rng.integers(0, 256, int(sizes.sum()), dtype=np.uint8)
+        base = torch.from_numpy(data).cuda()
+        offs = np.concatenate(([0], np.cumsum(sizes)))
+        dev = [base[int(offs[k]): int(offs[k + 1])] for k in range(n)]
+        probe = list(range(0, n, 997)) + [n // 2, n - 1]
+        want = {k: oracle_c.checksum32(data[int(offs[k]): int(offs[k + 1])]) for k in probe}
+        got = gpu_engine.checksum32(dev)
+        assert all(got[k] == want[k] for k in probe), n
+        plan = gpu_engine.verify_plan(dev)
+        for _ in range(2):
+            assert plan.checksums() == got, n
+        assert plan.digests() == gpu_engine.digest(dev), n
+        plan.close()
+
+
 def test_digest_reference_invariants_on_device(gpu_engine, oracle):
     a = np.arange(8192, dtype=np.int32)
     b = a.copy()
