@@ -515,6 +515,9 @@ def main() -> int:
                 ms = ev0.elapsed_time(ev1) / 10
                 ops[label] = {"bytes": nbytes, "ms": round(ms, 4), "gbps_algorithmic": round(2 * nbytes / ms / 1e6, 1),
                               "frac_of_hbm_peak": round(2 * nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                if ms < 0.02:
+                    ops[label]["note"] = ("one call moves %.0f MB: at this size a launch's fixed cost of a few microseconds is most of "
+                                          "the time; the 61-layer entries are the same transpose batched into one launch" % (2 * nbytes / 1e6))
                 del a, b
             # the other conversions of copy_ on 2^28 elements (6 bytes of traffic per element)
             n_el = 1 << 28
@@ -562,6 +565,10 @@ def main() -> int:
                 ms = ev0.elapsed_time(ev1) / 10
                 ops[label] = {"elements": n_el, "ms": round(ms, 4), "gbps_algorithmic": round((se + de) * n_el / ms / 1e6, 1),
                               "frac_of_hbm_peak": round((se + de) * n_el / ms / 1e6 / HBM_PEAK_GBPS, 4)}
+                if ms < 0.02:
+                    ops[label]["note"] = ("one call moves %.0f MB: at this size a launch's fixed cost of a few microseconds is most of "
+                                          "the time; the 61-layer entries below are the same transposes batched into one launch"
+                                          % ((se + de) * n_el / 1e6))
                 del a, b
             # the W_UK_T of every layer of a DeepSeek-V3-shaped model in one call (61 transposes, one launch)
             H, nope, lat, layers = 128, 128, 512, 61
