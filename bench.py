@@ -136,6 +136,9 @@ def _timed_resident(eng, plan, staged, dst, steps: int, warmup: int) -> dict:
     inside the timed region would slow the step they measure.  kernel <= device step <= wall step."""
     import torch
 
+    # pointer tables built once, as a serving loop that refits into the same buffers would: converting 200
+    # tensors to addresses costs Python ~0.1 ms a call, more than the whole step of the smallest configuration
+    staged, dst = eng.pointer_table(staged), eng.pointer_table(dst)
     for _ in range(warmup):
         eng.execute_resident(plan, staged, dst)
     torch.cuda.synchronize()

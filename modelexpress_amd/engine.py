@@ -275,13 +275,21 @@ class PlacementEngine:
 
     def execute_resident(self, plan: PlacementPlan, staged_files: Sequence, dst: Sequence, *, stream: int = 0,
                          timed: bool = False) -> dict | None:
-        """Placement from shard files already staged in HBM; one launch."""
-        fptrs = _ptr_array([_addr(t) for t in staged_files])
-        dptrs = _ptr_array([_addr(t) for t in dst])
+        """Placement from shard files already staged in HBM; one launch.  ``staged_files`` and ``dst`` are
+        torch tensors / raw addresses, or pointer tables built once with ``pointer_table`` (a serving loop
+        that refits into the same buffers every step then spends nothing on converting them again)."""
+        fptrs = staged_files if isinstance(staged_files, C.Array) else _ptr_array([_addr(t) for t in staged_files])
+        dptrs = dst if isinstance(dst, C.Array) else _ptr_array([_addr(t) for t in dst])
         stats = L.ExecStats() if timed else None
         L.check(L.lib().mxp_execute_resident(self._h, plan._h, fptrs, dptrs, C.c_void_p(stream),
                                              C.byref(stats) if timed else None))
         return stats.as_dict() if timed else None
+
+    @staticmethod
+    def pointer_table(buffers: Sequence):
+        """The ``void*`` array the C ABI takes for ``buffers`` (torch tensors or raw addresses).  The table
+        holds addresses only: the caller keeps the buffers alive and in place."""
+        return _ptr_array([_addr(t) for t in buffers])
 
     def set_direct_placement(self, min_bytes: int = 0) -> None:
         """Ingest copies contiguous unconverted pieces of at least ``min_bytes`` straight to their final address
