@@ -177,8 +177,9 @@ struct mxp_plan::Lowered {
   std::vector<void*> dst_host;        // what dst_bases currently holds
   std::vector<const void*> src_host;  // what src_bases currently holds
   // The pointer tables are rewritten with stream-ordered copies out of this pinned block
-  // ([destinations][sources]); `upload_done` guards the block, `launch_done` marks the last
-  // launch that reads the tables and accumulators, so a call on another stream waits for it.
+  // ([destinations][sources]); `upload_done` guards the block.  A call on another stream than the
+  // last launch's (`last_stream`) records `launch_done` on that stream and waits for it, so the
+  // tables and accumulators are not touched under a launch that still reads them.
   void** tab_host = nullptr;
   size_t tab_cap = 0;
   hipEvent_t upload_done = nullptr, launch_done = nullptr;
@@ -550,7 +551,18 @@ bool is_capturing(hipStream_t stream) {
 void upload_tables(mxp_plan::Lowered& L, const mxp_plan& pl, void* const* dst_ptrs, const void* const* file_ptrs,
                    size_t n_files, hipStream_t stream) {
   const bool capturing = is_capturing(stream);
-  if (!capturing && L.launch_rec && L.last_stream != stream) HIP_OK(hipStreamWaitEvent(stream, L.launch_done, 0));
+  if (!capturing && L.launch_rec && L.last_stream != stream) {
+    // The plan's last launch went to another stream: this one waits for what that stream holds now (the
+    // launch and whatever followed it).  The event is recorded here, when it is needed, and not behind
+    // every launch: an event between two back-to-back launches costs several microseconds of stream time.
+    if (hipEventRecord(L.launch_done, L.last_stream) == hipSuccess) {
+      HIP_OK(hipStreamWaitEvent(stream, L.launch_done, 0));
+    } else {
+      (void)hipGetLastError();  // that stream is gone; whatever it still runs is waited for the slow way
+      HIP_OK(hipDeviceSynchronize());
+    }
+    L.launch_rec = false;
+  }
   const size_t n = pl.params.size();
   const bool dst_changed = !(L.dst_host.size() == n && std::equal(L.dst_host.begin(), L.dst_host.end(), dst_ptrs));
   const bool src_changed =
@@ -575,7 +587,6 @@ void upload_tables(mxp_plan::Lowered& L, const mxp_plan& pl, void* const* dst_pt
 }
 void mark_launch(mxp_plan::Lowered& L, hipStream_t stream) {
   if (is_capturing(stream)) return;
-  HIP_OK(hipEventRecord(L.launch_done, stream));
   L.launch_rec = true;
   L.last_stream = stream;
 }
