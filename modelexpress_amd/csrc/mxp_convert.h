@@ -45,6 +45,24 @@ __device__ __forceinline__ uint32_t f32_to_f16_bits(uint32_t u) {
   return (a > 0x7F800000u) ? (((u >> 16) & 0x8000u) | 0x7E00u | ((a >> 13) & 0x3FFu)) : (uint32_t)hb;
 }
 
+// Two fp32 -> two fp16 (a in the low half), same result as f32_to_f16_bits on each, through the
+// packed converter.  Rounding a finite value gives at most an infinity, so a NaN half of the
+// converter's result marks a NaN input; only then (1e-6 of the elements at most in this path's
+// workloads) are the halves rebuilt from the input bits by the rule above.
+__device__ __forceinline__ uint32_t f32x2_to_f16x2(uint32_t a, uint32_t b) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  f32x2 f;
+  f.x = __uint_as_float(a);
+  f.y = __uint_as_float(b);
+  const f16x2 h = __builtin_convertvector(f, f16x2);
+  uint32_t p;
+  __builtin_memcpy(&p, &h, 4);
+  if (((p & 0x7FFF7FFFu) + 0x03FF03FFu) & 0x80008000u)  // a half above 0x7C00: a NaN
+    p = f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16);
+  return p;
+}
+
 // fp16 bits -> fp32 bits, exact (subnormals renormalised by the converter); NaNs made quiet.
 __device__ __forceinline__ uint32_t f16_to_f32_bits(uint32_t h) {
   const uint16_t hb = (uint16_t)h;
@@ -71,7 +89,7 @@ __device__ __forceinline__ uint32_t recode2(uint32_t w, uint32_t nan_bits) {
     __builtin_memcpy(&h, &w, 4);
     return f32x2_to_bf16x2(__float_as_uint((float)h.x), __float_as_uint((float)h.y), nan_bits);
   } else {
-    return recode1<OP>(w & 0xFFFFu, nan_bits) | (recode1<OP>(w >> 16, nan_bits) << 16);
+    return f32x2_to_f16x2(w << 16, w & 0xFFFF0000u);  // a bf16 is the upper half of its fp32
   }
 }
 
@@ -119,8 +137,9 @@ __device__ __forceinline__ uint2 narrow4(const uint4& a, uint32_t nan_bits) {
     o.x = f32x2_to_bf16x2(a.x, a.y, nan_bits);
     o.y = f32x2_to_bf16x2(a.z, a.w, nan_bits);
   } else {
-    o.x = narrow1<OP>(a.x, nan_bits) | (narrow1<OP>(a.y, nan_bits) << 16);
-    o.y = narrow1<OP>(a.z, nan_bits) | (narrow1<OP>(a.w, nan_bits) << 16);
+    static_assert(OP == kOpCastF32F16, "the narrowing conversions are fp32 -> bf16 and fp32 -> fp16");
+    o.x = f32x2_to_f16x2(a.x, a.y);
+    o.y = f32x2_to_f16x2(a.z, a.w);
   }
   return o;
 }

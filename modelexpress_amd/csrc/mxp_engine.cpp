@@ -200,23 +200,42 @@ struct mxp_engine {
   uint8_t* bounce_base = nullptr;
   std::vector<hipStream_t> streams;
   DevBuf<const void*> slot_ptrs;  // device table: slot i -> bounce address
-  // descriptor staging for the stand-alone operators
-  uint8_t* desc_host = nullptr;  // pinned
-  size_t desc_host_cap = 0;
-  DevBuf<uint8_t> desc_dev;
+  // Descriptor staging for the stand-alone operators: a pinned block and its device twin, kept
+  // twice and used in turn, so a call fills one while the device may still read what the call
+  // before it uploaded into the other (back-to-back calls do not wait for each other's kernels).
+  // `busy` is recorded after the last device use of an arena; whoever takes it next waits for it.
+  struct Arena {
+    uint8_t* host = nullptr;  // pinned
+    size_t host_cap = 0;
+    DevBuf<uint8_t> dev;
+    hipEvent_t busy = nullptr;
+    bool recorded = false;
+    ~Arena() {
+      if (busy) (void)hipEventDestroy(busy);
+      if (host) (void)hipHostFree(host);
+    }
+  };
+  Arena arenas[2];
+  unsigned arena_turn = 0;
   hipEvent_t ev_a = nullptr, ev_b = nullptr;
   hipEvent_t caller_ev = nullptr;   // what the caller had queued when an ingest started
   bool fused_digests = false;       // placements also accumulate the tensor_digest sums (mxp_engine_set_fused_digests)
   uint64_t direct_min = kDirectMinBytes;  // ingest copies contiguous pieces of at least this size straight to their
                                           // final address; 0 = none (mxp_engine_set_direct_placement)
-  hipEvent_t arena_busy = nullptr;  // recorded after the last device use of the descriptor arena
-  bool arena_recorded = false;
-  // descriptor table of batched transposes: same protocol as the arena, its own event
-  TransposeItem* items_host = nullptr;  // pinned
-  size_t items_cap = 0;
-  DevBuf<TransposeItem> items_dev;
-  hipEvent_t items_busy = nullptr;
-  bool items_recorded = false;
+  // descriptor table of batched transposes: same protocol as the arenas, also kept twice
+  struct ItemTable {
+    TransposeItem* host = nullptr;  // pinned
+    size_t cap = 0;
+    DevBuf<TransposeItem> dev;
+    hipEvent_t busy = nullptr;
+    bool recorded = false;
+    ~ItemTable() {
+      if (busy) (void)hipEventDestroy(busy);
+      if (host) (void)hipHostFree(host);
+    }
+  };
+  ItemTable item_tabs[2];
+  unsigned items_turn = 0;
   // launch timing (mxp_engine_set_launch_timing): event pairs around the placement kernel of the
   // last kTimingRing resident launches, recorded without synchronising
   std::vector<std::pair<hipEvent_t, hipEvent_t>> timing_ring;
@@ -229,16 +248,12 @@ struct mxp_engine {
   ~mxp_engine() {
     for (auto& pr : timing_ring) { (void)hipEventDestroy(pr.first); (void)hipEventDestroy(pr.second); }
     if (static_host) (void)hipHostFree(static_host);
-    if (arena_busy) (void)hipEventDestroy(arena_busy);
     if (caller_ev) (void)hipEventDestroy(caller_ev);
-    if (items_busy) (void)hipEventDestroy(items_busy);
-    if (items_host) (void)hipHostFree(items_host);
     for (auto s : streams) (void)hipStreamDestroy(s);
     for (auto& s : slots)
       if (s->done) (void)hipEventDestroy(s->done);
     if (pinned_base) (void)hipHostFree(pinned_base);
     if (bounce_base) (void)hipFree(bounce_base);
-    if (desc_host) (void)hipHostFree(desc_host);
     if (ev_a) (void)hipEventDestroy(ev_a);
     if (ev_b) (void)hipEventDestroy(ev_b);
   }
@@ -612,28 +627,31 @@ void pread_full(int fd, uint8_t* dst, uint64_t n, uint64_t off, const std::strin
   }
 }
 
-// The descriptor arena (pinned staging + its device twin) is shared by the stand-alone
-// operators.  A call may only overwrite or reallocate it once the previous user's device
-// work is done, whichever stream that ran on: users record `arena_busy` after their last
-// arena-dependent operation (release_arena) and wait for it before touching the arena.
-void acquire_arena(mxp_engine& e) {
-  if (e.arena_recorded) HIP_OK(hipEventSynchronize(e.arena_busy));
+// The descriptor arenas (pinned staging + its device twin, two of them taken in turn) are shared
+// by the stand-alone operators.  A call may only overwrite or reallocate an arena once its
+// previous user's device work is done, whichever stream that ran on: users record the arena's
+// `busy` event after their last arena-dependent operation (release_arena), and whoever takes the
+// arena next waits for it - which, with two arenas, is the call before the previous one.
+mxp_engine::Arena& acquire_arena(mxp_engine& e) {
+  mxp_engine::Arena& a = e.arenas[e.arena_turn++ & 1u];
+  if (a.recorded) HIP_OK(hipEventSynchronize(a.busy));
+  return a;
 }
-void release_arena(mxp_engine& e, hipStream_t stream) {
-  HIP_OK(hipEventRecord(e.arena_busy, stream));
-  e.arena_recorded = true;
+void release_arena(mxp_engine::Arena& a, hipStream_t stream) {
+  HIP_OK(hipEventRecord(a.busy, stream));
+  a.recorded = true;
 }
 
-void ensure_desc(mxp_engine& e, size_t bytes) {
-  if (bytes > e.desc_host_cap) {
-    if (e.desc_host) (void)hipHostFree(e.desc_host);
-    e.desc_host = nullptr;
-    e.desc_host_cap = 0;
+void ensure_desc(mxp_engine::Arena& a, size_t bytes) {
+  if (bytes > a.host_cap) {
+    if (a.host) (void)hipHostFree(a.host);
+    a.host = nullptr;
+    a.host_cap = 0;
     const size_t cap = align_up(bytes * 2, 1 << 16);
-    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e.desc_host), cap, hipHostMallocDefault));
-    e.desc_host_cap = cap;
+    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&a.host), cap, hipHostMallocDefault));
+    a.host_cap = cap;
   }
-  e.desc_dev.reserve(e.desc_host_cap);
+  a.dev.reserve(a.host_cap);
 }
 
 // Runs a batch of boxes whose sources / destinations are raw device pointers.
@@ -654,14 +672,14 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
   const Fan fan = sums_out ? make_fan(n_sums) : Fan{};
   const size_t o_out = align_up(o_sum + (sums_out ? fan_elems(fan) * 4 : 0), 256);
   const size_t total = align_up(o_out + (size_t)n_sums * 4, 256);
-  acquire_arena(e);
-  ensure_desc(e, total);
-  if (!segs.empty()) std::memcpy(e.desc_host + o_segs, segs.data(), segs.size() * sizeof(Seg));
-  if (!work.empty()) std::memcpy(e.desc_host + o_work, work.data(), work.size() * sizeof(WorkItem));
-  if (!srcs.empty()) std::memcpy(e.desc_host + o_src, srcs.data(), srcs.size() * sizeof(void*));
-  if (!dsts.empty()) std::memcpy(e.desc_host + o_dst, dsts.data(), dsts.size() * sizeof(void*));
-  HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, o_sum, hipMemcpyHostToDevice, stream));
-  uint8_t* d = e.desc_dev.p;
+  mxp_engine::Arena& ar = acquire_arena(e);
+  ensure_desc(ar, total);
+  if (!segs.empty()) std::memcpy(ar.host + o_segs, segs.data(), segs.size() * sizeof(Seg));
+  if (!work.empty()) std::memcpy(ar.host + o_work, work.data(), work.size() * sizeof(WorkItem));
+  if (!srcs.empty()) std::memcpy(ar.host + o_src, srcs.data(), srcs.size() * sizeof(void*));
+  if (!dsts.empty()) std::memcpy(ar.host + o_dst, dsts.data(), dsts.size() * sizeof(void*));
+  HIP_OK(hipMemcpyAsync(ar.dev.p, ar.host, o_sum, hipMemcpyHostToDevice, stream));
+  uint8_t* d = ar.dev.p;
   uint32_t* const fanned = reinterpret_cast<uint32_t*>(d + o_sum);
   if (sums_out) HIP_OK(launch_fill_u32(fanned, fan_elems(fan), 0u, stream));
   bool checksum_only = !boxes.empty(), widening_only = !boxes.empty();
@@ -675,11 +693,11 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
                       widening_only));
   if (sums_out && n_sums) {
     HIP_OK(launch_fold_fan(fanned, fan, 1, (uint64_t)n_sums, reinterpret_cast<uint32_t*>(d + o_out), false, stream));
-    HIP_OK(hipMemcpyAsync(e.desc_host + o_out, d + o_out, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(ar.host + o_out, d + o_out, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
-    std::memcpy(sums_out, e.desc_host + o_out, (size_t)n_sums * 4);
+    std::memcpy(sums_out, ar.host + o_out, (size_t)n_sums * 4);
   }
-  release_arena(e, stream);
+  release_arena(ar, stream);
 }
 
 // Splits an arbitrary device pointer into a 16-byte aligned base and an offset, so the
@@ -734,8 +752,8 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     }
     HIP_OK(hipEventCreate(&e->ev_a));
     HIP_OK(hipEventCreate(&e->ev_b));
-    HIP_OK(hipEventCreateWithFlags(&e->arena_busy, hipEventDisableTiming));
-    HIP_OK(hipEventCreateWithFlags(&e->items_busy, hipEventDisableTiming));
+    for (auto& a : e->arenas) HIP_OK(hipEventCreateWithFlags(&a.busy, hipEventDisableTiming));
+    for (auto& t : e->item_tabs) HIP_OK(hipEventCreateWithFlags(&t.busy, hipEventDisableTiming));
     HIP_OK(hipEventCreateWithFlags(&e->caller_ev, hipEventDisableTiming));
     e->static_dev = static_scratch_for(o.device);
     HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e->static_host), kStaticScratchBytes, hipHostMallocDefault));
@@ -1512,18 +1530,19 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
 void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hipStream_t stream) {
   uint32_t* sum_dev = nullptr;
   const Fan fan = make_fan(1);
+  mxp_engine::Arena* ar = nullptr;
   if (checksum) {
-    acquire_arena(e);
-    ensure_desc(e, fan_elems(fan) * 4);
-    sum_dev = reinterpret_cast<uint32_t*>(e.desc_dev.p);
+    ar = &acquire_arena(e);
+    ensure_desc(*ar, fan_elems(fan) * 4);
+    sum_dev = reinterpret_cast<uint32_t*>(ar->dev.p);
     HIP_OK(launch_fill_u32(sum_dev, fan_elems(fan), 0u, stream));
   }
   HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, e.opt.nan_bits, sum_dev, fan, stream));
   if (checksum) {
-    HIP_OK(hipMemcpyAsync(e.desc_host, sum_dev, fan_elems(fan) * 4, hipMemcpyDeviceToHost, stream));
+    HIP_OK(hipMemcpyAsync(ar->host, sum_dev, fan_elems(fan) * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
-    fold_fan(reinterpret_cast<const uint32_t*>(e.desc_host), fan, 1, 1, checksum);
-    release_arena(e, stream);
+    fold_fan(reinterpret_cast<const uint32_t*>(ar->host), fan, 1, 1, checksum);
+    release_arena(*ar, stream);
   }
 }
 
@@ -1597,23 +1616,24 @@ void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStr
   group_transposes(jobs, items, groups, singles);
   for (const auto& j : singles) run_transpose(e, j, nullptr, stream);
   if (groups.empty()) return;
-  if (e.items_recorded) HIP_OK(hipEventSynchronize(e.items_busy));
-  if (items.size() > e.items_cap) {
-    if (e.items_host) (void)hipHostFree(e.items_host);
-    e.items_host = nullptr;
-    e.items_cap = 0;
+  mxp_engine::ItemTable& tab = e.item_tabs[e.items_turn++ & 1u];
+  if (tab.recorded) HIP_OK(hipEventSynchronize(tab.busy));
+  if (items.size() > tab.cap) {
+    if (tab.host) (void)hipHostFree(tab.host);
+    tab.host = nullptr;
+    tab.cap = 0;
     const size_t cap = std::max<size_t>(64, items.size() * 2);
-    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&e.items_host), cap * sizeof(TransposeItem), hipHostMallocDefault));
-    e.items_cap = cap;
+    HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&tab.host), cap * sizeof(TransposeItem), hipHostMallocDefault));
+    tab.cap = cap;
   }
-  e.items_dev.reserve(e.items_cap);
-  std::memcpy(e.items_host, items.data(), items.size() * sizeof(TransposeItem));
-  HIP_OK(hipMemcpyAsync(e.items_dev.p, e.items_host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
+  tab.dev.reserve(tab.cap);
+  std::memcpy(tab.host, items.data(), items.size() * sizeof(TransposeItem));
+  HIP_OK(hipMemcpyAsync(tab.dev.p, tab.host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
   for (const TransposeGroup& g : groups)
-    HIP_OK(launch_transpose_batch(e.items_dev.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
+    HIP_OK(launch_transpose_batch(tab.dev.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
                                   e.opt.nan_bits, stream));
-  HIP_OK(hipEventRecord(e.items_busy, stream));
-  e.items_recorded = true;
+  HIP_OK(hipEventRecord(tab.busy, stream));
+  tab.recorded = true;
 }
 
 std::vector<uint64_t> strides_or_row_major(const int64_t* strides, const int64_t* shape, int32_t ndim, const char* what) {
@@ -2035,18 +2055,18 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
     const size_t o_fan = align_up(jobs.size() * sizeof(DigestJob), 256);
     const size_t o_out = align_up(o_fan + fan_elems(fan, 5) * 8, 256);
     const size_t total = o_out + (size_t)n * 5 * 8;
-    acquire_arena(e);
-    ensure_desc(e, total);
-    std::memcpy(e.desc_host + o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
-    HIP_OK(hipMemcpyAsync(e.desc_dev.p, e.desc_host, jobs.size() * sizeof(DigestJob), hipMemcpyHostToDevice, stream));
-    unsigned long long* const fanned = reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_fan);
+    mxp_engine::Arena& ar = acquire_arena(e);
+    ensure_desc(ar, total);
+    std::memcpy(ar.host + o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
+    HIP_OK(hipMemcpyAsync(ar.dev.p, ar.host, jobs.size() * sizeof(DigestJob), hipMemcpyHostToDevice, stream));
+    unsigned long long* const fanned = reinterpret_cast<unsigned long long*>(ar.dev.p + o_fan);
     HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(fanned), 2 * fan_elems(fan, 5), 0u, stream));
-    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(e.desc_dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks, fanned, fan, stream));
-    HIP_OK(launch_fold_fan(fanned, fan, 5, 5 * (uint64_t)n, reinterpret_cast<unsigned long long*>(e.desc_dev.p + o_out), false, stream));
-    HIP_OK(hipMemcpyAsync(e.desc_host + o_out, e.desc_dev.p + o_out, (size_t)n * 5 * 8, hipMemcpyDeviceToHost, stream));
+    HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(ar.dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks, fanned, fan, stream));
+    HIP_OK(launch_fold_fan(fanned, fan, 5, 5 * (uint64_t)n, reinterpret_cast<unsigned long long*>(ar.dev.p + o_out), false, stream));
+    HIP_OK(hipMemcpyAsync(ar.host + o_out, ar.dev.p + o_out, (size_t)n * 5 * 8, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
-    release_arena(e, stream);
-    const uint64_t* sums = reinterpret_cast<const uint64_t*>(e.desc_host + o_out);
+    release_arena(ar, stream);
+    const uint64_t* sums = reinterpret_cast<const uint64_t*>(ar.host + o_out);
     for (int64_t k = 0; k < n; ++k) {
       uint64_t sc[7] = {nbytes[k], sums[5 * k], sums[5 * k + 1], sums[5 * k + 2], sums[5 * k + 3], sums[5 * k + 4],
                         nbytes[k] % 4};
