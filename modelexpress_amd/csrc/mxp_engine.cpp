@@ -627,6 +627,27 @@ void pread_full(int fd, uint8_t* dst, uint64_t n, uint64_t off, const std::strin
   }
 }
 
+// Launch timing (mxp_engine_set_launch_timing): an event pair of the engine's ring around one
+// kernel launch on `stream`; nothing is recorded while the stream is being captured.
+struct LaunchTimer {
+  mxp_engine& e;
+  hipStream_t stream;
+  bool on;
+  hipEvent_t last = nullptr;
+  LaunchTimer(mxp_engine& eng, hipStream_t s) : e(eng), stream(s), on(eng.timing_on && !eng.timing_ring.empty() && !is_capturing(s)) {
+    if (!on) return;
+    const auto& pr = e.timing_ring[e.timing_count % e.timing_ring.size()];
+    last = pr.second;
+    HIP_OK(hipEventRecord(pr.first, stream));
+  }
+  void done() {
+    if (!on) return;
+    HIP_OK(hipEventRecord(last, stream));
+    ++e.timing_count;
+    on = false;
+  }
+};
+
 // The descriptor arenas (pinned staging + its device twin, two of them taken in turn) are shared
 // by the stand-alone operators.  A call may only overwrite or reallocate an arena once its
 // previous user's device work is done, whichever stream that ran on: users record the arena's
@@ -687,10 +708,12 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
     checksum_only = checksum_only && b.op == kOpChecksumOnly;
     widening_only = widening_only && op_widens(b.op);
   }
+  LaunchTimer timer(e, stream);
   HIP_OK(launch_place(reinterpret_cast<const Seg*>(d + o_segs), reinterpret_cast<const WorkItem*>(d + o_work),
                       (uint32_t)work.size(), reinterpret_cast<const void* const*>(d + o_src),
                       reinterpret_cast<void* const*>(d + o_dst), fanned, fan, e.opt.nan_bits, stream, checksum_only, nullptr, 0,
                       widening_only));
+  timer.done();
   if (sums_out && n_sums) {
     HIP_OK(launch_fold_fan(fanned, fan, 1, (uint64_t)n_sums, reinterpret_cast<uint32_t*>(d + o_out), false, stream));
     HIP_OK(hipMemcpyAsync(ar.host + o_out, d + o_out, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
@@ -1537,7 +1560,9 @@ void run_transpose(mxp_engine& e, const TransposeJob& t, uint32_t* checksum, hip
     sum_dev = reinterpret_cast<uint32_t*>(ar->dev.p);
     HIP_OK(launch_fill_u32(sum_dev, fan_elems(fan), 0u, stream));
   }
+  LaunchTimer timer(e, stream);
   HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, e.opt.nan_bits, sum_dev, fan, stream));
+  timer.done();
   if (checksum) {
     HIP_OK(hipMemcpyAsync(ar->host, sum_dev, fan_elems(fan) * 4, hipMemcpyDeviceToHost, stream));
     HIP_OK(hipStreamSynchronize(stream));
@@ -1629,9 +1654,12 @@ void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStr
   tab.dev.reserve(tab.cap);
   std::memcpy(tab.host, items.data(), items.size() * sizeof(TransposeItem));
   HIP_OK(hipMemcpyAsync(tab.dev.p, tab.host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
-  for (const TransposeGroup& g : groups)
+  for (const TransposeGroup& g : groups) {
+    LaunchTimer timer(e, stream);
     HIP_OK(launch_transpose_batch(tab.dev.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
                                   e.opt.nan_bits, stream));
+    timer.done();
+  }
   HIP_OK(hipEventRecord(tab.busy, stream));
   tab.recorded = true;
 }
