@@ -153,6 +153,10 @@ hipError_t launch_place_digest(const Seg* segs_dev, const WorkItem* work_dev, ui
 hipError_t launch_digest(const DigestJob* jobs_dev, uint32_t n_jobs, uint32_t n_blocks,
                          unsigned long long* out_dev, Fan fan, hipStream_t stream);
 hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_t stream);
+// Copies a small table (16-byte multiple, both sides 16-byte aligned) with a kernel; `src` may be
+// pinned host memory the device can address.  Stays on the launch stream's own queue, where a
+// copy call of this size costs a hand-over to a copy engine and back.
+hipError_t launch_copy_table(void* dst, const void* src, size_t bytes, hipStream_t stream);
 // Device-side fold_fan: out_dev[k] = sum over the copies of element k, k < n; with `clear` the
 // elements read are left at zero.  T is uint32_t or unsigned long long.
 template <typename T>

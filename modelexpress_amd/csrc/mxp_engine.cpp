@@ -205,7 +205,8 @@ struct mxp_engine {
   // before it uploaded into the other (back-to-back calls do not wait for each other's kernels).
   // `busy` is recorded after the last device use of an arena; whoever takes it next waits for it.
   struct Arena {
-    uint8_t* host = nullptr;  // pinned
+    uint8_t* host = nullptr;      // pinned
+    uint8_t* host_dev = nullptr;  // the address kernels read `host` at
     size_t host_cap = 0;
     DevBuf<uint8_t> dev;
     hipEvent_t busy = nullptr;
@@ -224,7 +225,8 @@ struct mxp_engine {
                                           // final address; 0 = none (mxp_engine_set_direct_placement)
   // descriptor table of batched transposes: same protocol as the arenas, also kept twice
   struct ItemTable {
-    TransposeItem* host = nullptr;  // pinned
+    TransposeItem* host = nullptr;      // pinned
+    TransposeItem* host_dev = nullptr;  // the address kernels read `host` at
     size_t cap = 0;
     DevBuf<TransposeItem> dev;
     hipEvent_t busy = nullptr;
@@ -671,8 +673,20 @@ void ensure_desc(mxp_engine::Arena& a, size_t bytes) {
     const size_t cap = align_up(bytes * 2, 1 << 16);
     HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&a.host), cap, hipHostMallocDefault));
     a.host_cap = cap;
+    HIP_OK(hipHostGetDevicePointer(reinterpret_cast<void**>(&a.host_dev), a.host, 0));
   }
   a.dev.reserve(a.host_cap);
+}
+
+// Sends the first `bytes` of an arena's pinned block to its device twin, ordered on `stream`.
+// Small tables go by a copy kernel that reads the pinned block over the bus: the launch that
+// consumes them follows on the same queue, where a copy call costs a hand-over to a copy engine
+// and back (some 15 us of stream time per operator call, measured).
+constexpr size_t kTableByKernelMax = 1u << 20;
+void upload_arena(mxp_engine::Arena& a, size_t bytes, hipStream_t stream) {
+  bytes = align_up(bytes, 16);
+  if (bytes <= kTableByKernelMax && bytes <= a.host_cap) HIP_OK(launch_copy_table(a.dev.p, a.host_dev, bytes, stream));
+  else HIP_OK(hipMemcpyAsync(a.dev.p, a.host, bytes, hipMemcpyHostToDevice, stream));
 }
 
 // Runs a batch of boxes whose sources / destinations are raw device pointers.
@@ -699,7 +713,7 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
   if (!work.empty()) std::memcpy(ar.host + o_work, work.data(), work.size() * sizeof(WorkItem));
   if (!srcs.empty()) std::memcpy(ar.host + o_src, srcs.data(), srcs.size() * sizeof(void*));
   if (!dsts.empty()) std::memcpy(ar.host + o_dst, dsts.data(), dsts.size() * sizeof(void*));
-  HIP_OK(hipMemcpyAsync(ar.dev.p, ar.host, o_sum, hipMemcpyHostToDevice, stream));
+  upload_arena(ar, o_sum, stream);
   uint8_t* d = ar.dev.p;
   uint32_t* const fanned = reinterpret_cast<uint32_t*>(d + o_sum);
   if (sums_out) HIP_OK(launch_fill_u32(fanned, fan_elems(fan), 0u, stream));
@@ -1650,10 +1664,15 @@ void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStr
     const size_t cap = std::max<size_t>(64, items.size() * 2);
     HIP_OK(hipHostMalloc(reinterpret_cast<void**>(&tab.host), cap * sizeof(TransposeItem), hipHostMallocDefault));
     tab.cap = cap;
+    HIP_OK(hipHostGetDevicePointer(reinterpret_cast<void**>(&tab.host_dev), tab.host, 0));
   }
   tab.dev.reserve(tab.cap);
   std::memcpy(tab.host, items.data(), items.size() * sizeof(TransposeItem));
-  HIP_OK(hipMemcpyAsync(tab.dev.p, tab.host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
+  static_assert(sizeof(TransposeItem) % 16 == 0, "the table copy kernel moves 16-byte units");
+  if (items.size() * sizeof(TransposeItem) <= kTableByKernelMax)
+    HIP_OK(launch_copy_table(tab.dev.p, tab.host_dev, items.size() * sizeof(TransposeItem), stream));
+  else
+    HIP_OK(hipMemcpyAsync(tab.dev.p, tab.host, items.size() * sizeof(TransposeItem), hipMemcpyHostToDevice, stream));
   for (const TransposeGroup& g : groups) {
     LaunchTimer timer(e, stream);
     HIP_OK(launch_transpose_batch(tab.dev.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
@@ -2086,7 +2105,7 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
     mxp_engine::Arena& ar = acquire_arena(e);
     ensure_desc(ar, total);
     std::memcpy(ar.host + o_jobs, jobs.data(), jobs.size() * sizeof(DigestJob));
-    HIP_OK(hipMemcpyAsync(ar.dev.p, ar.host, jobs.size() * sizeof(DigestJob), hipMemcpyHostToDevice, stream));
+    upload_arena(ar, jobs.size() * sizeof(DigestJob), stream);
     unsigned long long* const fanned = reinterpret_cast<unsigned long long*>(ar.dev.p + o_fan);
     HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(fanned), 2 * fan_elems(fan, 5), 0u, stream));
     HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(ar.dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks, fanned, fan, stream));

@@ -697,4 +697,18 @@ hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_
   return hipGetLastError();
 }
 
+// Table copy by plain 16-byte loads and stores (no memcpy node: callers may capture it).
+__global__ __launch_bounds__(256) void copy_table_kernel(uint4* __restrict__ dst, const uint4* __restrict__ src, uint64_t n16) {
+  for (uint64_t i = blockIdx.x * 256ull + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * 256ull) dst[i] = src[i];
+}
+
+hipError_t launch_copy_table(void* dst, const void* src, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  if ((bytes & 15u) || (reinterpret_cast<uintptr_t>(dst) & 15u) || (reinterpret_cast<uintptr_t>(src) & 15u)) return hipErrorInvalidValue;
+  const uint64_t n16 = bytes / 16, blocks = (n16 + 255) / 256;
+  hipLaunchKernelGGL(copy_table_kernel, dim3((uint32_t)(blocks > 1024 ? 1024 : blocks)), dim3(256), 0, stream,
+                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), n16);
+  return hipGetLastError();
+}
+
 }  // namespace mxp

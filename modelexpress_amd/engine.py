@@ -473,6 +473,12 @@ class PlacementEngine:
     def copy_views(self, views: Sequence[dict], *, stream: int = 0) -> None:
         """Many ``copy_view`` calls in one go (keys: src, dst, shape, elem_size and optionally src_strides,
         dst_strides, cast): all row / element boxes run in one launch, transposed views in one launch per element type and conversion."""
+        L.check(L.lib().mxp_copy_views(self._h, self.views_array(views), len(views), C.c_void_p(stream)))
+
+    @staticmethod
+    def views_array(views: Sequence[dict]):
+        """The ``_lib.ViewCopy`` array of ``views`` (the dicts ``copy_views`` takes), for callers that run the
+        same views again (``copy_views_array``, ``view_plan``) and need not rebuild it per call."""
         arr = (L.ViewCopy * max(1, len(views)))()
         for v, o in zip(views, arr):
             shape = [int(x) for x in v["shape"]]
@@ -484,7 +490,7 @@ class PlacementEngine:
                 setattr(o, flag, 1 if st is None else 0)
                 for d, x in enumerate(st or ()):
                     getattr(o, key)[d] = int(x)
-        L.check(L.lib().mxp_copy_views(self._h, arr, len(views), C.c_void_p(stream)))
+        return arr
 
     def copy_views_array(self, arr, n: int, *, stream: int = 0) -> None:
         """``copy_views`` on an ``_lib.ViewCopy`` array the caller built (and may keep between calls)."""
