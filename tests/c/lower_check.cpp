@@ -112,7 +112,7 @@ BoxCopy random_box(std::mt19937_64& g) {
   BoxCopy b;
   b.op = ops[g() % (sizeof ops / sizeof ops[0])];
   const uint64_t de = dst_elem(b.op), se = src_elem(b.op);
-  const int shape = (int)(g() % 4);
+  const int shape = (int)(g() % 5);
   uint64_t row_elems;
   if (shape == 0) {  // a contiguous run, sometimes long
     b.rows = 1;
@@ -123,9 +123,21 @@ BoxCopy random_box(std::mt19937_64& g) {
   } else if (shape == 2) {  // wide rows (split by columns beyond 32 KiB)
     b.rows = pick(2, 40);
     row_elems = pick(1000, 60000);
-  } else {  // aligned, power-of-two flavoured
+  } else if (shape == 3) {  // aligned, power-of-two flavoured
     b.rows = pick(1, 512);
     row_elems = 8 * pick(1, 1024);
+  } else {  // a column slice of a matrix whose row length is a multiple of 2 KiB, rows that fill whole batches
+    const uint64_t unit_elems = (op_narrows(b.op) ? 8 : 16) / de;  // elements per lane access of the wide path
+    row_elems = unit_elems << pick(0, 10);
+    const uint64_t tile_rows = std::max<uint64_t>(1, 8192 * unit_elems / row_elems);
+    b.rows = pick(tile_rows, 5 * tile_rows + 3);
+    b.row_bytes = row_elems * de;
+    const uint64_t src_row = op_src_bytes(b.op, b.row_bytes);
+    b.src_pitch = (src_row + 2047) / 2048 * 2048 + 2048 * pick(0, 3);
+    b.dst_pitch = g() % 2 ? b.row_bytes : (b.row_bytes + 2047) / 2048 * 2048 + 2048 * pick(0, 2);
+    b.dst_off = 16 * pick(0, 40);
+    b.src_off = 16 * pick(0, 40);
+    return b;
   }
   b.row_bytes = row_elems * de;
   const uint64_t src_row = op_src_bytes(b.op, b.row_bytes);

@@ -83,6 +83,12 @@ def test_llama3_8b_rank_slice_full_size(oracle, oracle_c, tmp_path, mxp):
     eng.execute_resident(plan, staged, dst)
     assert eng.checksums(plan) == fused
     assert all(torch.equal(a, b) for a, b in zip(before, dst[:8]))
+
+    # the tensor_digest sums accumulated by the placement itself equal a second pass over the finished buffers
+    eng.set_fused_digests(True)
+    eng.execute_resident(plan, staged, dst)
+    assert eng.digests(plan) == eng.digest(dst)
+    assert eng.checksums(plan) == fused
     eng.close()
 
 

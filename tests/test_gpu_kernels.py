@@ -578,3 +578,46 @@ def test_place_boxes_random_batches(gpu_engine, oracle, oracle_c, seed):
     sums = gpu_engine.place_boxes(boxes, len(boxes))
     assert np.array_equal(out.cpu().numpy(), want)
     assert sums == sums_want
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("cast", [0, 1, 2, 4, 5, 7])
+@pytest.mark.parametrize("row_bytes,src_extra,dst_pitched", [(1024, 7, False), (256, 1, True), (4096, 3, False), (16, 0, False)])
+def test_column_slices_out_of_power_of_two_pitches(gpu_engine, oracle, oracle_c, cast, row_bytes, src_extra, dst_pitched):
+    """Row gathers out of power-of-two flavoured pitches, whole batches of rows plus a ragged rest: the
+    o_proj slice of installer.py:292-317 (4096 rows of 1 KiB out of 8 KiB) and its like, also through
+    every kind of conversion, with a column offset and a pitched destination.  Bytes and checksums
+    against the oracle."""
+    rng = np.random.default_rng(cast * 131 + row_bytes)
+    narrow, widen = cast in (1, 4), cast in (2, 3, 5)
+    src_row = row_bytes * 2 if narrow else row_bytes // 2 if widen else row_bytes
+    units = row_bytes // (8 if narrow else 16)
+    tile_rows = 8192 // units
+    rows = 3 * tile_rows + tile_rows // 2 + 5  # three whole tiles and a ragged rest
+    src_pitch = (src_row + 2047) // 2048 * 2048 + 2048 * src_extra
+    dst_pitch = (row_bytes + 2047) // 2048 * 2048 + 2048 if dst_pitched else row_bytes
+    col = 3 * src_row if 4 * src_row <= src_pitch else 0
+    src = rng.integers(0, 256, rows * src_pitch, dtype=np.uint8)
+    if cast in (1, 4):  # a few NaNs, infinities and denormals among the fp32 inputs
+        w = src.view(np.uint32)
+        w[:: 977] = 0x7FC12345
+        w[5:: 1201] = 0xFF800000
+        w[7:: 1409] = 0x00000123
+    want = np.full(rows * dst_pitch + 64, 0xEE, dtype=np.uint8)
+    conv = {0: lambda s: s,
+            1: lambda s: oracle.cast_f32_bf16_bits(s.view(np.uint32)).view(np.uint8),
+            2: lambda s: oracle.cast_bf16_f32_bits(s.view(np.uint16)).view(np.uint8),
+            4: lambda s: oracle.cast_f32_f16_bits(s.view(np.uint32)).view(np.uint8),
+            5: lambda s: oracle.cast_f8e4m3_bf16_bits(s).view(np.uint8),
+            7: lambda s: oracle.cast_f32_f16_bits(oracle.cast_bf16_f32_bits(s.view(np.uint16))).view(np.uint8)}[cast]
+    csum = 0
+    for r in range(rows):
+        piece = conv(src[r * src_pitch + col: r * src_pitch + col + src_row])
+        want[32 + r * dst_pitch: 32 + r * dst_pitch + row_bytes] = piece
+        csum += int(oracle_c.checksum32(piece, first_index=77 + r * dst_pitch), 16)
+    d_src = _dev(src)
+    out = torch.full((want.size,), 0xEE, dtype=torch.uint8, device="cuda")
+    sums = gpu_engine.place_boxes([{"src": d_src.data_ptr() + col, "dst": out.data_ptr() + 32, "src_pitch": src_pitch, "dst_pitch": dst_pitch,
+                                    "rows": rows, "row_bytes": row_bytes, "csum_index": 77, "csum_group": 0, "cast": cast}], 1)
+    assert np.array_equal(out.cpu().numpy(), want)
+    assert sums == [format(csum & 0xFFFFFFFF, "08x")]
