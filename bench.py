@@ -463,7 +463,9 @@ def main() -> int:
                        "other_ranks_bytes_dropped": dropped,
                        "placed_bytes": placed, "buffers": len(plan.params),
                        "timed": "value = the device placement step with the checkpoint bytes already in HBM, one launch per "
-                                "step; the end-to-end rate from files (PCIe-bound) is roofline.e2e"},
+                                "step; the end-to-end rate from files (PCIe-bound) is roofline.e2e",
+                       "staging": "each shard file's bytes sit in one device buffer, placed so that the file's data section "
+                                  "starts on a 256-byte boundary (the address mxp_execute_resident recommends)"},
             "roofline": roofline,
         }
 

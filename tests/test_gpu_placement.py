@@ -11,8 +11,17 @@ from modelexpress_amd import synth
 pytestmark = pytest.mark.gpu
 
 
-def _stage_files(ck):
-    return [torch.from_numpy(np.fromfile(f["path"], dtype=np.uint8)).cuda() for f in ck.files()]
+def _stage_files(ck, shift=None):
+    """Every shard file's bytes in device memory, each `staging_pad` bytes (the address the library
+    recommends: data section on a 256-byte boundary) or `shift` bytes past an allocation's start."""
+    out = []
+    for f in ck.files():
+        pad = int(f["staging_pad"]) if shift is None else shift
+        host = np.fromfile(f["path"], dtype=np.uint8)
+        buf = torch.empty(host.size + pad, dtype=torch.uint8, device="cuda")
+        buf[pad:].copy_(torch.from_numpy(host))
+        out.append(buf[pad:])
+    return out
 
 
 @pytest.mark.parametrize("name", list(tiny_layouts()))
@@ -27,11 +36,12 @@ def test_families_match_oracle(name, gpu_engine, gpu_engine_band, oracle, tmp_pa
         ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
         # ingest: contiguous pieces of every size copied straight to their final address; ingest_bounce: every
         # byte through the bounce slot and the kernel; ingest_band: 64 KiB slots, row bands gathered on the device
-        for mode in ("ingest", "ingest_bounce", "ingest_band", "resident"):
+        # resident_off8: the staged files 8 bytes off the 16-byte grid (any 8-byte aligned address is accepted)
+        for mode in ("ingest", "ingest_bounce", "ingest_band", "resident", "resident_off8"):
             eng = gpu_engine_band if mode == "ingest_band" else gpu_engine
             dst = eng.allocate(plan, fill=0xAB)
-            if mode == "resident":
-                eng.execute_resident(plan, _stage_files(ck), dst)
+            if mode.startswith("resident"):
+                eng.execute_resident(plan, _stage_files(ck, 8 if mode == "resident_off8" else None), dst)
             else:
                 eng.set_direct_placement({"ingest": 1, "ingest_bounce": -1}.get(mode, 0))
                 try:
