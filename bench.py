@@ -49,7 +49,7 @@ HBM_PEAK_GBPS = 8000.0
 # counter scaled by its reading for plain device copies of known size).  Counters cannot be read
 # from inside this process, so the figure is carried here and reported only when the
 # workload is the profiled one.
-PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_099_000_000}
+PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_020_000_000}
 
 
 def _log(msg: str) -> None:
