@@ -803,6 +803,26 @@ def main() -> int:
                               "copy_, and safe_checksum as the reference writes it (int64 arange per byte)"}
         else:
             out["cpu_baseline"] = {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "skipped"}
+        # ---- the same step for the first and the last rank of the group (default run only): every rank's share has
+        # the same size, its column slices start elsewhere in each row ----
+        if args.config == 2 and not args.layers and not args.no_configs and not args.rank_local:
+            out["other_ranks"] = {}
+            for r in sorted({0, tp - 1} - {rank}):
+                rv_r = layout.rank_view(tp_size=tp, tp_rank=r)
+                plan_r = PlacementPlan(ck, rv_r.params, tp_size=tp, tp_rank=r, stacked_params_mapping=rv_r.stacked_params_mapping,
+                                       expert_mapping=rv_r.expert_mapping, allow_cast=cast)
+                dst_r = eng.allocate(plan_r, fill=0)
+                t_r = _timed_resident(eng, plan_r, staged, dst_r, 5, 2)
+                placed_r, algo_r = plan_r.totals()["placed_bytes"], plan_r.totals()["kernel_algorithmic_bytes"]
+                ok_r = eng.checksums(plan_r) == eng.checksum32(dst_r, [p.nbytes for p in plan_r.params])
+                agree = agree and ok_r
+                out["other_ranks"][f"rank{r}"] = {
+                    "placed_bytes": placed_r, "value": round(placed_r / (t_r["ms_per_step"] * 1e-3) / 1e9, 2), "unit": "GB/s",
+                    "ms_per_step": round(t_r["ms_per_step"], 4), "kernel_ms_avg": round(t_r["kernel_ms_avg"], 4),
+                    "frac_of_hbm_peak": round(algo_r / (t_r["kernel_ms_avg"] * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+                    "fused_checksums_equal_stand_alone": ok_r}
+                del dst_r
+                plan_r.close()
         out["checksums_agree"] = agree
         eng.close()
         # ---- the other four configurations, full size, HBM-resident (default run only) ----
