@@ -501,9 +501,16 @@ def main() -> int:
                 ev1.record()
                 torch.cuda.synchronize()
                 dev_ms = ev0.elapsed_time(ev1) / 10  # kernel + reduction + the host's turn-around between calls, as the stream sees them
+                eng.set_launch_timing(True)
+                for _ in range(10):
+                    fn()
+                k_times = eng.launch_times(10)
+                eng.set_launch_timing(False)
+                k_ms = sum(k_times) / len(k_times)
                 dt = res[""]
                 ops[op_name] = {"buffers": len(dst), "bytes": placed, "ms_per_call_wall": round(dt * 1e3, 4),
-                                "gbps_wall": round(placed / dt / 1e9, 1), "frac_of_hbm_peak": round(placed / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                                "gbps_wall": round(placed / dt / 1e9, 1), "frac_per_call": round(placed / dt / 1e9 / HBM_PEAK_GBPS, 4),
+                                "kernel_ms": round(k_ms, 4), "frac_of_hbm_peak": round(placed / (k_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                                 "device_ms_per_call": round(dev_ms, 4),
                                 "one_shot_ms_per_call_wall": round(res["one_shot_"] * 1e3, 4),
                                 "note": "through a verify plan (descriptors lowered once): per call one launch, a reduction of the "

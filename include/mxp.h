@@ -315,7 +315,8 @@ int mxp_engine_set_direct_placement(mxp_engine* engine, int64_t min_bytes);
  * NULL) records a HIP-event pair around its placement kernel on the launch stream and does NOT
  * synchronise, so a timed loop of K launches yields both its wall time and the K kernel
  * durations.  The stand-alone operators that launch through descriptor tables built per call
- * (mxp_cast, mxp_copy_view(s), mxp_permute_copy, mxp_place_boxes, mxp_copy_batch, mxp_checksum32)
+ * (mxp_cast, mxp_copy_view(s), mxp_permute_copy, mxp_place_boxes, mxp_copy_batch, mxp_checksum32) and the runs of a
+ * verify plan (mxp_verify_plan_checksums / _digests)
  * record a pair around each of their placement / transpose launches in the same way.  mxp_engine_launch_times waits for the launches and writes the durations (ms) of the
  * most recent min(capacity, recorded, 256) of them, oldest first.  Switching on or off restarts
  * the count.  No counterpart in the reference. */

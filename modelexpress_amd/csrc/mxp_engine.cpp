@@ -1834,9 +1834,11 @@ int mxp_verify_plan_checksums(mxp_engine* engine, mxp_verify_plan* plan, uint32_
     uint8_t* d = plan->tables.p;
     uint32_t* sums = reinterpret_cast<uint32_t*>(d + plan->o_sums);
     if (plan->cleared_rec) HIP_OK(hipStreamWaitEvent(stream, plan->cleared, 0));  // a run on another stream than the last
+    LaunchTimer timer(*engine, stream);
     HIP_OK(launch_place(reinterpret_cast<const Seg*>(d), reinterpret_cast<const WorkItem*>(d + plan->o_work), plan->n_work,
                         reinterpret_cast<const void* const*>(d + plan->o_src), nullptr, sums, plan->fan, engine->opt.nan_bits, stream,
                         true));
+    timer.done();
     // the copies are added up on the device, which leaves them cleared for the next run
     HIP_OK(launch_fold_fan(sums, plan->fan, 1, (uint64_t)plan->n, reinterpret_cast<uint32_t*>(plan->host_dev), true, stream));
     HIP_OK(hipEventRecord(plan->cleared, stream));
@@ -1856,8 +1858,10 @@ int mxp_verify_plan_digests(mxp_engine* engine, mxp_verify_plan* plan, uint8_t* 
     uint8_t* d = plan->tables.p;
     unsigned long long* dsums = reinterpret_cast<unsigned long long*>(d + plan->o_dsums);
     if (plan->cleared_rec) HIP_OK(hipStreamWaitEvent(stream, plan->cleared, 0));
+    LaunchTimer timer(*engine, stream);
     HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(d + plan->o_jobs), (uint32_t)plan->n, plan->n_blocks, dsums, plan->fan,
                          stream));
+    timer.done();
     const size_t h_off = align_up((size_t)plan->n * 4, 8);  // the 64-bit sums follow the checksums
     const uint8_t* h = plan->host + h_off;
     HIP_OK(launch_fold_fan(dsums, plan->fan, 5, 5 * (uint64_t)plan->n, reinterpret_cast<unsigned long long*>(plan->host_dev + h_off), true,
