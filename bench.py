@@ -44,12 +44,13 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes per place_kernel launch on the default workload, from the FETCH_SIZE and
-# WRITE_SIZE counter runs summarised in profiles/place_kernel_llama3_8b_tp8.txt (each
-# counter scaled by its reading for plain device copies of known size).  Counters cannot be read
+# HBM bytes per place_kernel launch on the profiled workloads, from the FETCH_SIZE and
+# WRITE_SIZE counter runs summarised under profiles/ (each counter scaled by its reading
+# for plain device copies of known size).  Counters cannot be read
 # from inside this process, so the figure is carried here and reported only when the
 # workload is the profiled one.
-PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_020_000_000}
+PROFILED_TRAFFIC_BYTES = {("llama", 32, 8, False): 4_020_000_000,   # profiles/place_kernel_llama3_8b_tp8.txt
+                          ("llama", 32, 8, True): 6_030_000_000}    # profiles/place_kernel_cast_llama3_8b_refit.txt
 
 
 def _log(msg: str) -> None:
