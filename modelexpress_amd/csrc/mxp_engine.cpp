@@ -729,10 +729,12 @@ void run_boxes(mxp_engine& e, const std::vector<BoxCopy>& boxes, const std::vect
                       widening_only));
   timer.done();
   if (sums_out && n_sums) {
-    HIP_OK(launch_fold_fan(fanned, fan, 1, (uint64_t)n_sums, reinterpret_cast<uint32_t*>(d + o_out), false, stream));
-    HIP_OK(hipMemcpyAsync(ar.host + o_out, d + o_out, (size_t)n_sums * 4, hipMemcpyDeviceToHost, stream));
-    HIP_OK(hipStreamSynchronize(stream));
+    // the kernel that adds the copies up stores the totals straight into the pinned block: no copy back
+    HIP_OK(launch_fold_fan(fanned, fan, 1, (uint64_t)n_sums, reinterpret_cast<uint32_t*>(ar.host_dev + o_out), false, stream));
+    release_arena(ar, stream);
+    HIP_OK(wait_event_promptly(ar.busy));
     std::memcpy(sums_out, ar.host + o_out, (size_t)n_sums * 4);
+    return;
   }
   release_arena(ar, stream);
 }
@@ -2113,10 +2115,9 @@ int mxp_digest(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbyt
     unsigned long long* const fanned = reinterpret_cast<unsigned long long*>(ar.dev.p + o_fan);
     HIP_OK(launch_fill_u32(reinterpret_cast<uint32_t*>(fanned), 2 * fan_elems(fan, 5), 0u, stream));
     HIP_OK(launch_digest(reinterpret_cast<const DigestJob*>(ar.dev.p + o_jobs), (uint32_t)n, (uint32_t)blocks, fanned, fan, stream));
-    HIP_OK(launch_fold_fan(fanned, fan, 5, 5 * (uint64_t)n, reinterpret_cast<unsigned long long*>(ar.dev.p + o_out), false, stream));
-    HIP_OK(hipMemcpyAsync(ar.host + o_out, ar.dev.p + o_out, (size_t)n * 5 * 8, hipMemcpyDeviceToHost, stream));
-    HIP_OK(hipStreamSynchronize(stream));
+    HIP_OK(launch_fold_fan(fanned, fan, 5, 5 * (uint64_t)n, reinterpret_cast<unsigned long long*>(ar.host_dev + o_out), false, stream));
     release_arena(ar, stream);
+    HIP_OK(wait_event_promptly(ar.busy));
     const uint64_t* sums = reinterpret_cast<const uint64_t*>(ar.host + o_out);
     for (int64_t k = 0; k < n; ++k) {
       uint64_t sc[7] = {nbytes[k], sums[5 * k], sums[5 * k + 1], sums[5 * k + 2], sums[5 * k + 3], sums[5 * k + 4],
