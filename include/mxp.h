@@ -480,6 +480,15 @@ int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dst
 /* Measured pinned host -> device bandwidth of this box in bytes per second
  * (hipMemcpyAsync of `bytes` from a pinned buffer, best of `repeats`). */
 int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double* bytes_per_second);
+/* What this box's memory system gives an access shape, measured with a bare kernel that has the
+ * placement kernel's workgroup shape and nothing else (no descriptor tables, no checksum, no
+ * conversion): `rows` rows of `row_bytes` bytes (a multiple of 16, at most 32 KiB), `src_pitch`
+ * bytes apart (a multiple of 16; == row_bytes for a contiguous copy), `col_offset` bytes into each
+ * pitch, gathered into a contiguous destination; the source buffer is filled with a seeded pattern.
+ * Writes bytes moved (read + written) per second, best of `repeats` launches.  Allocates and frees
+ * both buffers.  No counterpart in the reference: the library's own kernels are compared with it. */
+int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, uint64_t src_pitch, uint32_t col_offset,
+                       int32_t repeats, double* bytes_per_second);
 
 /* ---- host-only helpers ---------------------------------------------------- */
 /* blake2b-128 over the scalar list tensor_digest would hash (verify.py:152-155). */

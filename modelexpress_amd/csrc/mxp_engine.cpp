@@ -2171,6 +2171,59 @@ int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double*
   });
 }
 
+int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, uint64_t src_pitch, uint32_t col_offset,
+                       int32_t repeats, double* bytes_per_second) {
+  return guard([&] {
+    if (!engine || !bytes_per_second || rows == 0 || row_bytes == 0 || row_bytes % 16 || row_bytes > 32768 || src_pitch % 16 ||
+        col_offset % 16 || (uint64_t)col_offset + row_bytes > src_pitch || src_pitch >= (1ull << 31))
+      throw Error(MXP_ERR_ARG, "mxp_measure_gather: bad argument");
+    mxp_engine& e = *engine;
+    HIP_OK(hipSetDevice(e.opt.device));
+    if (repeats < 1) repeats = 1;
+    const uint32_t upr = row_bytes / 16;
+    const uint32_t rpt = (uint32_t)std::min<uint64_t>(rows, (uint64_t)kPlaceThreads * kPlaceBatch / upr);
+    const uint64_t n_tiles = rows / rpt;
+    if (n_tiles == 0 || n_tiles > 0x7FFFFFFFull) throw Error(MXP_ERR_ARG, "mxp_measure_gather: bad argument");
+    const uint64_t used_rows = n_tiles * rpt, src_bytes = used_rows * src_pitch, dst_bytes = used_rows * row_bytes;
+    DevBuf<uint8_t> src, dst;
+    src.reserve(src_bytes);
+    dst.reserve(dst_bytes);
+    HIP_OK(launch_synth(src.p, src_bytes / 2, MXP_DTYPE_BF16, 0u, 0x6a7468ull, e.streams[0]));
+    float best = 1e30f;
+    for (int r = 0; r < repeats + 1; ++r) {
+      HIP_OK(hipEventRecord(e.ev_a, e.streams[0]));
+      HIP_OK(launch_probe_gather(src.p + col_offset, dst.p, upr, (uint32_t)src_pitch, rpt, (uint32_t)n_tiles, e.streams[0]));
+      HIP_OK(hipEventRecord(e.ev_b, e.streams[0]));
+      HIP_OK(hipEventSynchronize(e.ev_b));
+      float ms = 0;
+      HIP_OK(hipEventElapsedTime(&ms, e.ev_a, e.ev_b));
+      if (r > 0 && ms < best) best = ms;  // the first launch warms up
+    }
+    // The probe is only worth its figure if it moved the right bytes: the library's own gather of
+    // the same rows (checksummed as it stores) must leave the checksum the probe's output has.
+    {
+      DevBuf<uint8_t> again;
+      again.reserve(dst_bytes);
+      BoxCopy g;
+      g.src_off = col_offset;
+      g.src_pitch = src_pitch;
+      g.dst_pitch = row_bytes;
+      g.rows = used_rows;
+      g.row_bytes = row_bytes;
+      g.csum_slot = 0;
+      uint32_t want = 0, got = 0;
+      run_boxes(e, {g}, {src.p}, {again.p}, 1, &want, e.streams[0]);
+      BoxCopy c;
+      c.row_bytes = dst_bytes;
+      c.op = kOpChecksumOnly;
+      c.csum_slot = 0;
+      run_boxes(e, {c}, {dst.p}, {}, 1, &got, e.streams[0]);
+      if (want != got) throw Error(MXP_ERR_STATE, "mxp_measure_gather: the probe kernel and the placement kernel disagree");
+    }
+    *bytes_per_second = 2.0 * (double)dst_bytes / ((double)best * 1e-3);
+  });
+}
+
 int mxp_synth_host(void* dst, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed, int32_t threads) {
   return guard([&] {
     if (n_elems && !dst) throw Error(MXP_ERR_ARG, "mxp_synth_host: null dst");

@@ -169,4 +169,67 @@ void synth_host(void* dst, uint64_t n_elems, uint32_t dtype_code, uint32_t kind,
   for (auto& th : pool) th.join();
 }
 
+// ---------------------------------------------------------------------------
+// Measurement support: a bare row gather with the placement kernel's workgroup shape (1024 lanes,
+// eight 16-byte units per lane, all loads before all stores, non-temporal accesses, one workgroup
+// per compute unit) and nothing else - no descriptor tables, no checksum, no conversion.  What it
+// reaches for an access shape on a given box is what the memory system gives that shape; the
+// library's kernels are compared with it (mxp_measure_gather).
+// ---------------------------------------------------------------------------
+namespace {
+typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kProbeThreads = 1024, kProbeBatch = 8;
+
+__global__ __launch_bounds__(kProbeThreads) void probe_gather_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                                     uint32_t units_per_row, uint32_t magic, uint32_t src_pitch,
+                                                                     uint32_t rows_per_tile) {
+  const uint64_t t = blockIdx.x;
+  const uint8_t* s = src + t * rows_per_tile * (uint64_t)src_pitch;
+  uint8_t* d = dst + t * rows_per_tile * (uint64_t)units_per_row * 16u;
+  const uint32_t n_units = rows_per_tile * units_per_row;
+  probe_u32x4 a[kProbeBatch];
+  uint32_t so[kProbeBatch], d_o[kProbeBatch];
+  bool ok[kProbeBatch];
+#pragma unroll
+  for (int k = 0; k < kProbeBatch; ++k) {
+    const uint32_t v0 = threadIdx.x + (uint32_t)k * kProbeThreads;
+    ok[k] = v0 < n_units;
+    const uint32_t v = ok[k] ? v0 : 0u;
+    const uint32_t row = units_per_row == 1u ? v : __umulhi(v, magic);
+    const uint32_t col = v - row * units_per_row;
+    so[k] = row * src_pitch + col * 16u;
+    d_o[k] = v * 16u;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int k = 0; k < kProbeBatch; ++k) a[k] = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(s + so[k]));
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int k = 0; k < kProbeBatch; ++k)
+    if (ok[k]) __builtin_nontemporal_store(a[k], reinterpret_cast<probe_u32x4*>(d + d_o[k]));
+}
+}  // namespace
+
+// Gathers n_tiles * rows_per_tile rows of units_per_row * 16 bytes, `src_pitch` bytes apart, into a
+// contiguous destination.  rows_per_tile * units_per_row <= 8192; both buffers 16-byte aligned.
+hipError_t launch_probe_gather(const void* src, void* dst, uint32_t units_per_row, uint32_t src_pitch, uint32_t rows_per_tile,
+                               uint32_t n_tiles, hipStream_t stream) {
+  if (n_tiles == 0) return hipSuccess;
+  if (units_per_row == 0 || rows_per_tile == 0 || (uint64_t)rows_per_tile * units_per_row > (uint64_t)kProbeThreads * kProbeBatch ||
+      (uint64_t)rows_per_tile * src_pitch >= (1ull << 32) || src_pitch % 16u)
+    return hipErrorInvalidValue;
+  constexpr int kOnePerCu = 96 * 1024;  // more than half a compute unit's LDS: one resident workgroup
+  static bool configured = false;
+  if (!configured) {
+    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(probe_gather_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, kOnePerCu); e != hipSuccess)
+      return e;
+    configured = true;
+  }
+  const uint32_t magic = units_per_row > 1 ? (uint32_t)((1ull << 32) / units_per_row) + 1u : 0u;
+  hipLaunchKernelGGL(probe_gather_kernel, dim3(n_tiles), dim3(kProbeThreads), kOnePerCu, stream, static_cast<const uint8_t*>(src),
+                     static_cast<uint8_t*>(dst), units_per_row, magic, src_pitch, rows_per_tile);
+  return hipGetLastError();
+}
+
 }  // namespace mxp

@@ -621,3 +621,19 @@ def test_column_slices_out_of_power_of_two_pitches(gpu_engine, oracle, oracle_c,
                                     "rows": rows, "row_bytes": row_bytes, "csum_index": 77, "csum_group": 0, "cast": cast}], 1)
     assert np.array_equal(out.cpu().numpy(), want)
     assert sums == [format(csum & 0xFFFFFFFF, "08x")]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,row_bytes,pitch,col", [(4096, 8192, None, 0), (8192, 1024, 8192, 3072), (2341, 3584, 28672, 10752),
+                                                      (100000, 64, 512, 192), (7, 16, 48, 32)])
+def test_bare_gather_probe_moves_what_the_placement_kernel_moves(gpu_engine, mxp, rows, row_bytes, pitch, col):
+    """``mxp_measure_gather`` times a bare kernel on an access shape; before it reports a rate it checks
+    its own output against the placement kernel's gather of the same rows (it fails with MXP_ERR_STATE
+    otherwise), so a positive figure here means the probe moved the right bytes."""
+    rate = gpu_engine.measure_gather(rows, row_bytes, pitch, col, repeats=2)
+    assert rate > 0
+    with pytest.raises(mxp.MxpError):
+        gpu_engine.measure_gather(16, 24, 64)  # rows that are not a multiple of 16 bytes
+    with pytest.raises(mxp.MxpError):
+        gpu_engine.measure_gather(16, 64, 96, 48)  # the column runs past the pitch
+
