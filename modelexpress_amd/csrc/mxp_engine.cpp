@@ -326,6 +326,11 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
     uint64_t rows = 1, file_pitch = 0;  // rows > 1: strided in the file, packed in the slot
   };
   std::vector<Piece> pieces;
+  // A strided row packed by a reader costs a read call of its own, about as much as copying a page:
+  // towards a chunk's capacity it counts as at least 4 KiB, so a chunk of 1 KiB rows holds a quarter
+  // of the rows it has room for and the readers share such tensors more evenly (the end-to-end rate
+  // of the Llama rank rose from 94.7-96.6 % to 95.4-98.4 % of pinned H2D in same-box runs).
+  constexpr uint64_t kPackedRowCost = 4096;
   const uint64_t slot = L->direct_io ? eng.opt.slot_bytes - 2 * blk : eng.opt.slot_bytes;
   for (const auto& w : pl.writes) {
     const TensorRec& t = ck.tensors[w.tensor];
@@ -356,7 +361,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       // strided source, packed by the readers: only the needed bytes cross PCIe and the
       // slot holds the rows back to back, so the device sees a plain copy
       if (row_src > slot) throw Error(MXP_ERR_UNSUPPORTED, "a source row of '" + t.name + "' does not fit a staging slot");
-      const uint64_t max_rows = slot / row_src;
+      const uint64_t max_rows = slot / std::max<uint64_t>(row_src, kPackedRowCost);
       for (uint64_t r = 0; r < w.rows; r += max_rows) {
         const uint64_t nr = std::min(max_rows, w.rows - r);
         Piece p{t.file_index, t0 + r * w.src_pitch, row_src, b, nr, w.src_pitch};
@@ -393,6 +398,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
     std::vector<Seg> segs;
     std::vector<WorkItem> work;
     Chunk cur;
+    uint64_t cur_cost = 0;
     auto close = [&] {
       if (cur.ranges.empty()) return;
       cur.seg_count = (uint32_t)segs.size() - cur.seg_begin;
@@ -401,6 +407,7 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       for (const auto& r : cur.bounce_runs) L->h2d_bytes += r.second;
       L->chunks.push_back(cur);
       cur = Chunk();
+      cur_cost = 0;
     };
     // Chunk capacity ramps up: every reader thread starts on a small chunk, so the first
     // host-to-device copy is issued after a 2 MiB read instead of a whole slot's, and the
@@ -461,10 +468,12 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
           p.nbytes = a1 - a0;
         }
         const uint64_t in_slot = p.nbytes * p.rows;
-        if (!cur.ranges.empty() && at + in_slot > cap) {
+        const uint64_t piece_cost = p.rows > 1 ? p.rows * std::max<uint64_t>(p.nbytes, kPackedRowCost) : in_slot;
+        if (!cur.ranges.empty() && (at + in_slot > cap || cur_cost + piece_cost > cap)) {
           close();
           at = 0;
         }
+        cur_cost += piece_cost;
         if (at + in_slot > eng.opt.slot_bytes) throw Error(MXP_ERR_STATE, "internal: a piece does not fit a staging slot");
         if (cur.ranges.empty()) {
           cur.seg_begin = (uint32_t)segs.size();
