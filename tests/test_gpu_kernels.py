@@ -637,3 +637,44 @@ def test_bare_gather_probe_moves_what_the_placement_kernel_moves(gpu_engine, mxp
     with pytest.raises(mxp.MxpError):
         gpu_engine.measure_gather(16, 64, 96, 48)  # the column runs past the pitch
 
+
+@pytest.mark.gpu
+def test_operator_calls_back_to_back_on_two_streams_keep_their_own_tables(gpu_engine):
+    """Stand-alone operator calls take their descriptor tables from two staging arenas in turn and do not
+    wait for each other's kernels: sixty calls of changing shapes, alternating between two streams with
+    nothing synchronised in between, must each move exactly their own rows (a table overwritten under a
+    running launch, or read before its upload, would show up as rows from another call's geometry)."""
+    rng = np.random.default_rng(99)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    src = torch.from_numpy(rng.integers(0, 256, 80 << 20, dtype=np.uint8)).cuda()
+    torch.cuda.synchronize()
+    calls = []
+    for k in range(60):
+        rows = int(rng.choice([1, 3, 64, 500, 2048]))
+        row_bytes = int(rng.choice([16, 48, 1024, 3584, 8192]))
+        pitch = row_bytes + 16 * int(rng.integers(0, 9)) if rows > 1 else row_bytes
+        first = 16 * int(rng.integers(0, 1000))
+        big = k % 7 == 0  # some calls long enough for the next ones to be issued while they run
+        if big:
+            rows, row_bytes, pitch = 8192, 4096, 8192
+        assert first + (rows - 1) * pitch + row_bytes <= src.numel()  # the library is handed raw addresses: bounds are the caller's
+        out = torch.full((rows * row_bytes,), 0xEE, dtype=torch.uint8, device="cuda")
+        st = streams[k % 2]
+        with torch.cuda.stream(st):
+            if k % 3 == 2 and row_bytes % 2 == 0 and rows > 1:  # a transposed view: the other launch path and its own table
+                n_el = row_bytes // 2
+                gpu_engine.copy_view(src[first:], out, (n_el, rows), 2, src_strides=(1, pitch // 2), stream=st.cuda_stream, checksum=False)
+                calls.append(("t", first, rows, n_el, pitch, out))
+            else:
+                gpu_engine.copy_view(src[first:], out, (rows, row_bytes), 1, src_strides=(pitch, 1), stream=st.cuda_stream, checksum=False)
+                calls.append(("g", first, rows, row_bytes, pitch, out))
+    torch.cuda.synchronize()
+    host = src.cpu().numpy()
+    for kind, first, rows, width, pitch, out in calls:
+        got = out.cpu().numpy()
+        if kind == "g":
+            want = np.lib.stride_tricks.as_strided(host[first:], (rows, width), (pitch, 1)).reshape(-1)
+        else:
+            want = np.lib.stride_tricks.as_strided(host[first:].view(np.uint16), (width, rows), (2, pitch)).reshape(-1).view(np.uint8)
+        assert np.array_equal(got, want), (kind, first, rows, width, pitch)
+
