@@ -463,13 +463,15 @@ def main() -> int:
             for wr in plan.writes():
                 strided = wr.rows > 1 and wr.src_pitch != wr.row_bytes and wr.dst_pitch == wr.row_bytes and wr.row_bytes % 16 == 0 \
                     and wr.row_bytes <= 32768 and wr.src_pitch % 16 == 0
-                key = (wr.row_bytes, wr.src_pitch, wr.src_offset % wr.src_pitch // 16 * 16) if strided else None
+                contiguous = wr.rows == 1 or (wr.src_pitch == wr.row_bytes and wr.dst_pitch == wr.row_bytes)
+                key = (wr.row_bytes, wr.src_pitch, wr.src_offset % wr.src_pitch // 16 * 16) if strided else None if contiguous else "other"
                 shapes[key] = shapes.get(key, 0) + wr.rows * wr.row_bytes
             if len(shapes) <= 6:
                 limits, t_total = {}, 0.0
-                for key, nbytes in sorted(shapes.items(), key=lambda kv: -kv[1]):
-                    if key is None:
-                        rate, label = eng.measure_gather(GiB // 8192, 8192), "contiguous runs"
+                for key, nbytes in sorted(shapes.items(), key=lambda kv: -kv[1]):  # by share of the bytes
+                    if key is None or key == "other":
+                        rate = eng.measure_gather(GiB // 8192, 8192)
+                        label = "contiguous runs" if key is None else "strided shapes the probe does not cover (priced as contiguous)"
                     else:
                         rb, pitch, col = key
                         rate, label = eng.measure_gather(GiB // rb, rb, pitch, col), f"rows of {rb} B out of {pitch} B at column byte {col}"
