@@ -453,40 +453,6 @@ def main() -> int:
                     "device_ms_per_step_is": "one HIP-event pair around the K timed launches / K (kernel + dispatch gap)",
                     "algorithmic_bytes": algo, "workgroups": info["n_workgroups"], "segments": info["n_segments"]}
 
-        if not args.no_ops and not cast:
-            # What the memory system of this box gives the access shapes of this workload to a bare kernel (no descriptor
-            # tables, no checksum): the ceiling the placement kernel is held against, measured in the same run.  One probe
-            # per shape of write (contiguous; each distinct strided row length / pitch / column offset), 1 GiB written each,
-            # and their composite: the rate at which the bare kernel would move this workload's bytes.
-            GiB = 1 << 30
-            shapes = {}
-            for wr in plan.writes():
-                strided = wr.rows > 1 and wr.src_pitch != wr.row_bytes and wr.dst_pitch == wr.row_bytes and wr.row_bytes % 16 == 0 \
-                    and wr.row_bytes <= 32768 and wr.src_pitch % 16 == 0
-                contiguous = wr.rows == 1 or (wr.src_pitch == wr.row_bytes and wr.dst_pitch == wr.row_bytes)
-                key = (wr.row_bytes, wr.src_pitch, wr.src_offset % wr.src_pitch // 16 * 16) if strided else None if contiguous else "other"
-                shapes[key] = shapes.get(key, 0) + wr.rows * wr.row_bytes
-            try:
-                if len(shapes) > 6:
-                    raise ValueError(f"{len(shapes)} shapes of write: more than this leg probes")
-                limits, t_total = {}, 0.0
-                for key, nbytes in sorted(shapes.items(), key=lambda kv: -kv[1]):  # by share of the bytes
-                    if key is None or key == "other":
-                        rate = eng.measure_gather(GiB // 8192, 8192)
-                        label = "contiguous runs" if key is None else "strided shapes the probe does not cover (priced as contiguous)"
-                    else:
-                        rb, pitch, col = key
-                        rate, label = eng.measure_gather(GiB // rb, rb, pitch, col), f"rows of {rb} B out of {pitch} B at column byte {col}"
-                    limits[label] = {"share_of_placed_bytes": round(nbytes / placed, 4), "frac_of_hbm_peak": round(rate / 1e9 / HBM_PEAK_GBPS, 4)}
-                    t_total += 2 * nbytes / rate
-                roofline["memory_system_limits"] = {
-                    "what": "fraction of HBM peak that a bare kernel with the placement kernel's workgroup shape (no descriptor "
-                            "tables, no checksum) reaches on each shape of write of this workload, 1 GiB written per probe, "
-                            "and the bytes-weighted composite of those rates",
-                    "shapes": limits, "composite_frac_of_hbm_peak": round(2 * placed / t_total / 1e9 / HBM_PEAK_GBPS, 4)}
-            except Exception as exc:  # noqa: BLE001 - a probe must not lose the headline line
-                roofline["memory_system_limits"] = {"skipped": f"{type(exc).__name__}: {exc}"}
-
         out = {
             "metric": "placed-weight GB/s into HBM end-to-end + kernel HBM GB/s vs peak, Llama-3-8B",
             "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -845,6 +811,43 @@ def main() -> int:
                               "copy_, and safe_checksum as the reference writes it (int64 arange per byte)"}
         else:
             out["cpu_baseline"] = {"value": None, "unit": "GB/s", "cores": 0, "kind": "port", "sample": "skipped"}
+        # (This leg allocates and frees several GiB per probe.  It runs after the ingest legs on purpose: for a few hundred
+        # milliseconds after a free of that size the platform does work of its own on the copy engines, and an ingest
+        # measured then ran at 50 GB/s instead of 56.)
+        if not args.no_ops and not cast:
+            # What the memory system of this box gives the access shapes of this workload to a bare kernel (no descriptor
+            # tables, no checksum): the ceiling the placement kernel is held against, measured in the same run.  One probe
+            # per shape of write (contiguous; each distinct strided row length / pitch / column offset), 1 GiB written each,
+            # and their composite: the rate at which the bare kernel would move this workload's bytes.
+            GiB = 1 << 30
+            shapes = {}
+            for wr in plan.writes():
+                strided = wr.rows > 1 and wr.src_pitch != wr.row_bytes and wr.dst_pitch == wr.row_bytes and wr.row_bytes % 16 == 0 \
+                    and wr.row_bytes <= 32768 and wr.src_pitch % 16 == 0
+                contiguous = wr.rows == 1 or (wr.src_pitch == wr.row_bytes and wr.dst_pitch == wr.row_bytes)
+                key = (wr.row_bytes, wr.src_pitch, wr.src_offset % wr.src_pitch // 16 * 16) if strided else None if contiguous else "other"
+                shapes[key] = shapes.get(key, 0) + wr.rows * wr.row_bytes
+            try:
+                if len(shapes) > 6:
+                    raise ValueError(f"{len(shapes)} shapes of write: more than this leg probes")
+                limits, t_total = {}, 0.0
+                for key, nbytes in sorted(shapes.items(), key=lambda kv: -kv[1]):  # by share of the bytes
+                    if key is None or key == "other":
+                        rate = eng.measure_gather(GiB // 8192, 8192)
+                        label = "contiguous runs" if key is None else "strided shapes the probe does not cover (priced as contiguous)"
+                    else:
+                        rb, pitch, col = key
+                        rate, label = eng.measure_gather(GiB // rb, rb, pitch, col), f"rows of {rb} B out of {pitch} B at column byte {col}"
+                    limits[label] = {"share_of_placed_bytes": round(nbytes / placed, 4), "frac_of_hbm_peak": round(rate / 1e9 / HBM_PEAK_GBPS, 4)}
+                    t_total += 2 * nbytes / rate
+                roofline["memory_system_limits"] = {
+                    "what": "fraction of HBM peak that a bare kernel with the placement kernel's workgroup shape (no descriptor "
+                            "tables, no checksum) reaches on each shape of write of this workload, 1 GiB written per probe, "
+                            "and the bytes-weighted composite of those rates",
+                    "shapes": limits, "composite_frac_of_hbm_peak": round(2 * placed / t_total / 1e9 / HBM_PEAK_GBPS, 4)}
+            except Exception as exc:  # noqa: BLE001 - a probe must not lose the headline line
+                roofline["memory_system_limits"] = {"skipped": f"{type(exc).__name__}: {exc}"}
+
         # ---- the same step for the first and the last rank of the group (default run only): every rank's share has
         # the same size, its column slices start elsewhere in each row ----
         if args.config == 2 and not args.layers and not args.no_configs and not args.rank_local:
