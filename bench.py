@@ -250,6 +250,56 @@ def _fs_type(path: str) -> str:
     return kind
 
 
+def _memory_system_limits(eng, plan, placed: int) -> dict:
+    """What the memory system of this box gives the access shapes of a workload to a bare kernel (no descriptor
+    tables, no checksum): the ceiling the placement kernel is held against, measured in the same run.  One probe
+    per shape of write (contiguous; each distinct strided row length / pitch / column offset; as they are or
+    narrowed from fp32 to bf16), 1 GiB written each, and their composite: the rate at which the bare kernel would
+    move this workload's bytes."""
+    from modelexpress_amd.engine import CAST_CODES
+
+    GiB = 1 << 30
+    F32_BF16 = CAST_CODES[("F32", "BF16")]
+    shapes = {}
+    for wr in plan.writes():
+        ratio = 2 if wr.cast == F32_BF16 else 1  # source bytes per destination byte
+        src_row = wr.row_bytes * ratio
+        probed = wr.cast in (0, F32_BF16)
+        contiguous = wr.rows == 1 or (wr.src_pitch == src_row and wr.dst_pitch == wr.row_bytes)
+        strided = probed and not contiguous and wr.dst_pitch == wr.row_bytes and wr.row_bytes % 16 == 0 and src_row <= 32768 \
+            and wr.src_pitch % 16 == 0
+        if strided:
+            key = (wr.cast, wr.row_bytes, wr.src_pitch, wr.src_offset % wr.src_pitch // 16 * 16)
+        else:
+            key = (wr.cast, None) if (probed and contiguous) else "other"
+        entry = shapes.setdefault(key, [0, 0])
+        entry[0] += wr.rows * wr.row_bytes                # destination bytes
+        entry[1] += wr.rows * wr.row_bytes * (1 + ratio)  # bytes moved
+    try:
+        if len(shapes) > 8:
+            raise ValueError(f"{len(shapes)} shapes of write: more than this leg probes")
+        limits, t_total, moved_total = {}, 0.0, 0
+        for key, (nbytes, moved) in sorted(shapes.items(), key=lambda kv: -kv[1][0]):  # by share of the bytes
+            if key == "other":
+                rate, label = eng.measure_gather(GiB // 8192, 8192), "shapes the probe does not cover (priced as a contiguous copy)"
+            elif key[1] is None:
+                rate = eng.measure_gather(GiB // 8192, 8192, cast=key[0])
+                label = "contiguous runs" + (", fp32 -> bf16" if key[0] else "")
+            else:
+                c, rb, pitch, col = key
+                rate = eng.measure_gather(GiB // rb, rb, pitch, col, cast=c)
+                label = f"rows of {rb} B out of {pitch} B at column byte {col}" + (" (fp32 source rows of twice that, stored as bf16)" if c else "")
+            limits[label] = {"share_of_placed_bytes": round(nbytes / placed, 4), "frac_of_hbm_peak": round(rate / 1e9 / HBM_PEAK_GBPS, 4)}
+            t_total += moved / rate
+            moved_total += moved
+        return {"what": "fraction of HBM peak that a bare kernel with the placement kernel's workgroup shape (no descriptor "
+                        "tables, no checksum) reaches on each shape of write of this workload, 1 GiB written per probe, "
+                        "and the composite of those rates weighted by the bytes each shape moves",
+                "shapes": limits, "composite_frac_of_hbm_peak": round(moved_total / t_total / 1e9 / HBM_PEAK_GBPS, 4)}
+    except Exception as exc:  # noqa: BLE001 - a probe must not lose the line it belongs to
+        return {"skipped": f"{type(exc).__name__}: {exc}"}
+
+
 def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int = 2) -> dict:
     """One of the other benchmark configurations at full size, HBM-resident: headers on disk only, the
     checkpoint bytes generated on the device, a few timed launches, and the fused checksums compared with
@@ -295,6 +345,7 @@ def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int
                             "unit": "GB/s", "frac": round(algo / (k_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                             "algorithmic_bytes": algo, "kernel": "place_kernel"},
                "checksums_agree": fused == alone}
+        out["roofline"]["memory_system_limits"] = _memory_system_limits(eng, plan, placed)
         eng.close()
         plan.close()
         ck.close()
@@ -814,39 +865,8 @@ def main() -> int:
         # (This leg allocates and frees several GiB per probe.  It runs after the ingest legs on purpose: for a few hundred
         # milliseconds after a free of that size the platform does work of its own on the copy engines, and an ingest
         # measured then ran at 50 GB/s instead of 56.)
-        if not args.no_ops and not cast:
-            # What the memory system of this box gives the access shapes of this workload to a bare kernel (no descriptor
-            # tables, no checksum): the ceiling the placement kernel is held against, measured in the same run.  One probe
-            # per shape of write (contiguous; each distinct strided row length / pitch / column offset), 1 GiB written each,
-            # and their composite: the rate at which the bare kernel would move this workload's bytes.
-            GiB = 1 << 30
-            shapes = {}
-            for wr in plan.writes():
-                strided = wr.rows > 1 and wr.src_pitch != wr.row_bytes and wr.dst_pitch == wr.row_bytes and wr.row_bytes % 16 == 0 \
-                    and wr.row_bytes <= 32768 and wr.src_pitch % 16 == 0
-                contiguous = wr.rows == 1 or (wr.src_pitch == wr.row_bytes and wr.dst_pitch == wr.row_bytes)
-                key = (wr.row_bytes, wr.src_pitch, wr.src_offset % wr.src_pitch // 16 * 16) if strided else None if contiguous else "other"
-                shapes[key] = shapes.get(key, 0) + wr.rows * wr.row_bytes
-            try:
-                if len(shapes) > 6:
-                    raise ValueError(f"{len(shapes)} shapes of write: more than this leg probes")
-                limits, t_total = {}, 0.0
-                for key, nbytes in sorted(shapes.items(), key=lambda kv: -kv[1]):  # by share of the bytes
-                    if key is None or key == "other":
-                        rate = eng.measure_gather(GiB // 8192, 8192)
-                        label = "contiguous runs" if key is None else "strided shapes the probe does not cover (priced as contiguous)"
-                    else:
-                        rb, pitch, col = key
-                        rate, label = eng.measure_gather(GiB // rb, rb, pitch, col), f"rows of {rb} B out of {pitch} B at column byte {col}"
-                    limits[label] = {"share_of_placed_bytes": round(nbytes / placed, 4), "frac_of_hbm_peak": round(rate / 1e9 / HBM_PEAK_GBPS, 4)}
-                    t_total += 2 * nbytes / rate
-                roofline["memory_system_limits"] = {
-                    "what": "fraction of HBM peak that a bare kernel with the placement kernel's workgroup shape (no descriptor "
-                            "tables, no checksum) reaches on each shape of write of this workload, 1 GiB written per probe, "
-                            "and the bytes-weighted composite of those rates",
-                    "shapes": limits, "composite_frac_of_hbm_peak": round(2 * placed / t_total / 1e9 / HBM_PEAK_GBPS, 4)}
-            except Exception as exc:  # noqa: BLE001 - a probe must not lose the headline line
-                roofline["memory_system_limits"] = {"skipped": f"{type(exc).__name__}: {exc}"}
+        if not args.no_ops:
+            roofline["memory_system_limits"] = _memory_system_limits(eng, plan, placed)
 
         # ---- the same step for the first and the last rank of the group (default run only): every rank's share has
         # the same size, its column slices start elsewhere in each row ----

@@ -485,10 +485,12 @@ int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double*
  * conversion): `rows` rows of `row_bytes` bytes (a multiple of 16, at most 32 KiB), `src_pitch`
  * bytes apart (a multiple of 16; == row_bytes for a contiguous copy), `col_offset` bytes into each
  * pitch, gathered into a contiguous destination; the source buffer is filled with a seeded pattern.
- * Writes bytes moved (read + written) per second, best of `repeats` launches.  Allocates and frees
- * both buffers.  No counterpart in the reference: the library's own kernels are compared with it. */
+ * `cast` is MXP_CAST_NONE or MXP_CAST_F32_BF16 (the rows are fp32, twice `row_bytes` long in the
+ * source, and are stored as bf16).  Writes bytes moved (read + written) per second, best of
+ * `repeats` launches.  Allocates and frees both buffers.  No counterpart in the reference: the
+ * library's own kernels are compared with it. */
 int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, uint64_t src_pitch, uint32_t col_offset,
-                       int32_t repeats, double* bytes_per_second);
+                       int32_t cast, int32_t repeats, double* bytes_per_second);
 
 /* ---- host-only helpers ---------------------------------------------------- */
 /* blake2b-128 over the scalar list tensor_digest would hash (verify.py:152-155). */

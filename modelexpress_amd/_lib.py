@@ -147,7 +147,7 @@ SIGNATURES = {
     "mxp_execute_after": (C.c_int, [_P, _P, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_execute_resident": (C.c_int, [_P, _P, _PP, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_engine_set_direct_placement": (C.c_int, [_P, C.c_int64]),
-    "mxp_measure_gather": (C.c_int, [_P, C.c_uint64, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int32, C.POINTER(C.c_double)]),
+    "mxp_measure_gather": (C.c_int, [_P, C.c_uint64, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_engine_set_launch_timing": (C.c_int, [_P, C.c_int32]),
     "mxp_engine_launch_times": (C.c_int, [_P, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
     "mxp_plan_checksums": (C.c_int, [_P, _P, _U32P, C.c_int64]),

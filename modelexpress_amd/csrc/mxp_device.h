@@ -159,7 +159,7 @@ hipError_t launch_fill_u32(uint32_t* ptr, uint64_t n, uint32_t value, hipStream_
 hipError_t launch_copy_table(void* dst, const void* src, size_t bytes, hipStream_t stream);
 // Measurement support (mxp_synth.hip): a bare row gather with the placement kernel's workgroup shape.
 hipError_t launch_probe_gather(const void* src, void* dst, uint32_t units_per_row, uint32_t src_pitch, uint32_t rows_per_tile,
-                               uint32_t n_tiles, hipStream_t stream);
+                               uint32_t n_tiles, bool narrow, hipStream_t stream);
 // Device-side fold_fan: out_dev[k] = sum over the copies of element k, k < n; with `clear` the
 // elements read are left at zero.  T is uint32_t or unsigned long long.
 template <typename T>

@@ -2181,15 +2181,19 @@ int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double*
 }
 
 int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, uint64_t src_pitch, uint32_t col_offset,
-                       int32_t repeats, double* bytes_per_second) {
+                       int32_t cast, int32_t repeats, double* bytes_per_second) {
   return guard([&] {
-    if (!engine || !bytes_per_second || rows == 0 || row_bytes == 0 || row_bytes % 16 || row_bytes > 32768 || src_pitch % 16 ||
-        col_offset % 16 || (uint64_t)col_offset + row_bytes > src_pitch || src_pitch >= (1ull << 31))
+    if (cast != MXP_CAST_NONE && cast != MXP_CAST_F32_BF16) throw Error(MXP_ERR_ARG, "mxp_measure_gather: cast must be none or fp32 -> bf16");
+    const bool narrow = cast == MXP_CAST_F32_BF16;
+    const uint64_t src_row = narrow ? 2ull * row_bytes : row_bytes;  // source bytes of a row
+    const uint32_t out_unit = narrow ? 8u : 16u;                     // destination bytes per 16 source bytes
+    if (!engine || !bytes_per_second || rows == 0 || row_bytes == 0 || row_bytes % out_unit || src_row > 32768 || src_pitch % 16 ||
+        col_offset % 16 || (uint64_t)col_offset + src_row > src_pitch || src_pitch >= (1ull << 31))
       throw Error(MXP_ERR_ARG, "mxp_measure_gather: bad argument");
     mxp_engine& e = *engine;
     HIP_OK(hipSetDevice(e.opt.device));
     if (repeats < 1) repeats = 1;
-    const uint32_t upr = row_bytes / 16;
+    const uint32_t upr = (uint32_t)(src_row / 16);
     const uint32_t rpt = (uint32_t)std::min<uint64_t>(rows, (uint64_t)kPlaceThreads * kPlaceBatch / upr);
     const uint64_t n_tiles = rows / rpt;
     if (n_tiles == 0 || n_tiles > 0x7FFFFFFFull) throw Error(MXP_ERR_ARG, "mxp_measure_gather: bad argument");
@@ -2197,11 +2201,12 @@ int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, ui
     DevBuf<uint8_t> src, dst;
     src.reserve(src_bytes);
     dst.reserve(dst_bytes);
+    // bf16 values ~N(0, 0.02): read as fp32, every pair of them is a finite number, so the narrowing probe meets no NaN
     HIP_OK(launch_synth(src.p, src_bytes / 2, MXP_DTYPE_BF16, 0u, 0x6a7468ull, e.streams[0]));
     float best = 1e30f;
     for (int r = 0; r < repeats + 1; ++r) {
       HIP_OK(hipEventRecord(e.ev_a, e.streams[0]));
-      HIP_OK(launch_probe_gather(src.p + col_offset, dst.p, upr, (uint32_t)src_pitch, rpt, (uint32_t)n_tiles, e.streams[0]));
+      HIP_OK(launch_probe_gather(src.p + col_offset, dst.p, upr, (uint32_t)src_pitch, rpt, (uint32_t)n_tiles, narrow, e.streams[0]));
       HIP_OK(hipEventRecord(e.ev_b, e.streams[0]));
       HIP_OK(hipEventSynchronize(e.ev_b));
       float ms = 0;
@@ -2219,6 +2224,7 @@ int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, ui
       g.dst_pitch = row_bytes;
       g.rows = used_rows;
       g.row_bytes = row_bytes;
+      g.op = narrow ? kOpCastF32Bf16 : kOpCopy;
       g.csum_slot = 0;
       uint32_t want = 0, got = 0;
       run_boxes(e, {g}, {src.p}, {again.p}, 1, &want, e.streams[0]);
@@ -2229,7 +2235,7 @@ int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, ui
       run_boxes(e, {c}, {dst.p}, {}, 1, &got, e.streams[0]);
       if (want != got) throw Error(MXP_ERR_STATE, "mxp_measure_gather: the probe kernel and the placement kernel disagree");
     }
-    *bytes_per_second = 2.0 * (double)dst_bytes / ((double)best * 1e-3);
+    *bytes_per_second = ((double)dst_bytes + (double)used_rows * (double)src_row) / ((double)best * 1e-3);
   });
 }
 

@@ -180,12 +180,17 @@ namespace {
 typedef uint32_t probe_u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kProbeThreads = 1024, kProbeBatch = 8;
 
+// NARROW: the rows are fp32 and are stored as bf16 (round to nearest even; the probe's inputs hold no NaN):
+// 16 bytes in and 8 bytes out per unit, the shape of the placement kernel's narrowing path.
+typedef uint32_t probe_u32x2 __attribute__((ext_vector_type(2)));
+template <bool NARROW>
 __global__ __launch_bounds__(kProbeThreads) void probe_gather_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
                                                                      uint32_t units_per_row, uint32_t magic, uint32_t src_pitch,
                                                                      uint32_t rows_per_tile) {
+  constexpr uint32_t kOut = NARROW ? 8u : 16u;  // destination bytes per unit (a unit reads 16 source bytes)
   const uint64_t t = blockIdx.x;
   const uint8_t* s = src + t * rows_per_tile * (uint64_t)src_pitch;
-  uint8_t* d = dst + t * rows_per_tile * (uint64_t)units_per_row * 16u;
+  uint8_t* d = dst + t * rows_per_tile * (uint64_t)units_per_row * kOut;
   const uint32_t n_units = rows_per_tile * units_per_row;
   probe_u32x4 a[kProbeBatch];
   uint32_t so[kProbeBatch], d_o[kProbeBatch];
@@ -198,37 +203,51 @@ __global__ __launch_bounds__(kProbeThreads) void probe_gather_kernel(const uint8
     const uint32_t row = units_per_row == 1u ? v : __umulhi(v, magic);
     const uint32_t col = v - row * units_per_row;
     so[k] = row * src_pitch + col * 16u;
-    d_o[k] = v * 16u;
+    d_o[k] = v * kOut;
   }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int k = 0; k < kProbeBatch; ++k) a[k] = __builtin_nontemporal_load(reinterpret_cast<const probe_u32x4*>(s + so[k]));
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int k = 0; k < kProbeBatch; ++k)
-    if (ok[k]) __builtin_nontemporal_store(a[k], reinterpret_cast<probe_u32x4*>(d + d_o[k]));
+  for (int k = 0; k < kProbeBatch; ++k) {
+    if (!ok[k]) continue;
+    if constexpr (NARROW) {
+      auto rne = [](uint32_t u) { return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16; };
+      probe_u32x2 o;
+      o.x = rne(a[k].x) | (rne(a[k].y) << 16);
+      o.y = rne(a[k].z) | (rne(a[k].w) << 16);
+      __builtin_nontemporal_store(o, reinterpret_cast<probe_u32x2*>(d + d_o[k]));
+    } else {
+      __builtin_nontemporal_store(a[k], reinterpret_cast<probe_u32x4*>(d + d_o[k]));
+    }
+  }
 }
 }  // namespace
 
-// Gathers n_tiles * rows_per_tile rows of units_per_row * 16 bytes, `src_pitch` bytes apart, into a
-// contiguous destination.  rows_per_tile * units_per_row <= 8192; both buffers 16-byte aligned.
+// Gathers n_tiles * rows_per_tile rows of units_per_row * 16 source bytes, `src_pitch` bytes apart, into a
+// contiguous destination (as they are, or narrowed from fp32 to bf16).  rows_per_tile * units_per_row <= 8192;
+// both buffers 16-byte aligned.
 hipError_t launch_probe_gather(const void* src, void* dst, uint32_t units_per_row, uint32_t src_pitch, uint32_t rows_per_tile,
-                               uint32_t n_tiles, hipStream_t stream) {
+                               uint32_t n_tiles, bool narrow, hipStream_t stream) {
   if (n_tiles == 0) return hipSuccess;
   if (units_per_row == 0 || rows_per_tile == 0 || (uint64_t)rows_per_tile * units_per_row > (uint64_t)kProbeThreads * kProbeBatch ||
-      (uint64_t)rows_per_tile * src_pitch >= (1ull << 32) || src_pitch % 16u)
+      (uint64_t)rows_per_tile * src_pitch >= (1ull << 32) || src_pitch % 16u || (uint64_t)units_per_row * 16u > src_pitch)
     return hipErrorInvalidValue;
   constexpr int kOnePerCu = 96 * 1024;  // more than half a compute unit's LDS: one resident workgroup
   static bool configured = false;
   if (!configured) {
-    if (hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(probe_gather_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, kOnePerCu); e != hipSuccess)
-      return e;
+    for (const void* f : {reinterpret_cast<const void*>(probe_gather_kernel<false>), reinterpret_cast<const void*>(probe_gather_kernel<true>)})
+      if (hipError_t e = hipFuncSetAttribute(f, hipFuncAttributeMaxDynamicSharedMemorySize, kOnePerCu); e != hipSuccess) return e;
     configured = true;
   }
   const uint32_t magic = units_per_row > 1 ? (uint32_t)((1ull << 32) / units_per_row) + 1u : 0u;
-  hipLaunchKernelGGL(probe_gather_kernel, dim3(n_tiles), dim3(kProbeThreads), kOnePerCu, stream, static_cast<const uint8_t*>(src),
-                     static_cast<uint8_t*>(dst), units_per_row, magic, src_pitch, rows_per_tile);
+  if (narrow)
+    hipLaunchKernelGGL(probe_gather_kernel<true>, dim3(n_tiles), dim3(kProbeThreads), kOnePerCu, stream, static_cast<const uint8_t*>(src),
+                       static_cast<uint8_t*>(dst), units_per_row, magic, src_pitch, rows_per_tile);
+  else
+    hipLaunchKernelGGL(probe_gather_kernel<false>, dim3(n_tiles), dim3(kProbeThreads), kOnePerCu, stream, static_cast<const uint8_t*>(src),
+                       static_cast<uint8_t*>(dst), units_per_row, magic, src_pitch, rows_per_tile);
   return hipGetLastError();
 }
 

@@ -515,13 +515,16 @@ class PlacementEngine:
                                        out if checksums else None, C.c_void_p(stream)))
         return [format(out[i], "08x") for i in range(n)] if checksums else None
 
-    def measure_gather(self, rows: int, row_bytes: int, src_pitch: int | None = None, col_offset: int = 0, repeats: int = 5) -> float:
+    def measure_gather(self, rows: int, row_bytes: int, src_pitch: int | None = None, col_offset: int = 0, repeats: int = 5,
+                       cast: int = 0) -> float:
         """Bytes per second (read + written) that a bare kernel of the placement kernel's workgroup shape reaches
-        on ``rows`` rows of ``row_bytes`` bytes gathered out of a ``src_pitch`` (default: contiguous): what the
-        memory system of this box gives the shape, for comparison with the library's own kernels."""
+        on ``rows`` rows of ``row_bytes`` destination bytes gathered out of a ``src_pitch`` (default: contiguous):
+        what the memory system of this box gives the shape, for comparison with the library's own kernels.
+        ``cast``: 0, or ``CAST_CODES[("F32", "BF16")]`` for fp32 rows (twice as long in the source) stored as bf16."""
         out = C.c_double()
-        L.check(L.lib().mxp_measure_gather(self._h, rows, row_bytes, row_bytes if src_pitch is None else src_pitch, col_offset,
-                                           repeats, C.byref(out)))
+        src_row = row_bytes * 2 if cast else row_bytes
+        L.check(L.lib().mxp_measure_gather(self._h, rows, row_bytes, src_row if src_pitch is None else src_pitch, col_offset,
+                                           cast, repeats, C.byref(out)))
         return float(out.value)
 
     def measure_h2d(self, nbytes: int = 256 << 20, repeats: int = 5) -> float:

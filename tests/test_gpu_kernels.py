@@ -632,6 +632,10 @@ def test_bare_gather_probe_moves_what_the_placement_kernel_moves(gpu_engine, mxp
     otherwise), so a positive figure here means the probe moved the right bytes."""
     rate = gpu_engine.measure_gather(rows, row_bytes, pitch, col, repeats=2)
     assert rate > 0
+    if row_bytes % 32 == 0 and pitch is not None:  # the same source rows read as fp32 and stored as bf16
+        assert gpu_engine.measure_gather(rows, row_bytes // 2, pitch, col, repeats=2, cast=1) > 0
+    elif pitch is None:
+        assert gpu_engine.measure_gather(rows, row_bytes // 2, None, 0, repeats=2, cast=1) > 0
     with pytest.raises(mxp.MxpError):
         gpu_engine.measure_gather(16, 24, 64)  # rows that are not a multiple of 16 bytes
     with pytest.raises(mxp.MxpError):
