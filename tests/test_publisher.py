@@ -86,10 +86,9 @@ def test_digest_publication_follows_the_environment_live(gpu_engine, monkeypatch
 @pytest.mark.gpu
 def test_colocated_refit_trainer_snapshot_to_engine_parameters(gpu_engine):
     """Both ends on one GPU: the trainer's fp32 state dict is snapshotted into bf16 arenas (one launch), the
-    engine's own loaders are captured once on a meta twin, and each step re-slices the arenas into the live
+    engine's loaders are described once as recorded copies, and each step re-slices the arenas into the live
     parameters (one launch) - the bytes are those of the loaders fed the bf16 tensors on the CPU."""
-    from test_capture import MiniDecoderLayer, _plain_default_loader
-    from modelexpress_amd.capture import capture_geometry
+    from decoder_layer import MiniDecoderLayer
     from modelexpress_amd.reshard import ReslicePlan
 
     tp_size, tp_rank = 2, 1
@@ -98,17 +97,15 @@ def test_colocated_refit_trainer_snapshot_to_engine_parameters(gpu_engine):
               "down": (256, 768), "embed": (1000, 256), "c_fc": (256, 768), "norm": (256,)}
     g = torch.Generator().manual_seed(33)
     trainer = {n: torch.randn(s, generator=g).cuda() for n, s in shapes.items()}
-    with torch.device("meta"):
-        twin = MiniDecoderLayer(tp_size, tp_rank, **kw)
-    capture = capture_geometry(twin, [(n, WIRE_DTYPE, list(s)) for n, s in shapes.items()], default_weight_loader=_plain_default_loader)
     live = MiniDecoderLayer(tp_size, tp_rank, **kw).cuda()
+    copies = live.recorded_copies(premerged=False, dtype=WIRE_DTYPE)
     params = dict(live.named_parameters())
     stager = WireStager(gpu_engine)
     plan = None
     for step in range(3):
         served = stager.stage(trainer)["served"]
         if plan is None:
-            plan = ReslicePlan(capture.copies, served, params)
+            plan = ReslicePlan(copies, served, params)
             plan.run(gpu_engine, served, params)
         else:
             plan.replay()

@@ -394,3 +394,63 @@ def test_view_plan_runs_from_a_hip_graph(gpu_engine):
         torch.cuda.synchronize()
         assert all(torch.equal(d, w) for d, w in zip(dsts, want())), step
     plan.close()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("tp_size,tp_rank,premerged", [(1, 0, False), (2, 1, False), (4, 3, True)])
+def test_decoder_layer_descriptors_replayed_on_the_device(gpu_engine, tp_size, tp_rank, premerged):
+    """fp32 trainer tensors into bf16 engine parameters: the descriptors of a decoder layer's loaders (written by
+    hand, decoder_layer.py), run on the device and replayed after the sources changed, give the bytes the loaders
+    themselves give on the CPU."""
+    from decoder_layer import MiniDecoderLayer
+    from modelexpress_amd.reshard import ReslicePlan
+
+    hidden, heads, kv_heads, head_dim, inter, vocab = 256, 8, 4, 32, 768, 1000
+    shapes = {"q": (heads * head_dim, hidden), "k": (kv_heads * head_dim, hidden), "v": (kv_heads * head_dim, hidden),
+              "o_proj": (hidden, heads * head_dim), "down": (hidden, inter), "embed": (vocab, hidden), "c_fc": (hidden, inter), "norm": (hidden,)}
+    shapes.update({"gate_up_merged": (2 * inter, hidden)} if premerged else {"gate": (inter, hidden), "up": (inter, hidden)})
+    kw = dict(hidden=hidden, heads=heads, kv_heads=kv_heads, head_dim=head_dim, inter=inter, vocab=vocab)
+    g = torch.Generator().manual_seed(70 + tp_rank)
+    live = MiniDecoderLayer(tp_size, tp_rank, **kw).cuda()
+    copies = live.recorded_copies(premerged)
+    assert len(copies) == len(shapes) + (1 if premerged else 0)  # the pre-merged source yields two copies
+    assert {c.src_name for c in copies} == set(shapes)
+    params = dict(live.named_parameters())
+    plan = dev = None
+    for step in range(2):
+        srcs = {n: torch.randn(s, generator=g) * 2 for n, s in shapes.items()}
+        truth = MiniDecoderLayer(tp_size, tp_rank, **kw)
+        truth.load_weights(list(srcs.items()))
+        if step == 0:
+            dev = {n: t.cuda() for n, t in srcs.items()}
+            plan = ReslicePlan(copies, dev, params)
+            plan.run(gpu_engine, dev, params)
+        else:
+            for n, t in srcs.items():
+                dev[n].copy_(t)   # new values at the same addresses
+            plan.replay()
+        for name, p in truth.named_parameters():
+            assert torch.equal(params[name].cpu().view(torch.int16), p.view(torch.int16)), (step, name)
+    plan.close()
+
+
+def test_decoder_layer_descriptors_equal_the_loaders_on_the_cpu():
+    """The hand-written descriptors are themselves checked against the loaders, on the CPU, with torch's own
+    ``as_strided().copy_()`` (the operation the reference performs per recorded copy)."""
+    from decoder_layer import MiniDecoderLayer
+
+    for tp_size, tp_rank, premerged in [(1, 0, False), (2, 1, True), (4, 3, False), (4, 0, True)]:
+        kw = dict(hidden=64, heads=8, kv_heads=4, head_dim=8, inter=96, vocab=101)
+        shapes = {"q": (64, 64), "k": (32, 64), "v": (32, 64), "o_proj": (64, 64), "down": (64, 96), "embed": (101, 64),
+                  "c_fc": (64, 96), "norm": (64,)}
+        shapes.update({"gate_up_merged": (192, 64)} if premerged else {"gate": (96, 64), "up": (96, 64)})
+        g = torch.Generator().manual_seed(5 + tp_rank)
+        srcs = {n: torch.randn(s, generator=g).to(torch.bfloat16) for n, s in shapes.items()}
+        truth = MiniDecoderLayer(tp_size, tp_rank, **kw)
+        truth.load_weights(list(srcs.items()))
+        recon = MiniDecoderLayer(tp_size, tp_rank, **kw)
+        params = dict(recon.named_parameters())
+        for c in recon.recorded_copies(premerged):
+            params[c.param_name].data.as_strided(c.dest_shape, c.dest_stride, c.dest_offset).copy_(_apply(c.op_chain, srcs[c.src_name]))
+        for name, p in truth.named_parameters():
+            assert torch.equal(params[name].view(torch.int16), p.view(torch.int16)), (tp_size, tp_rank, name)
