@@ -209,7 +209,7 @@ def _scenarios(ref, workdir: str, scenario: str) -> dict:
     rv = layout.rank_view(tp_size=tp, tp_rank=rank)
     device = "cuda" if torch.cuda.is_available() else "cpu"
 
-    class ToyModel(torch.nn.Module):
+    class RankModule(torch.nn.Module):
         stacked_params_mapping = [("qkv_proj", "q_proj"), ("qkv_proj", "k_proj"), ("qkv_proj", "v_proj"),
                                   ("gate_up_proj", "gate_proj"), ("gate_up_proj", "up_proj")]
 
@@ -238,7 +238,7 @@ def _scenarios(ref, workdir: str, scenario: str) -> dict:
 
         def reinit_for_retry(self, result):
             self.reinit_calls += 1
-            fresh = ToyModel()
+            fresh = RankModule()
             return ref.LoadResult(value=fresh, model=fresh)
 
         def load_via_native(self, result):
@@ -280,7 +280,7 @@ def _scenarios(ref, workdir: str, scenario: str) -> dict:
         out["placing_overrides"] = type(PlacingAdapter()).placement_layout is not ref.EngineAdapter.placement_layout
         log: list = []
         ad = BareAdapter()
-        model = ToyModel()
+        model = RankModule()
         got = run_chain(ref, model, ctx_for(ad, workdir), strategies(), log)
         out["chain_log"], out["native_calls"], out["same_model"] = log, ad.native_calls, got is model
         return out
@@ -295,7 +295,7 @@ def _scenarios(ref, workdir: str, scenario: str) -> dict:
         # eligibility needs a device; the failure semantics do not
         chain = [s for s in strategies()]
         chain[0].is_available = lambda _ctx: True
-        model = ToyModel()
+        model = RankModule()
         got = run_chain(ref, model, ctx, chain, log)
         out["chain_log"], out["reinit_calls"], out["native_calls"] = log, ad.reinit_calls, ad.native_calls
         out["same_model"] = got is model
@@ -311,7 +311,7 @@ def _scenarios(ref, workdir: str, scenario: str) -> dict:
     if scenario == "success":
         ad = PlacingAdapter()
         log = []
-        model = ToyModel()
+        model = RankModule()
         ctx = ctx_for(ad, workdir)
         out["eligible_with_plain_backend"] = LS.HipPlacementStrategy().is_available(ctx)
         got = run_chain(ref, model, ctx, strategies(), log)
@@ -337,7 +337,7 @@ def _scenarios(ref, workdir: str, scenario: str) -> dict:
         E.PlacementEngine.execute = execute_after_truncation
         ad = PlacingAdapter()
         log = []
-        model = ToyModel()
+        model = RankModule()
         got = run_chain(ref, model, ctx_for(ad, workdir), strategies(), log)
         out["chain_log"], out["reinit_calls"], out["native_calls"] = log, ad.reinit_calls, ad.native_calls
         out["fresh_model_returned"] = got is not model

@@ -21,7 +21,7 @@ LAYOUT = models.Llama(layers=2, hidden=64, ffn=96, q_heads=8, kv_heads=4, head_d
 TP, RANK = 4, 1
 
 
-class ToyModel(nn.Module):
+class RankModule(nn.Module):
     """A module whose parameters are exactly one rank's table (what an engine allocates)."""
 
     stacked_params_mapping = [("qkv_proj", "q_proj"), ("qkv_proj", "k_proj"), ("qkv_proj", "v_proj"),
@@ -41,7 +41,7 @@ class ToyModel(nn.Module):
             yield name, getattr(self, key)
 
 
-class ToyAdapter(EngineAdapter):
+class RankAdapter(EngineAdapter):
     def __init__(self, rv):
         self.rv = rv
         self.reinit_calls = 0
@@ -55,7 +55,7 @@ class ToyAdapter(EngineAdapter):
 
     def reinit_for_retry(self, result):
         self.reinit_calls += 1
-        fresh = ToyModel(self.rv)
+        fresh = RankModule(self.rv)
         return LoadResult(value=fresh, model=fresh)
 
     def load_via_native(self, result):
@@ -72,9 +72,9 @@ def test_chain_places_into_param_data(oracle, tmp_path, monkeypatch, mxp):
     rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
     want = oracle_place(oracle, str(tmp_path), rv, tp_size=TP, tp_rank=RANK)
     monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
-    model = ToyModel(rv)
+    model = RankModule(rv)
     ptrs = {n: p.data_ptr() for n, p in model.named_parameters()}
-    ad = ToyAdapter(rv)
+    ad = RankAdapter(rv)
     ctx = _ctx(ad, str(tmp_path))
     out = LoadStrategyChain.run(model, ctx)
     assert out is model and ad.reinit_calls == 0 and ad.native_calls == 0
@@ -97,8 +97,8 @@ def test_manifest_of_a_placed_rank_matches_a_source_manifest(oracle, tmp_path, m
     source = [TensorRecord(p.name, p.nbytes, p.dtype, oracle.safe_checksum(want[p.name]), oracle.tensor_digest(want[p.name]))
               for p in rv.params]
     monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
-    model = ToyModel(rv)
-    ad = ToyAdapter(rv)
+    model = RankModule(rv)
+    ad = RankAdapter(rv)
     result = HipPlacementStrategy().load(LoadResult(value=model, model=model), _ctx(ad, str(tmp_path)))
     assert compare_manifests(source, result.metadata["manifest"], require_exact_match=True) == len(rv.params)
     eng = PlacementEngine(0)
@@ -131,14 +131,14 @@ def test_truncated_shard_fails_the_strategy_and_the_chain_recovers(tmp_path, mon
         return real_execute(eng, plan, dst, **kw)
 
     monkeypatch.setattr(E.PlacementEngine, "execute", execute_after_truncation)
-    model = ToyModel(rv)
-    ad = ToyAdapter(rv)
+    model = RankModule(rv)
+    ad = RankAdapter(rv)
     with pytest.raises(StrategyFailed) as e:
         HipPlacementStrategy().load(LoadResult(value=model, model=model), _ctx(ad, str(tmp_path)))
     assert "MXP_ERR_IO" in str(e.value)
 
     synth.write_checkpoint(LAYOUT.checkpoint(), str(tmp_path), n_shards=2, seed=22)
-    model2 = ToyModel(rv)
+    model2 = RankModule(rv)
     out = LoadStrategyChain.run(model2, _ctx(ad, str(tmp_path)))
     assert ad.native_calls == 1  # hip_placement failed, model_streamer is not offered by this adapter
     assert (out is not model2) == (ad.reinit_calls == 1)
@@ -148,9 +148,9 @@ def test_bad_checkpoint_is_a_clean_miss(tmp_path, monkeypatch, mxp):
     (tmp_path / "model.safetensors").write_bytes(b"\x05\x00\x00\x00\x00\x00\x00\x00{nope")
     rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
     monkeypatch.setenv("MX_MODEL_URI", str(tmp_path))
-    model = ToyModel(rv)
+    model = RankModule(rv)
     with pytest.raises(StrategyFailed) as e:
-        HipPlacementStrategy().load(LoadResult(value=model, model=model), _ctx(ToyAdapter(rv), str(tmp_path)))
+        HipPlacementStrategy().load(LoadResult(value=model, model=model), _ctx(RankAdapter(rv), str(tmp_path)))
     assert e.value.mutated is False
     assert all(int(p.data.view(torch.uint8).sum()) == 0 for _n, p in model.named_parameters())
 
@@ -186,11 +186,11 @@ def test_refit_stage_verify_apply(oracle, tmp_path, mxp):
     synth.write_checkpoint(LAYOUT.checkpoint(), str(base), n_shards=2, seed=24)
     synth.write_checkpoint(LAYOUT.checkpoint(dtype="F32", edge_cases=models.NORMAL_EDGE_DENSE), str(new), n_shards=3, seed=25)
     rv = LAYOUT.rank_view(tp_size=TP, tp_rank=RANK)
-    model = ToyModel(rv)
+    model = RankModule(rv)
     layout = layout_from_module(model, tp_size=TP, tp_rank=RANK)
     os.environ["MX_MODEL_URI"] = str(base)
     try:
-        LoadStrategyChain.run(model, _ctx(ToyAdapter(rv), str(base)))
+        LoadStrategyChain.run(model, _ctx(RankAdapter(rv), str(base)))
     finally:
         del os.environ["MX_MODEL_URI"]
     v0 = {n: p.data.view(torch.uint8).cpu().numpy().tobytes() for n, p in model.named_parameters()}
