@@ -14,6 +14,10 @@
  * calling thread is available from mxp_last_error().  Handles are not re-entrant: use
  * one plan / engine from one thread at a time.
  *
+ * The library is built for one part: MI355X (gfx950), 256 compute units in 8 XCDs; launch
+ * shapes and the sizes of accumulator tables assume that count.  Entry points that exist
+ * only for measurements and test inputs are declared in mxp_bench.h, not here.
+ *
  * Each entry point names the piece of the reference (ai-dynamo/modelexpress,
  * modelexpress_client/python/modelexpress/...) whose behaviour it replaces.
  */
@@ -297,7 +301,9 @@ int mxp_execute_after(mxp_engine* engine, mxp_plan* plan, void* const* dst_ptrs,
  * for the whole plan; asynchronous unless `stats` is non-NULL (then it synchronises and
  * reports the HIP-event time of the launch in stats->kernel_ms).  A plan's pointer tables and
  * accumulators are its own: launches of one plan are serialised (a call on another stream than
- * the previous one waits for that launch), and changed `dst_ptrs` / `file_dev_ptrs` reach the
+ * the previous one waits for that launch, through an event it records on the previous stream:
+ * a stream a plan was launched on must stay alive until the plan's next launch or the plan's
+ * destruction), and changed `dst_ptrs` / `file_dev_ptrs` reach the
  * device by copies ordered on `stream`, never under a launch that still runs. */
 int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* file_dev_ptrs,
                          void* const* dst_ptrs, void* stream, mxp_exec_stats* stats);
@@ -310,18 +316,6 @@ int mxp_execute_resident(mxp_engine* engine, mxp_plan* plan, const void* const* 
  * bounce slot and the placement kernel.  min_bytes: 0 = the default (64 KiB), a negative value =
  * off (every byte takes the bounce slot).  Results are identical either way. */
 int mxp_engine_set_direct_placement(mxp_engine* engine, int64_t min_bytes);
-
-/* Launch timing for measurements.  Switched on, every asynchronous mxp_execute_resident (stats ==
- * NULL) records a HIP-event pair around its placement kernel on the launch stream and does NOT
- * synchronise, so a timed loop of K launches yields both its wall time and the K kernel
- * durations.  The stand-alone operators that launch through descriptor tables built per call
- * (mxp_cast, mxp_copy_view(s), mxp_permute_copy, mxp_place_boxes, mxp_copy_batch, mxp_checksum32) and the runs of a
- * verify plan (mxp_verify_plan_checksums / _digests)
- * record a pair around each of their placement / transpose launches in the same way.  mxp_engine_launch_times waits for the launches and writes the durations (ms) of the
- * most recent min(capacity, recorded, 256) of them, oldest first.  Switching on or off restarts
- * the count.  No counterpart in the reference. */
-int mxp_engine_set_launch_timing(mxp_engine* engine, int32_t on);
-int mxp_engine_launch_times(mxp_engine* engine, float* out_ms, int32_t capacity, int32_t* n_out);
 
 /* Checksums accumulated by the last execute, one per parameter (tensor_utils.py:27-44
  * over the parameter's row-major bytes).  Synchronises the engine first. */
@@ -344,8 +338,8 @@ int mxp_plan_digests(mxp_engine* engine, mxp_plan* plan, uint8_t* out16, int64_t
  *   out[k] = sum_i byte_i * ((i * 2654435761 + 1) mod 2^32) mod 2^32. */
 int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
                    uint32_t* out, void* stream);
-/* mxp_checksum32 for callers that cannot allocate (code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments and
+/* mxp_checksum32 for callers that cannot allocate (tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same arguments and
  * results as mxp_checksum32; the descriptor tables and accumulators its kernel reads live in a
  * 1 MiB device array that is part of the library image (one copy per GPU, held until the process
  * ends) and in a pinned mirror allocated by mxp_engine_create, so the call itself allocates and
@@ -353,7 +347,9 @@ int mxp_checksum32(mxp_engine* engine, const void* const* ptrs, const uint64_t* 
  * workgroups of 128 KiB in all (about 12 GiB); beyond them the call fails with MXP_ERR_ARG and
  * launches nothing.  Every call on a GPU - from any engine - uses that GPU's one array: calls
  * that overlap in time on one GPU race and must be serialised by the caller.  Blocks until
- * `stream` is idle, like mxp_checksum32. */
+ * `stream` is idle, like mxp_checksum32, and returns its results on the host: it cannot be
+ * recorded into a HIP graph, and a `stream` that is being captured is refused with MXP_ERR_STATE
+ * before anything is queued (the capture stays valid). */
 int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uint64_t* nbytes, int64_t n,
                           uint32_t* out, void* stream);
 /* mxp_checksum32 / mxp_digest over a FIXED set of device buffers, lowered once: a refit loop
@@ -477,21 +473,6 @@ void mxp_view_plan_destroy(mxp_view_plan* plan);
  * be 16-byte aligned and must not overlap each other. */
 int mxp_copy_batch(mxp_engine* engine, const void* const* srcs, void* const* dsts, const uint64_t* nbytes,
                    int64_t n, uint32_t* out_checksums, void* stream);
-/* Measured pinned host -> device bandwidth of this box in bytes per second
- * (hipMemcpyAsync of `bytes` from a pinned buffer, best of `repeats`). */
-int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double* bytes_per_second);
-/* What this box's memory system gives an access shape, measured with a bare kernel that has the
- * placement kernel's workgroup shape and nothing else (no descriptor tables, no checksum, no
- * conversion): `rows` rows of `row_bytes` bytes (a multiple of 16, at most 32 KiB), `src_pitch`
- * bytes apart (a multiple of 16; == row_bytes for a contiguous copy), `col_offset` bytes into each
- * pitch, gathered into a contiguous destination; the source buffer is filled with a seeded pattern.
- * `cast` is MXP_CAST_NONE or MXP_CAST_F32_BF16 (the rows are fp32, twice `row_bytes` long in the
- * source, and are stored as bf16).  Writes bytes moved (read + written) per second, best of
- * `repeats` launches.  Allocates and frees both buffers.  No counterpart in the reference: the
- * library's own kernels are compared with it. */
-int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, uint64_t src_pitch, uint32_t col_offset,
-                       int32_t cast, int32_t repeats, double* bytes_per_second);
-
 /* ---- host-only helpers ---------------------------------------------------- */
 /* blake2b-128 over the scalar list tensor_digest would hash (verify.py:152-155). */
 int mxp_digest_from_scalars(const uint64_t scalars[7], uint8_t out16[16]);
@@ -504,15 +485,6 @@ int mxp_digest_from_scalars(const uint64_t scalars[7], uint8_t out16[16]);
 uint32_t mxp_crc32c(uint32_t seed, const void* data, uint64_t nbytes);
 int mxp_file_crc32c(const char* path, uint64_t chunk_size, uint32_t* file_crc, uint32_t* chunk_crcs,
                     uint64_t max_chunks, uint64_t* n_chunks);
-
-/* Seeded synthetic contents (test and benchmark inputs; same bytes on host and device).
- * kind: 0 ~N(0,0.02), 1 ones, 2 zeros, 3 normal with denormal/inf/NaN/tie edge cases at
- * 1e-6 density, 4 fp8 bytes over the finite e4m3 codes, 5 fp32 scales in [1e-4,1e-2],
- * 6 as 3 at 1/64 density. */
-int mxp_synth_host(void* dst, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed,
-                   int32_t threads);
-int mxp_synth_device(void* dst_dev, uint64_t n_elems, int32_t dtype, uint32_t kind, uint64_t seed,
-                     void* stream);
 
 #ifdef __cplusplus
 }

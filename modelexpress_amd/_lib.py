@@ -1,4 +1,5 @@
-"""ctypes binding of libmxplace.so (the C ABI declared in include/mxp.h).
+"""ctypes binding of libmxplace.so (the C ABI declared in include/mxp.h, plus the measurement entry points of
+include/mxp_bench.h).
 
 The library is the product: there is no Python or CPU fallback for anything it does.
 If it is missing, or was built without a symbol the header declares, importing this
@@ -109,7 +110,7 @@ _PP = C.POINTER(C.c_void_p)
 _U64P = C.POINTER(C.c_uint64)
 _U32P = C.POINTER(C.c_uint32)
 
-# name -> (restype, argtypes); every symbol include/mxp.h declares.
+# name -> (restype, argtypes); every symbol include/mxp.h declares (the product ABI).
 SIGNATURES = {
     "mxp_last_error": (C.c_char_p, []),
     "mxp_abi_version": (C.c_int, []),
@@ -147,9 +148,6 @@ SIGNATURES = {
     "mxp_execute_after": (C.c_int, [_P, _P, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_execute_resident": (C.c_int, [_P, _P, _PP, _PP, _P, C.POINTER(ExecStats)]),
     "mxp_engine_set_direct_placement": (C.c_int, [_P, C.c_int64]),
-    "mxp_measure_gather": (C.c_int, [_P, C.c_uint64, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
-    "mxp_engine_set_launch_timing": (C.c_int, [_P, C.c_int32]),
-    "mxp_engine_launch_times": (C.c_int, [_P, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
     "mxp_plan_checksums": (C.c_int, [_P, _P, _U32P, C.c_int64]),
     "mxp_checksum32": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
     "mxp_checksum32_static": (C.c_int, [_P, _PP, _U64P, C.c_int64, _U32P, _P]),
@@ -172,10 +170,17 @@ SIGNATURES = {
     "mxp_view_plan_bytes": (C.c_int, [_P, _U64P]),
     "mxp_view_plan_destroy": (None, [_P]),
     "mxp_copy_batch": (C.c_int, [_P, _PP, _PP, _U64P, C.c_int64, _U32P, _P]),
-    "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_digest_from_scalars": (C.c_int, [_U64P, C.POINTER(C.c_uint8)]),
     "mxp_crc32c": (C.c_uint32, [C.c_uint32, _P, C.c_uint64]),
     "mxp_file_crc32c": (C.c_int, [C.c_char_p, C.c_uint64, _U32P, _U32P, C.c_uint64, _U64P]),
+}
+
+# The measurement and test-input entry points of include/mxp_bench.h (same library, no part of the drop-in boundary).
+BENCH_SIGNATURES = {
+    "mxp_measure_gather": (C.c_int, [_P, C.c_uint64, C.c_uint32, C.c_uint64, C.c_uint32, C.c_int32, C.c_int32, C.POINTER(C.c_double)]),
+    "mxp_engine_set_launch_timing": (C.c_int, [_P, C.c_int32]),
+    "mxp_engine_launch_times": (C.c_int, [_P, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
+    "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
     "mxp_synth_host": (C.c_int, [_P, C.c_uint64, C.c_int32, C.c_uint32, C.c_uint64, C.c_int32]),
     "mxp_synth_device": (C.c_int, [_P, C.c_uint64, C.c_int32, C.c_uint32, C.c_uint64, _P]),
 }
@@ -194,7 +199,7 @@ def lib() -> C.CDLL:
             "Run `python -m modelexpress_amd.build`; there is no fallback path."
         )
     handle = C.CDLL(str(LIB_PATH))
-    for name, (restype, argtypes) in SIGNATURES.items():
+    for name, (restype, argtypes) in {**SIGNATURES, **BENCH_SIGNATURES}.items():
         try:
             fn = getattr(handle, name)
         except AttributeError as exc:

@@ -64,7 +64,7 @@ def build_library(force: bool = True, jobs: int = 4) -> Path:
     hipcc = _hipcc()
     obj_dir = PKG_DIR / "build"
     obj_dir.mkdir(exist_ok=True)
-    headers = list(CSRC.glob("*.h")) + list(CSRC.glob("*.hpp")) + [INCLUDE / "mxp.h"]
+    headers = list(CSRC.glob("*.h")) + list(CSRC.glob("*.hpp")) + [INCLUDE / "mxp.h", INCLUDE / "mxp_bench.h"]
     newest_header = max(h.stat().st_mtime for h in headers)
     todo = []
     objs = []

@@ -107,15 +107,22 @@ struct Fan {
   uint32_t lanes() const { return mask + 1; }
 };
 // Fan for `n_slots` accumulators: copies a multiple of 256 bytes apart, so that the copies of one
-// accumulator fall into different cache lines; tables too large to be worth copying stay plain.
+// accumulator fall into different cache lines.  The fanned table is bounded by size, not by slot
+// count: copies x pitch stays at or below 65,536 elements (64 copies up to 1,024 slots, halved
+// for every doubling after that, one copy - the plain layout - above 16,384), so a plan's two sets
+// of checksum and digest accumulators (44 bytes per slot and copy) never take more than 5.5 MiB
+// and clearing one set is at most 2.75 MiB of stores.  The more slots a launch feeds, the fewer
+// workgroups meet in any one of them, so the narrower fan loses nothing.
 inline Fan make_fan(uint64_t n_slots) {
   Fan f;
   if (n_slots > 16384) {
     f.pitch = (uint32_t)n_slots;
     return f;
   }
-  f.mask = kFanLanes - 1;
   f.pitch = (uint32_t)((n_slots ? n_slots : 1) + 63) / 64 * 64;
+  uint32_t lanes = kFanLanes;
+  while (lanes > 1 && (uint64_t)lanes * f.pitch > 65536) lanes >>= 1;
+  f.mask = lanes - 1;
   return f;
 }
 // Elements (of either kind) the fanned array of `per_slot`-element accumulators holds.

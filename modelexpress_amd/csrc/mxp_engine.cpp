@@ -1243,6 +1243,11 @@ int mxp_checksum32_static(mxp_engine* engine, const void* const* ptrs, const uin
     mxp_engine& e = *engine;
     hipStream_t stream = static_cast<hipStream_t>(stream_v);
     HIP_OK(hipSetDevice(e.opt.device));
+    // The call ends with a wait for `stream` and hands its results back on the host: neither can be
+    // recorded.  Refused before anything is queued, so the caller's capture stays valid.
+    if (is_capturing(stream))
+      throw Error(MXP_ERR_STATE, "mxp_checksum32_static: the stream is being captured; the call waits for the stream and "
+                                 "returns host results, so it cannot be recorded into a graph");
     // Tables are lowered straight into the pinned mirror; the previous call synchronised
     // `stream` before it returned, so nothing still reads it.
     unsigned char* h = e.static_host;

@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "mxp.h"
+#include "mxp_bench.h"
 #include "mxp_device.h"
 
 namespace mxp {

@@ -396,10 +396,12 @@ bool with_instance(int elem_size, uint32_t op, F&& f) {
 
 // A workgroup's LDS is sized by the wavefronts it is launched with (a 2-wavefront workgroup that
 // reserved room for 8 left a compute unit with four resident wavefronts).  Above 64 KiB the
-// kernel instance needs the attribute once per device.
-template <typename K>
-hipError_t allow_lds(K kernel, uint32_t bytes) {
-  static std::atomic<uint64_t> allowed{0};  // per kernel instance: bit per device
+// kernel needs the attribute once per device.  The flag is kept per kernel: `Kernel` is the
+// function itself, so every instantiation of the transpose kernels has its own bit mask.
+template <auto Kernel>
+hipError_t allow_lds(uint32_t bytes) {
+  static std::atomic<uint64_t> allowed{0};  // bit per device
+  constexpr auto kernel = Kernel;
   if (bytes <= 64u * 1024u) return hipSuccess;
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return e;
@@ -424,7 +426,7 @@ struct LaunchOne {
   template <int ES, int OP>
   void operator()() const {
     const uint32_t lds = (block.x / 64u) * Sub<ES, OP>::kLdsBytes;
-    err = allow_lds(transpose_kernel<ES, OP>, lds);
+    err = allow_lds<transpose_kernel<ES, OP>>(lds);
     if (err != hipSuccess) return;
     hipLaunchKernelGGL((transpose_kernel<ES, OP>), grid, block, lds, stream, s, t, d, nan_bits, sum_out, fan);
   }
@@ -439,7 +441,7 @@ struct LaunchBatch {
   template <int ES, int OP>
   void operator()() const {
     const uint32_t lds = (block.x / 64u) * Sub<ES, OP>::kLdsBytes;
-    err = allow_lds(transpose_batch_kernel<ES, OP>, lds);
+    err = allow_lds<transpose_batch_kernel<ES, OP>>(lds);
     if (err != hipSuccess) return;
     hipLaunchKernelGGL((transpose_batch_kernel<ES, OP>), grid, block, lds, stream, items, n_items, nan_bits);
   }

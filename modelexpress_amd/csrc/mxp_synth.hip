@@ -12,6 +12,7 @@
 
 #include "mxp_device.h"
 #include "mxp.h"
+#include "mxp_bench.h"
 
 namespace mxp {
 

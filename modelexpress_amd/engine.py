@@ -615,8 +615,10 @@ def digest_from_scalars(scalars: Sequence[int]) -> str:
 
 def _current_stream(device: int) -> int:
     """The raw handle of the calling thread's current torch stream on ``device`` (0 = the default stream)."""
-    import torch
-
+    try:
+        import torch
+    except ImportError:  # a caller that hands over raw device addresses needs no torch: the default stream
+        return 0
     if not torch.cuda.is_available():
         return 0
     return int(torch.cuda.current_stream(device).cuda_stream)

@@ -13,22 +13,28 @@ import pytest
 ROOT = Path(__file__).resolve().parent.parent
 
 
-def _declared():
-    text = (ROOT / "include" / "mxp.h").read_text()
+def _declared(header="mxp.h"):
+    text = (ROOT / "include" / header).read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(mxp_[a-z0-9_]+)\s*\(", text)))
 
 
+BENCH_ONLY = ["mxp_engine_launch_times", "mxp_engine_set_launch_timing", "mxp_measure_gather", "mxp_measure_h2d",
+              "mxp_synth_device", "mxp_synth_host"]
+
+
 def test_library_exports_every_declared_symbol(mxp):
-    declared = _declared()
+    declared, bench = _declared(), _declared("mxp_bench.h")
     assert len(declared) >= 35
+    # measurement and test-input entry points stay out of the drop-in header
+    assert bench == BENCH_ONLY and not set(bench) & set(declared)
     out = subprocess.run(["nm", "-D", "--defined-only", str(mxp.LIB_PATH)], capture_output=True, text=True, check=True)
     exported = {line.split()[-1] for line in out.stdout.splitlines() if " T " in line}
-    assert [s for s in declared if s not in exported] == []
+    assert [s for s in declared + bench if s not in exported] == []
     # and nothing undeclared leaks out under the mxp_ prefix
-    assert sorted(s for s in exported if s.startswith("mxp_")) == declared
-    # the ctypes binding covers the same set
-    assert sorted(mxp.SIGNATURES) == declared
+    assert sorted(s for s in exported if s.startswith("mxp_")) == sorted(declared + bench)
+    # the ctypes binding covers the same sets
+    assert sorted(mxp.SIGNATURES) == declared and sorted(mxp.BENCH_SIGNATURES) == bench
     assert mxp.lib().mxp_abi_version() == 1
 
 
@@ -64,7 +70,7 @@ def test_rust_sys_generator_covers_the_header():
 
 def test_header_is_plain_c(tmp_path):
     src = tmp_path / "t.c"
-    src.write_text('#include "mxp.h"\nint main(void){ mxp_engine_options o; (void)o; return MXP_OK; }\n')
+    src.write_text('#include "mxp.h"\n#include "mxp_bench.h"\nint main(void){ mxp_engine_options o; (void)o; return MXP_OK; }\n')
     subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", f"-I{ROOT / 'include'}", "-c", str(src), "-o",
                     str(tmp_path / "t.o")], check=True)
 

@@ -62,3 +62,26 @@ def test_static_checksum_second_engine_shares_the_scratch(gpu_engine, oracle_c):
         assert gpu_engine.checksum32_static([_dev(b), _dev(a)]) == [oracle_c.checksum32(b), oracle_c.checksum32(a)]
     finally:
         other.close()
+
+
+def test_static_checksum_refuses_a_capturing_stream_and_leaves_the_capture_valid(gpu_engine, mxp):
+    """The call waits for its stream and returns host results, so it cannot be recorded: a stream under capture is
+    refused before anything is queued, and the caller's graph still captures and replays."""
+    x = torch.zeros(1024, dtype=torch.int32, device="cuda")
+    d = torch.arange(4096, dtype=torch.int32, device="cuda").view(torch.uint8)
+    want = gpu_engine.checksum32([d])
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            x.add_(1)
+            with pytest.raises(mxp.MxpError) as refused:
+                gpu_engine.checksum32_static([d], stream=torch.cuda.current_stream().cuda_stream)
+            x.add_(2)
+    assert refused.value.code == mxp.ERR_STATE and "captured" in refused.value.message
+    torch.cuda.synchronize()
+    for replay in range(2):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert int(x[0]) == 3 * (replay + 1)
+    assert gpu_engine.checksum32_static([d]) == want  # and the entry point works as before outside a capture
