@@ -1,4 +1,5 @@
 import ctypes
+import os
 import subprocess
 import sys
 from pathlib import Path
@@ -12,6 +13,11 @@ if str(ROOT) not in sys.path:
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+    trace = os.environ.get("MXP_ABI_TRACE")
+    if trace:  # test_host_sanitizers.py runs a session of its own with this set: record the host-side ABI calls
+        import abi_trace
+
+        abi_trace.install(trace)
 
 
 @pytest.fixture(scope="session")
