@@ -250,12 +250,14 @@ def _fs_type(path: str) -> str:
     return kind
 
 
-def _memory_system_limits(eng, plan, placed: int) -> dict:
-    """What the memory system of this box gives the access shapes of a workload to a bare kernel (no descriptor
-    tables, no checksum): the ceiling the placement kernel is held against, measured in the same run.  One probe
-    per shape of write (contiguous; each distinct strided row length / pitch / column offset; as they are or
-    narrowed from fp32 to bf16), 1 GiB written each, and their composite: the rate at which the bare kernel would
-    move this workload's bytes."""
+def _bare_kernel_same_shape(eng, plan, placed: int) -> dict:
+    """The workload's access shapes through a bare kernel that has the placement kernel's own workgroup shape and
+    addressing but no descriptor tables and no checksum, measured in the same run.  It is a comparison, not a
+    ceiling: a kernel of another shape may do better or worse on the same accesses, and the library's launch can
+    exceed the composite.  What "library = bare" shows is that descriptors and checksums cost nothing.  One probe per
+    shape of write (contiguous; each distinct strided row length / pitch / column offset; as they are or narrowed
+    from fp32 to bf16), 1 GiB written each, and their composite: the rate at which the bare kernel would move this
+    workload's bytes."""
     from modelexpress_amd.engine import CAST_CODES
 
     GiB = 1 << 30
@@ -294,16 +296,78 @@ def _memory_system_limits(eng, plan, placed: int) -> dict:
             moved_total += moved
         return {"what": "fraction of HBM peak that a bare kernel with the placement kernel's workgroup shape (no descriptor "
                         "tables, no checksum) reaches on each shape of write of this workload, 1 GiB written per probe, "
-                        "and the composite of those rates weighted by the bytes each shape moves",
+                        "and the composite of those rates weighted by the bytes each shape moves; a comparison at equal "
+                        "shape (what descriptors and checksums cost), not an upper bound",
                 "shapes": limits, "composite_frac_of_hbm_peak": round(moved_total / t_total / 1e9 / HBM_PEAK_GBPS, 4)}
     except Exception as exc:  # noqa: BLE001 - a probe must not lose the line it belongs to
         return {"skipped": f"{type(exc).__name__}: {exc}"}
 
 
-def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int = 2) -> dict:
-    """One of the other benchmark configurations at full size, HBM-resident: headers on disk only, the
-    checkpoint bytes generated on the device, a few timed launches, and the fused checksums compared with
-    a stand-alone checksum pass over every finished buffer."""
+def _ingest_leg(plan, dst, resident_sums, h2d_peak: float, source: str, *, pack: bool = True, runs: int = 4, ring_slots: int = 32,
+                slot_mib: int = 16, readers: int = 16, tile_bytes: int = 0, direct_min: int = 0) -> dict:
+    """End-to-end ingest of ``plan`` from its files through the pinned ring (first run warms up, best of the others)."""
+    from modelexpress_amd.engine import PlacementEngine
+
+    e2 = PlacementEngine(0, ring_slots=ring_slots, slot_bytes=slot_mib << 20, reader_threads=readers, streams=4,
+                         tile_bytes=tile_bytes, pack_strided_on_host=pack)
+    if direct_min:
+        e2.set_direct_placement(direct_min)
+    best = None
+    for i in range(runs):
+        st = e2.execute(plan, dst)
+        if i and (best is None or st["wall_seconds"] < best["wall_seconds"]):
+            best = st
+    sums = e2.checksums(plan)
+    e2.close()
+    w = best["wall_seconds"]
+    return {"placed_gbps": round(best["placed_bytes"] / w / 1e9, 2), "h2d_gbps": round(best["h2d_bytes"] / w / 1e9, 2),
+            "h2d_peak_gbps": round(h2d_peak, 2), "frac_of_h2d_peak": round(best["h2d_bytes"] / w / 1e9 / h2d_peak, 4),
+            "wall_s": round(w, 4), "file_bytes": best["file_bytes"], "h2d_bytes": best["h2d_bytes"],
+            "strided_slices": "rows packed into the pinned slot by the readers" if pack else
+                              "whole row bands staged, gathered on the device",
+            "reader_threads": readers, "ring": f"{ring_slots} x {slot_mib} MiB pinned", "source": source,
+            "checksums_match_resident": sums == resident_sums}
+
+
+def _refit_cycle(rv, dst, tp: int, rank: int, workdir: str, placed: int, resident_sums, *, ring_slots: int = 32, slot_mib: int = 16,
+                 readers: int = 16) -> dict:
+    """One RL refit cycle through the adapter interface (modelexpress_rl/inference/adapter.py:59-93): plan, ingest
+    with the fp32 -> bf16 cast into staging (checksums and digest sums fused), verify, one batched install into
+    the live buffers.  Best of three."""
+    from modelexpress_amd.adapter import PlacementLayout
+    from modelexpress_amd.engine import PlacementEngine
+    from modelexpress_amd.refit import HipRefitAdapter, RefitInputs
+
+    lay = PlacementLayout(params=rv.params, destinations=dst, tp_size=tp, tp_rank=rank,
+                          stacked_params_mapping=rv.stacked_params_mapping)
+    e3 = PlacementEngine(0, ring_slots=ring_slots, slot_bytes=slot_mib << 20, reader_threads=readers, streams=4)
+    ad = HipRefitAdapter(lay, engine=e3)
+    cycles, applied = [], None
+    for i in range(3):
+        t0 = time.perf_counter()
+        rplan = ad.create_transfer_plan(RefitInputs(f"v{i}", workdir, "bench", {}, require_digests=False))
+        staged = ad.stage_weight(rplan)
+        applied = ad.apply_weight(staged)
+        ad.release_staged_weight(staged)
+        rec = ad.timing.as_dict()
+        rec["wall_s"] = round(time.perf_counter() - t0, 4)
+        cycles.append(rec)
+    best = min(cycles, key=lambda r: r["wall_s"])
+    e3.close()
+    return {"wall_s": best["wall_s"], "placed_gbps": round(placed / best["wall_s"] / 1e9, 2),
+            "stages_s": {k: v["duration_s"] for k, v in best["stages"].items()},
+            "note": "plan + ingest with fp32->bf16 cast into staging (checksums and digest sums fused) + verify + one batched install "
+                    "into the live buffers, through HipRefitAdapter (best of 3)",
+            "checksums_match_resident": [applied[p.name] for p in rv.params] == resident_sums}
+
+
+def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int = 2, *, e2e: bool = False, h2d_peak: float = 0.0,
+                  host_threads: int = 16) -> dict:
+    """One of the other benchmark configurations at full size, HBM-resident: the checkpoint bytes generated on
+    the device, a few timed launches, and the fused checksums compared with a stand-alone checksum pass over
+    every finished buffer.  With ``e2e`` (configurations 1 and 3, when the page-cache file system has room) the
+    checkpoint files are written as well and ingested end to end through the pinned ring, and configuration 3
+    runs its refit cycle through the adapter; otherwise only headers go to disk."""
     import torch
 
     from modelexpress_amd import synth
@@ -317,9 +381,21 @@ def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int
     base = {"workload": WORKLOADS[config], "checkpoint_bytes": w["total_bytes"], "rank_local_checkpoint": w["rank_local"]}
     if need > free:
         return {**base, "skipped": f"needs {need / 1e9:.1f} GB of HBM (staged checkpoint + destinations), {free / 1e9:.1f} GB free"}
-    hdr = tempfile.mkdtemp(prefix=f"mxp_bench_cfg{config}_")
+    hdr, e2e_skip = None, None
+    if e2e:
+        hdr = _pick_workdir(w["total_bytes"])
+        if hdr is None:
+            e2e_skip = f"no file system with {w['total_bytes'] * 1.15 / 1e9:.1f} GB free for the checkpoint files"
+    files_real = hdr is not None
+    if hdr is None:
+        hdr = tempfile.mkdtemp(prefix=f"mxp_bench_cfg{config}_")
     try:
-        synth.write_headers_only(w["tensors"], hdr, n_shards=w["n_shards"])
+        if files_real:
+            t0 = time.perf_counter()
+            synth.write_checkpoint(w["tensors"], hdr, n_shards=w["n_shards"], seed=seed, threads=host_threads)
+            _log(f"config {config}: wrote {w['total_bytes'] / 1e9:.2f} GB checkpoint to {hdr} in {time.perf_counter() - t0:.1f}s")
+        else:
+            synth.write_headers_only(w["tensors"], hdr, n_shards=w["n_shards"])
         ck = Checkpoint(hdr)
         plan = PlacementPlan(ck, rv.params, tp_size=tp, tp_rank=w["rank"], stacked_params_mapping=rv.stacked_params_mapping,
                              expert_mapping=rv.expert_mapping, allow_cast=cast)
@@ -345,7 +421,17 @@ def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int
                             "unit": "GB/s", "frac": round(algo / (k_avg * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
                             "algorithmic_bytes": algo, "kernel": "place_kernel"},
                "checksums_agree": fused == alone}
-        out["roofline"]["memory_system_limits"] = _memory_system_limits(eng, plan, placed)
+        if files_real:
+            # the metric's end-to-end half for this configuration: files (page cache) -> pinned ring -> HBM
+            out["e2e"] = _ingest_leg(plan, dst, fused, h2d_peak or eng.measure_h2d(256 << 20, 5) / 1e9, f"page cache ({hdr})",
+                                     runs=6 if placed < 1e9 else 4, readers=host_threads)
+            out["checksums_agree"] = out["checksums_agree"] and out["e2e"]["checksums_match_resident"]
+            if cast:
+                out["refit_cycle"] = _refit_cycle(rv, dst, tp, w["rank"], hdr, placed, fused, readers=host_threads)
+                out["checksums_agree"] = out["checksums_agree"] and out["refit_cycle"]["checksums_match_resident"]
+        elif e2e:
+            out["e2e"] = {"skipped": e2e_skip}
+        out["roofline"]["bare_kernel_same_shape"] = _bare_kernel_same_shape(eng, plan, placed)
         eng.close()
         plan.close()
         ck.close()
@@ -414,6 +500,8 @@ def main() -> int:
     ap.add_argument("--slot-mib", type=int, default=16, help="pinned ring slot size for the ingest leg")
     ap.add_argument("--ring-slots", type=int, default=32)
     ap.add_argument("--readers", type=int, default=0, help="reader threads for the ingest leg (0 = host cores, at most 16)")
+    ap.add_argument("--cold-readers", type=int, default=0,
+                    help="reader threads of the O_DIRECT leg and of its storage-rate probe (0 = twice the host cores used)")
     ap.add_argument("--cold", action="store_true",
                     help="also run the ingest leg with O_DIRECT from a file system that supports it (MXP_BENCH_DIR), "
                          "bypassing the page cache")
@@ -702,32 +790,14 @@ def main() -> int:
 
         # ---- end-to-end ingest from files through the pinned ring ----
         agree = True
+        h2d_peak_run = 0.0
         if files_real and not args.no_e2e:
-            h2d_peak = eng.measure_h2d(256 << 20, 5) / 1e9
+            h2d_peak = h2d_peak_run = eng.measure_h2d(256 << 20, 5) / 1e9
             for key, pack in (("e2e_ingest", True), ("e2e_ingest_band", False)):
-                e2 = PlacementEngine(0, ring_slots=args.ring_slots, slot_bytes=args.slot_mib << 20,
-                                     reader_threads=args.readers or host_threads, streams=4,
-                                     tile_bytes=args.tile_kib * 1024, pack_strided_on_host=pack)
-                if args.direct_min:
-                    e2.set_direct_placement(args.direct_min)
-                best = None
-                for i in range(4 if placed > 8e9 else 7):  # the first run warms up; the best of the others is reported
-                    st = e2.execute(plan, dst)
-                    if i and (best is None or st["wall_seconds"] < best["wall_seconds"]):
-                        best = st
-                ingest_sums = e2.checksums(plan)
-                e2.close()
-                agree = agree and ingest_sums == resident_sums
-                w = best["wall_seconds"]
-                out[key] = {
-                    "placed_gbps": round(best["placed_bytes"] / w / 1e9, 2), "h2d_gbps": round(best["h2d_bytes"] / w / 1e9, 2),
-                    "h2d_peak_gbps": round(h2d_peak, 2), "frac_of_h2d_peak": round(best["h2d_bytes"] / w / 1e9 / h2d_peak, 4),
-                    "wall_s": round(w, 4), "file_bytes": best["file_bytes"], "h2d_bytes": best["h2d_bytes"],
-                    "strided_slices": "rows packed into the pinned slot by the readers" if pack else
-                                      "whole row bands staged, gathered on the device",
-                    "reader_threads": args.readers or host_threads,
-                    "ring": f"{args.ring_slots} x {args.slot_mib} MiB pinned", "source": f"page cache ({workdir})",
-                    "checksums_match_resident": ingest_sums == resident_sums}
+                out[key] = _ingest_leg(plan, dst, resident_sums, h2d_peak, f"page cache ({workdir})", pack=pack,
+                                       runs=4 if placed > 8e9 else 7, ring_slots=args.ring_slots, slot_mib=args.slot_mib,
+                                       readers=args.readers or host_threads, tile_bytes=args.tile_kib * 1024, direct_min=args.direct_min)
+                agree = agree and out[key]["checksums_match_resident"]
                 _log(f"{key}: {out[key]}")
             # the metric's first half, next to the kernel's roofline: PCIe is what bounds it
             e = out["e2e_ingest"]
@@ -764,23 +834,46 @@ def main() -> int:
                     ck_c = Checkpoint(cold_dir)
                     plan_c = PlacementPlan(ck_c, rv.params, tp_size=tp, tp_rank=rank, stacked_params_mapping=rv.stacked_params_mapping,
                                            expert_mapping=rv.expert_mapping, allow_cast=cast)
+                    from modelexpress_amd.engine import measure_read
+
+                    # direct reads block in the kernel, not on a core: twice as many readers as cores keeps the disk's queue full
+                    # while some readers copy a finished chunk into the ring; the probe uses the same count
+                    readers = args.cold_readers or 2 * host_threads
+                    paths = [f["path"] for f in ck_c.files()]
+                    # the denominator: the same files read whole by the same number of threads with the same request
+                    # size and O_DIRECT, no GPU work - before and after the ingest legs (a shared virtual disk drifts)
+                    peak0 = measure_read(paths, threads=readers, request_bytes=args.slot_mib << 20, direct=True)
                     legs = {}
                     for label, pack in (("packed_rows", True), ("row_bands", False)):
                         e2 = PlacementEngine(0, ring_slots=args.ring_slots, slot_bytes=args.slot_mib << 20,
-                                             reader_threads=args.readers or host_threads, streams=4, use_o_direct=True,
+                                             reader_threads=readers, streams=4, use_o_direct=True,
                                              pack_strided_on_host=pack)
+                        e2.prepare(plan_c)  # lowering and the pinned ring, as a loader does at start-up: the one pass is the reads
                         st = e2.execute(plan_c, dst)
                         cold_sums = e2.checksums(plan_c)
                         e2.close()
                         agree = agree and cold_sums == resident_sums
                         legs[label] = {"placed_gbps": round(st["placed_bytes"] / st["wall_seconds"] / 1e9, 3),
                                        "file_gbps": round(st["file_bytes"] / st["wall_seconds"] / 1e9, 3),
+                                       "h2d_gbps": round(st["h2d_bytes"] / st["wall_seconds"] / 1e9, 3),
                                        "wall_s": round(st["wall_seconds"], 3), "file_bytes": st["file_bytes"],
                                        "checksums_match_resident": cold_sums == resident_sums}
+                    peak1 = measure_read(paths, threads=readers, request_bytes=args.slot_mib << 20, direct=True)
+                    storage_peak = max(peak0["bytes_per_second"], peak1["bytes_per_second"]) / 1e9
+                    for leg in legs.values():
+                        leg["frac_of_storage_peak"] = round(leg["file_gbps"] / storage_peak, 4)
                     plan_c.close()
                     ck_c.close()
                     out["e2e_ingest_direct_io"] = {
                         "source": f"O_DIRECT reads from {cold_dir} ({_fs_type(cold_dir)}), one pass each, no page cache: storage-bound",
+                        "bound": "storage", "storage_peak_gbps": round(storage_peak, 3),
+                        "storage_peak_is": f"plain O_DIRECT read of the same {len(paths)} shard files ({peak0['bytes'] / 1e9:.2f} GB), {readers} threads, "
+                                           f"{args.slot_mib} MiB requests, no GPU work; the better of a pass before and a pass after the ingest legs "
+                                           f"({peak0['bytes_per_second'] / 1e9:.2f} / {peak1['bytes_per_second'] / 1e9:.2f} GB/s)",
+                        "strided_slices_under_direct_io": "packed_rows is the default: the readers fetch a band's rows with large requests into "
+                                                          "their own buffers and copy only the rows into the ring (a third of the bytes cross "
+                                                          "PCIe); row_bands stages whole bands and gathers on the device - each reader then "
+                                                          "copies a whole 16 MiB chunk into the ring between two requests, which is what it loses",
                         "checkpoint_write_s": round(write_s, 1), **legs}
                     _log(f"e2e_ingest_direct_io: {out['e2e_ingest_direct_io']}")
                 finally:
@@ -788,33 +881,10 @@ def main() -> int:
 
         # ---- one RL refit cycle through the adapter interface (configuration 3 only) ----
         if files_real and cast and not args.no_e2e:
-            from modelexpress_amd.adapter import PlacementLayout
-            from modelexpress_amd.refit import HipRefitAdapter, RefitInputs
-
-            lay = PlacementLayout(params=rv.params, destinations=dst, tp_size=tp, tp_rank=rank,
-                                  stacked_params_mapping=rv.stacked_params_mapping)
-            e3 = PlacementEngine(0, ring_slots=args.ring_slots, slot_bytes=args.slot_mib << 20,
-                                 reader_threads=args.readers or host_threads, streams=4)
-            ad = HipRefitAdapter(lay, engine=e3)
-            cycles = []
-            for i in range(3):
-                t0 = time.perf_counter()
-                rplan = ad.create_transfer_plan(RefitInputs(f"v{i}", workdir, "bench", {}, require_digests=False))
-                staged = ad.stage_weight(rplan)
-                applied = ad.apply_weight(staged)
-                ad.release_staged_weight(staged)
-                rec = ad.timing.as_dict()
-                rec["wall_s"] = round(time.perf_counter() - t0, 4)
-                cycles.append(rec)
-            best = min(cycles, key=lambda r: r["wall_s"])
-            agree = agree and [applied[p.name] for p in rv.params] == resident_sums
-            out["refit_cycle"] = {"wall_s": best["wall_s"], "placed_gbps": round(placed / best["wall_s"] / 1e9, 2),
-                                  "stages_s": {k: v["duration_s"] for k, v in best["stages"].items()},
-                                  "note": "plan + ingest with fp32->bf16 cast into staging (checksums and digest sums fused) + verify + one batched install "
-                                          "into the live buffers, through HipRefitAdapter (best of 3)",
-                                  "checksums_match_resident": [applied[p.name] for p in rv.params] == resident_sums}
+            out["refit_cycle"] = _refit_cycle(rv, dst, tp, rank, workdir, placed, resident_sums, ring_slots=args.ring_slots,
+                                              slot_mib=args.slot_mib, readers=args.readers or host_threads)
+            agree = agree and out["refit_cycle"]["checksums_match_resident"]
             _log(f"refit_cycle: {out['refit_cycle']}")
-            e3.close()
 
         # ---- CPU baseline: the oracle placing the same rank from the same files ----
         if files_real and not args.no_cpu:
@@ -866,7 +936,7 @@ def main() -> int:
         # milliseconds after a free of that size the platform does work of its own on the copy engines, and an ingest
         # measured then ran at 50 GB/s instead of 56.)
         if not args.no_ops:
-            roofline["memory_system_limits"] = _memory_system_limits(eng, plan, placed)
+            roofline["bare_kernel_same_shape"] = _bare_kernel_same_shape(eng, plan, placed)
 
         # ---- the same step for the first and the last rank of the group (default run only): every rank's share has
         # the same size, its column slices start elsewhere in each row ----
@@ -897,11 +967,15 @@ def main() -> int:
         if args.config == 2 and not args.layers and not args.no_configs:
             del staged, dst
             torch.cuda.empty_cache()
+            plan.close()
+            ck.close()
+            shutil.rmtree(workdir, ignore_errors=True)  # the page-cache file system is needed again below
             out["configs"] = {}
             for cfg in (1, 3, 4, 5):
                 t0 = time.perf_counter()
                 try:
-                    out["configs"][f"config{cfg}"] = _other_config(cfg, args.rank, args.seed)
+                    out["configs"][f"config{cfg}"] = _other_config(cfg, args.rank, args.seed, e2e=cfg in (1, 3) and not args.no_e2e,
+                                                                    h2d_peak=h2d_peak_run, host_threads=host_threads)
                 except Exception as exc:  # noqa: BLE001 - one leg must not lose the headline line
                     out["configs"][f"config{cfg}"] = {"workload": WORKLOADS[cfg], "error": f"{type(exc).__name__}: {exc}"}
                 _log(f"config {cfg}: {out['configs'][f'config{cfg}']} ({time.perf_counter() - t0:.1f}s)")

@@ -245,9 +245,10 @@ typedef struct mxp_engine_options {
   uint32_t tile_bytes;     /* source bytes per workgroup, 1 KiB .. 128 KiB; 0 = 128 KiB */
   uint16_t nan_bits;       /* bf16 image of every NaN in the cast; 0 = default 0x7FC0 */
   uint16_t pack_strided_on_host; /* strided slices: 1 = readers pack the needed rows into the
-                                    slot (only placed bytes cross PCIe), 2 = stage whole row
-                                    bands and gather on the device, 0 = default (1, or 2
-                                    with use_o_direct) */
+                                    slot (only placed bytes cross PCIe; with use_o_direct they
+                                    read the rows of a band with large requests into their
+                                    own buffers first), 2 = stage whole row bands and gather
+                                    on the device, 0 = default (1) */
   int32_t use_o_direct;    /* 1 = open files with O_DIRECT (falls back if unsupported) */
 } mxp_engine_options;
 
@@ -269,8 +270,9 @@ typedef struct mxp_exec_stats {
 int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out);
 void mxp_engine_destroy(mxp_engine* engine);
 
-/* Lowers `plan` to the engine's descriptor tables and chunk list without running it
- * (mxp_execute does this on first use); afterwards mxp_plan_totals is complete. */
+/* Lowers `plan` to the engine's descriptor tables and chunk list and allocates the engine's pinned
+ * ring without running anything (mxp_execute does both on first use); afterwards mxp_plan_totals
+ * is complete and the first mxp_execute starts reading at once. */
 int mxp_prepare(mxp_engine* engine, mxp_plan* plan);
 
 /* Ingest from storage: reader threads pread each planned byte range into a pinned

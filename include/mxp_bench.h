@@ -32,6 +32,12 @@ int mxp_engine_launch_times(mxp_engine* engine, float* out_ms, int32_t capacity,
 /* Measured pinned host -> device bandwidth of this box in bytes per second
  * (hipMemcpyAsync of `bytes` from a pinned buffer, best of `repeats`). */
 int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double* bytes_per_second);
+/* Plain read rate of a set of files, no GPU work: `threads` threads claim requests of `request_bytes`
+ * (a multiple of 4096) in file order and read them into private block-aligned buffers, with O_DIRECT
+ * when `direct` is non-zero (no page cache) - the way the ingest's readers read whole row bands.
+ * What a cold ingest from the same files is compared with. */
+int mxp_measure_read(const char* const* paths, int64_t n_paths, int32_t threads, uint64_t request_bytes, int32_t direct,
+                     uint64_t* total_bytes, double* bytes_per_second);
 /* What this box's memory system gives an access shape, measured with a bare kernel that has the
  * placement kernel's workgroup shape and nothing else (no descriptor tables, no checksum, no
  * conversion): `rows` rows of `row_bytes` bytes (a multiple of 16, at most 32 KiB), `src_pitch`

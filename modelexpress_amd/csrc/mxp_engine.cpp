@@ -7,6 +7,7 @@
 // the device bounce slots, streams, events and descriptor tables.  All HIP work issued
 // by a call has completed when the call returns, unless documented otherwise.
 #include <fcntl.h>
+#include <sys/stat.h>
 #include <hip/hip_runtime.h>
 #include <unistd.h>
 
@@ -266,6 +267,28 @@ namespace {
 
 void free_lowered(mxp_plan::Lowered* l) { delete l; }
 
+// Direct I/O, rows packed by the readers: how many consecutive rows (`pitch` bytes apart, `row_bytes`
+// long) one read request covers.  A request per row is a 4-8 KiB random read, and the device's request
+// rate then bounds the ingest (262,144 of them for a Llama-3-8B rank's column slices: 1.3 GB/s on a disk
+// that gives 5 GB/s to large requests).  Where the rows lie close enough that reading what is between
+// them costs less than that - at most eight times the blocks the rows themselves touch - a request
+// covers as many rows as the reader's block-aligned buffer holds, and the rows are copied out of it.
+inline uint64_t direct_rows_per_read(uint64_t buf_bytes, uint64_t pitch, uint64_t row_bytes) {
+  const uint64_t window = align_up(row_bytes + 4095, 4096);  // blocks one unaligned row can touch
+  if (pitch > 8 * window || buf_bytes < 2 * 4096 + row_bytes) return 1;
+  return std::max<uint64_t>(1, (buf_bytes - 2 * 4096 - row_bytes) / pitch + 1);
+}
+// Bytes the requests for `rows` such rows starting at file offset `off` read in all.
+inline uint64_t direct_rows_file_bytes(uint64_t buf_bytes, uint64_t off, uint64_t rows, uint64_t pitch, uint64_t row_bytes) {
+  const uint64_t per = direct_rows_per_read(buf_bytes, pitch, row_bytes);
+  uint64_t total = 0;
+  for (uint64_t r = 0; r < rows; r += per) {
+    const uint64_t nr = std::min(per, rows - r), o0 = off + r * pitch;
+    total += align_up(o0 + (nr - 1) * pitch + row_bytes, 4096) - o0 / 4096 * 4096;
+  }
+  return total;
+}
+
 // Splits every write into slot-sized pieces, packs their byte ranges into chunks in
 // (file, offset) order, and lowers both the ingest and the resident descriptor tables.
 void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
@@ -453,12 +476,10 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
         }
         uint64_t lead = 0, need = 0;
         if (L->direct_io && p.rows > 1) {
-          // packed rows: each row is read as whole blocks into the reader's own buffer and only
-          // its bytes are copied into the slot, so the slot layout is that of buffered packing
-          for (uint64_t r = 0; r < p.rows; ++r) {
-            const uint64_t o0 = p.file_off + r * p.file_pitch;
-            L->file_bytes += align_up(o0 + p.nbytes, blk) - o0 / blk * blk;
-          }
+          // packed rows: whole blocks are read into the reader's own buffer (several rows per request
+          // where they lie close together) and only the rows' bytes are copied into the slot, so the
+          // slot layout is that of buffered packing
+          L->file_bytes += direct_rows_file_bytes(eng.opt.slot_bytes, p.file_off, p.rows, p.file_pitch, p.nbytes);
           L->file_bytes -= p.nbytes * p.rows;  // added back below with the slot bytes
         } else if (L->direct_io) {
           const uint64_t a0 = p.file_off / blk * blk, a1 = align_up(p.file_off + p.nbytes, blk);
@@ -777,11 +798,13 @@ int mxp_engine_create(const mxp_engine_options* opts, mxp_engine** out) {
     if (o.streams <= 0) o.streams = 4;
     if (o.tile_bytes == 0) o.tile_bytes = kPlaceThreads * kPlaceBatch * 16;
     if (o.nan_bits == 0) o.nan_bits = 0x7FC0;
-    // Packing strided rows on the host issues one read per row: right for the page cache.  Under
-    // direct I/O every row read is widened to whole 4 KiB blocks, so whole row bands staged and
-    // gathered on the device are the default there; packing stays available (it reads less when
-    // rows are far apart: 4 KiB per 1 KiB row of an 8 KiB pitch instead of 8 KiB).
-    if (o.pack_strided_on_host == 0) o.pack_strided_on_host = o.use_o_direct ? 2 : 1;
+    // Packing strided rows on the host is the default in both modes.  From the page cache it is one read
+    // call per row; under direct I/O the readers fetch the rows of a band with large requests into their
+    // own buffers (direct_rows_per_read) and copy only the rows into the slot - the same bytes leave
+    // storage as when whole bands are staged, a third of them cross PCIe (Llama-3-8B rank share) and
+    // the reader spends less time copying between two requests (measured 6.1-6.6 against 5.6-6.3 GB/s
+    // from a disk that gave a plain read 6.6-7.1 GB/s).
+    if (o.pack_strided_on_host == 0) o.pack_strided_on_host = 1;
     if (o.pack_strided_on_host > 2) throw Error(MXP_ERR_ARG, "pack_strided_on_host must be 0, 1 or 2");
     if (o.slot_bytes < (1u << 16) || o.slot_bytes % 4096) throw Error(MXP_ERR_ARG, "slot_bytes must be a multiple of 4096, at least 64 KiB");
     if (o.tile_bytes < 1024 || o.tile_bytes > (uint32_t)(kPlaceThreads * kPlaceBatch * 16))
@@ -895,45 +918,66 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
   auto worker = [&](int tid) {
     // The kernel refuses direct I/O into HIP pinned memory (EFAULT: the mapping cannot be
     // pinned again by the block layer), so direct reads land in an ordinary block-aligned
-    // buffer and are copied into the slot.
+    // buffer and are copied into the slot.  `stage_buf` is that buffer: the chunk as the slot will
+    // hold it; `direct_buf` is where several packed rows are read at once before they are gathered.
     void* direct_buf = nullptr;
-    struct Free { void*& p; ~Free() { std::free(p); } } free_direct{direct_buf};
+    void* stage_buf = nullptr;
+    struct Free { void*& p; ~Free() { std::free(p); } } free_direct{direct_buf}, free_stage{stage_buf};
     try {
       HIP_OK(hipSetDevice(e.opt.device));
-      if (L.direct_io && ::posix_memalign(&direct_buf, 4096, e.opt.slot_bytes) != 0)
-        throw Error(MXP_ERR_STATE, "out of host memory for the direct I/O buffer");
+      if (L.direct_io && (::posix_memalign(&direct_buf, 4096, e.opt.slot_bytes) != 0 ||
+                          ::posix_memalign(&stage_buf, 4096, e.opt.slot_bytes) != 0))
+        throw Error(MXP_ERR_STATE, "out of host memory for the direct I/O buffers");
       for (;;) {
         const size_t c = next.fetch_add(1);
         if (c >= n_chunks || abort.load()) break;
         const Chunk& ch = L.chunks[c];
         Slot& sl = *e.slots[c % n_slots];
         const uint64_t turn = c / n_slots;
-        {
-          // Wait until the previous chunk carried by this slot has been submitted, then
-          // until the GPU has finished with it.
-          std::unique_lock<std::mutex> lk(sl.mu);
-          sl.cv.wait(lk, [&] { return sl.submitted == turn || abort.load(); });
-        }
-        if (abort.load()) break;
-        if (turn > 0) HIP_OK(hipEventSynchronize(sl.done));
+        auto wait_for_slot = [&]() -> bool {
+          {
+            // Wait until the previous chunk carried by this slot has been submitted, then
+            // until the GPU has finished with it.
+            std::unique_lock<std::mutex> lk(sl.mu);
+            sl.cv.wait(lk, [&] { return sl.submitted == turn || abort.load(); });
+          }
+          if (abort.load()) return false;
+          if (turn > 0) HIP_OK(hipEventSynchronize(sl.done));
+          return true;
+        };
         const double t0 = now_s();
-        for (const auto& r : ch.ranges)
-          for (uint64_t row = 0; row < r.rows; ++row) {
-            uint8_t* into = sl.host + r.slot_off + row * r.nbytes;
-            if (direct_buf && r.rows > 1) {
+        if (direct_buf) {
+          // Direct I/O: the whole chunk is read into the reader's own block-aligned copy of the slot BEFORE
+          // the slot is waited for, so the number of storage requests in flight is the number of readers,
+          // whatever the ring holds; a slot is then only needed for one copy out of that buffer.
+          uint8_t* const stage = static_cast<uint8_t*>(stage_buf);
+          for (const auto& r : ch.ranges) {
+            if (r.rows == 1) {  // slot offsets are block aligned in this mode: read in place
+              pread_full(fds[r.file], stage + r.slot_off, r.nbytes, r.file_off, ck.files[r.file].path, r.need);
+              continue;
+            }
+            // packed rows: several rows per request (direct_rows_per_read), gathered out of the request's buffer
+            const uint64_t per = direct_rows_per_read(e.opt.slot_bytes, r.file_pitch, r.nbytes);
+            for (uint64_t row = 0; row < r.rows; row += per) {
+              const uint64_t nr = std::min(per, r.rows - row);
               const uint64_t o0 = r.file_off + row * r.file_pitch, a0 = o0 / 4096 * 4096;
-              const uint64_t a1 = align_up(o0 + r.nbytes, 4096);
-              pread_full(fds[r.file], static_cast<uint8_t*>(direct_buf), a1 - a0, a0, ck.files[r.file].path,
-                         o0 - a0 + r.nbytes);
-              std::memcpy(into, static_cast<uint8_t*>(direct_buf) + (o0 - a0), r.nbytes);
-            } else if (direct_buf) {
-              pread_full(fds[r.file], static_cast<uint8_t*>(direct_buf), r.nbytes, r.file_off + row * r.file_pitch,
-                         ck.files[r.file].path, r.need);
-              std::memcpy(into, direct_buf, r.need ? r.need : r.nbytes);
-            } else {
-              pread_full(fds[r.file], into, r.nbytes, r.file_off + row * r.file_pitch, ck.files[r.file].path, r.need);
+              const uint64_t last = o0 + (nr - 1) * r.file_pitch + r.nbytes;
+              pread_full(fds[r.file], static_cast<uint8_t*>(direct_buf), align_up(last, 4096) - a0, a0, ck.files[r.file].path,
+                         last - a0);
+              for (uint64_t k = 0; k < nr; ++k)
+                std::memcpy(stage + r.slot_off + (row + k) * r.nbytes,
+                            static_cast<uint8_t*>(direct_buf) + (o0 - a0) + k * r.file_pitch, r.nbytes);
             }
           }
+          if (!wait_for_slot()) break;
+          std::memcpy(sl.host, stage, ch.used_bytes);
+        } else {
+          if (!wait_for_slot()) break;
+          for (const auto& r : ch.ranges)
+            for (uint64_t row = 0; row < r.rows; ++row)
+              pread_full(fds[r.file], sl.host + r.slot_off + row * r.nbytes, r.nbytes, r.file_off + row * r.file_pitch,
+                         ck.files[r.file].path, r.need);
+        }
         read_s[tid] += now_s() - t0;
         hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
         mutated.store(1);
@@ -1097,6 +1141,7 @@ int mxp_prepare(mxp_engine* engine, mxp_plan* plan) {
     if (!engine || !plan) throw Error(MXP_ERR_ARG, "mxp_prepare: null handle");
     HIP_OK(hipSetDevice(engine->opt.device));
     lower_plan(*plan, *engine);
+    ensure_ring(*engine);  // the pinned ring too: allocating it takes longer than ingesting a small checkpoint
   });
 }
 
@@ -2182,6 +2227,67 @@ int mxp_measure_h2d(mxp_engine* engine, uint64_t bytes, int32_t repeats, double*
     (void)hipHostFree(h);
     if (err != hipSuccess) throw Error(MXP_ERR_DEVICE, std::string("mxp_measure_h2d: ") + hipGetErrorString(err));
     *bytes_per_second = (double)bytes / ((double)best * 1e-3);
+  });
+}
+
+int mxp_measure_read(const char* const* paths, int64_t n_paths, int32_t threads, uint64_t request_bytes, int32_t direct,
+                     uint64_t* total_bytes, double* bytes_per_second) {
+  return guard([&] {
+    if (!paths || n_paths <= 0 || !bytes_per_second || threads < 1 || request_bytes == 0 || request_bytes % 4096)
+      throw Error(MXP_ERR_ARG, "mxp_measure_read: bad argument");
+    struct Req { int file; uint64_t off, n; };
+    std::vector<int> fds((size_t)n_paths, -1);
+    struct FdCloser {
+      std::vector<int>& f;
+      ~FdCloser() { for (int fd : f) if (fd >= 0) ::close(fd); }
+    } closer{fds};
+    std::vector<Req> reqs;
+    uint64_t total = 0;
+    for (int64_t f = 0; f < n_paths; ++f) {
+      int flags = O_RDONLY;
+#ifdef O_DIRECT
+      if (direct) flags |= O_DIRECT;
+#endif
+      fds[(size_t)f] = ::open(paths[f], flags);
+      if (fds[(size_t)f] < 0) throw Error(MXP_ERR_IO, std::string("cannot open ") + paths[f] + ": " + std::strerror(errno));
+      struct stat st;
+      if (::fstat(fds[(size_t)f], &st) != 0) throw Error(MXP_ERR_IO, std::string("cannot stat ") + paths[f]);
+      for (uint64_t off = 0; off < (uint64_t)st.st_size; off += request_bytes)
+        reqs.push_back(Req{(int)f, off, std::min<uint64_t>(request_bytes, (uint64_t)st.st_size - off)});
+      total += (uint64_t)st.st_size;
+    }
+    std::atomic<size_t> next{0};
+    std::atomic<bool> failed{false};
+    std::mutex err_mu;
+    std::string err;
+    const double t0 = now_s();
+    auto worker = [&] {
+      void* buf = nullptr;
+      if (::posix_memalign(&buf, 4096, request_bytes) != 0) { failed.store(true); return; }
+      try {
+        for (;;) {
+          const size_t i = next.fetch_add(1);
+          if (i >= reqs.size() || failed.load()) break;
+          const Req& r = reqs[i];
+          // whole blocks, as direct I/O wants them; the last request of a file may end short
+          pread_full(fds[(size_t)r.file], static_cast<uint8_t*>(buf), align_up(r.n, 4096), r.off, paths[r.file], r.n);
+        }
+      } catch (const std::exception& ex) {
+        std::lock_guard<std::mutex> lk(err_mu);
+        if (err.empty()) err = ex.what();
+        failed.store(true);
+      }
+      std::free(buf);
+    };
+    {
+      std::vector<std::thread> pool;
+      for (int t = 0; t < threads; ++t) pool.emplace_back(worker);
+      for (auto& t : pool) t.join();
+    }
+    const double dt = now_s() - t0;
+    if (failed.load()) throw Error(MXP_ERR_IO, "mxp_measure_read: " + (err.empty() ? std::string("out of host memory") : err));
+    if (total_bytes) *total_bytes = total;
+    *bytes_per_second = dt > 0 ? (double)total / dt : 0.0;
   });
 }
 

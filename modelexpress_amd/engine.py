@@ -533,6 +533,14 @@ class PlacementEngine:
         return float(out.value)
 
 
+def measure_read(paths: Sequence[str], *, threads: int = 16, request_bytes: int = 16 << 20, direct: bool = True) -> dict:
+    """Plain read rate of ``paths`` (no GPU work): what a cold ingest of the same files is compared with."""
+    arr = (C.c_char_p * len(paths))(*[str(p).encode() for p in paths])
+    total, rate = C.c_uint64(), C.c_double()
+    L.check(L.lib().mxp_measure_read(arr, len(paths), threads, request_bytes, 1 if direct else 0, C.byref(total), C.byref(rate)))
+    return {"bytes": int(total.value), "bytes_per_second": float(rate.value)}
+
+
 class VerifyPlan:
     """Handle of ``mxp_verify_plan``: a fixed set of device buffers lowered once for repeated ``checksum32`` /
     ``tensor_digest`` passes; a run is one launch, a small reduction into pinned memory and an event wait."""

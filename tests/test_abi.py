@@ -20,7 +20,7 @@ def _declared(header="mxp.h"):
 
 
 BENCH_ONLY = ["mxp_engine_launch_times", "mxp_engine_set_launch_timing", "mxp_measure_gather", "mxp_measure_h2d",
-              "mxp_synth_device", "mxp_synth_host"]
+              "mxp_measure_read", "mxp_synth_device", "mxp_synth_host"]
 
 
 def test_library_exports_every_declared_symbol(mxp):

@@ -217,6 +217,91 @@ def test_deepseek_v3_layers_real_shapes(oracle, oracle_c, tmp_path, mxp):
     eng.close()
 
 
+def _room_for(n_bytes: int):
+    """A directory on a file system with room for ``n_bytes`` of checkpoint files, page cache first; None if none."""
+    import os
+    import shutil
+    import tempfile
+
+    for base in ("/dev/shm", tempfile.gettempdir()):
+        try:
+            if os.path.isdir(base) and shutil.disk_usage(base).free > n_bytes * 1.2 + (2 << 30):
+                return tempfile.mkdtemp(prefix="mxp_fullsize_", dir=base)
+        except OSError:
+            continue
+    return None
+
+
+def _whole_checkpoint_against_cpu_oracle(config: int, rank: int, n_files_expected: int, placed_expected: int, oracle, oracle_c):
+    """Writes one benchmark configuration's checkpoint files at full size, places the whole rank share on the CPU with
+    the oracle (numpy planner + C executor over the same files) and on the GPU twice - ingested from the files and
+    from the staged copy - and compares EVERY parameter buffer byte for byte, every checksum with the oracle's
+    safe_checksum and every digest with the oracle's tensor_digest (engines/vllm/refit/installer.py:419-424,
+    tensor_utils.py:27-44, refit/reshard/verify.py:79-155)."""
+    import shutil
+
+    from oracle import cpu_path
+
+    layout, tp, ep, n_shards, ck_dtype, ck_kind = models.baseline_config(config)
+    kw = {"dtype": ck_dtype, "edge_cases": ck_kind} if ck_dtype and config in (2, 3) else {}
+    tensors = layout.checkpoint(**kw)
+    total = sum(t.nbytes for t in tensors)
+    workdir = _room_for(total)
+    if workdir is None:
+        pytest.skip(f"no file system with room for the {total / 1e9:.1f} GB checkpoint of configuration {config}")
+    try:
+        synth.write_checkpoint(tensors, workdir, n_shards=n_shards, seed=SEED, threads=16)
+        ck = Checkpoint(workdir)
+        assert len(ck.files()) == n_files_expected and sum(t.nbytes for t in ck.tensors()) == total
+        rv = layout.rank_view(tp_size=tp, tp_rank=rank, ep_size=ep, ep_rank=rank % ep)
+        plan = PlacementPlan(ck, rv.params, tp_size=tp, tp_rank=rank, stacked_params_mapping=rv.stacked_params_mapping,
+                             expert_mapping=rv.expert_mapping)
+        assert plan.totals()["placed_bytes"] == placed_expected
+        cpu = cpu_path.run(workdir, [(p.name, p.dtype, p.shape) for p in rv.params], tp_size=tp, tp_rank=rank,
+                           stacked=rv.stacked_params_mapping, threads=16)
+        assert cpu["placed_bytes"] == placed_expected
+        want = {n: np.frombuffer(t.tobytes(), dtype=np.uint8) for n, t in cpu["params"].items()}
+        want_sums = [cpu["checksums"][p.name] for p in plan.params]
+        # the C executor's checksums are the oracle's own, checked against the numpy statement on the smaller buffers
+        for p in plan.params:
+            if p.nbytes <= (8 << 20):
+                assert cpu["checksums"][p.name] == oracle.safe_checksum_bytes(want[p.name]), p.name
+        want_digests = [oracle.tensor_digest_bytes(want[p.name]) for p in plan.params]
+        eng = PlacementEngine(0)
+        eng.set_fused_digests(True)
+        for mode in ("ingest", "resident"):
+            dst = eng.allocate(plan, fill=0xE7)
+            if mode == "ingest":
+                stats = eng.execute(plan, dst)
+                assert stats["placed_bytes"] == placed_expected
+            else:
+                staged = [torch.from_numpy(np.fromfile(f["path"], dtype=np.uint8)).cuda() for f in ck.files()]
+                eng.execute_resident(plan, staged, dst)
+                del staged
+            sums, digests = eng.checksums(plan), eng.digests(plan)
+            assert sums == want_sums, (mode, [p.name for p, a, b in zip(plan.params, sums, want_sums) if a != b][:5])
+            assert digests == want_digests, (mode, [p.name for p, a, b in zip(plan.params, digests, want_digests) if a != b][:5])
+            assert eng.digest(dst) == want_digests  # the stand-alone pass over the finished buffers
+            for p, d in zip(plan.params, dst):
+                assert np.array_equal(d.view(torch.uint8).reshape(-1).cpu().numpy(), want[p.name]), (mode, p.name)
+            del dst
+        eng.close()
+        plan.close()
+        ck.close()
+    finally:
+        shutil.rmtree(workdir, ignore_errors=True)
+
+
+def test_gpt2_small_whole_checkpoint_at_real_shapes(oracle, oracle_c, mxp):
+    """Configuration 1 at its real shapes: one file, 148 fp16 tensors, 248,879,616 bytes, TP=1 - all buffers."""
+    _whole_checkpoint_against_cpu_oracle(1, 0, 1, 248_879_616, oracle, oracle_c)
+
+
+def test_llama3_8b_whole_rank_share_against_the_cpu_oracle(oracle, oracle_c, mxp):
+    """Configuration 2: the 16 GB checkpoint in 4 shard files, rank 5 of 8 - all 195 buffers byte for byte."""
+    _whole_checkpoint_against_cpu_oracle(2, RANK, 4, 2_008_031_232, oracle, oracle_c)
+
+
 def test_buffer_beyond_4_gib_wraps_positions_like_the_reference(oracle_c, gpu_engine):
     """A single buffer of 2^32 + 12,345 bytes: checksum positions wrap mod 2^32 exactly as the
     reference's masked int64 weights do (tensor_utils.py:39-42), in the stand-alone checksum,

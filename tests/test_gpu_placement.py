@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from helpers import cast_setup, make_plan, oracle_place, tiny_layouts
-from modelexpress_amd import synth
+from modelexpress_amd import models, synth
 
 pytestmark = pytest.mark.gpu
 
@@ -57,22 +57,27 @@ def test_families_match_oracle(name, gpu_engine, gpu_engine_band, oracle, tmp_pa
                 assert s == oracle.safe_checksum(want[p.name]), (name, mode, tp_rank, p.name)
 
 
-@pytest.mark.parametrize("name", ["llama_tp4", "llama_f32_refit", "llama_bf16_into_f32", "deepseek_ep"])
+# o_proj rows of 2,560 bytes out of a pitch of 81,920: far enough apart that packed rows under direct I/O are
+# read one request per row, where the tiny layouts' rows share requests
+WIDE_ROWS = (models.Llama(layers=1, hidden=64, ffn=3072, q_heads=512, kv_heads=32, head_dim=80, vocab=256), 32, 1, 2, {})
+
+
+@pytest.mark.parametrize("name", ["llama_tp4", "llama_f32_refit", "llama_bf16_into_f32", "deepseek_ep", "wide_rows"])
 def test_direct_io_ranges_match_oracle(name, oracle, tmp_path, mxp):
     """O_DIRECT mode: every range is widened to 4 KiB blocks (also past the end of the last
     tensor) and boxes start inside the slot; results must not change.  Where the file system
     refuses O_DIRECT the engine falls back to buffered reads of the same widened ranges."""
     from modelexpress_amd.engine import PlacementEngine
 
-    layout, tp, ep, shards, ck_kw = tiny_layouts()[name]
+    layout, tp, ep, shards, ck_kw = WIDE_ROWS if name == "wide_rows" else tiny_layouts()[name]
     ck_kw, param_dtype, cast, _ratio = cast_setup(ck_kw)
     synth.write_checkpoint(layout.checkpoint(**ck_kw), str(tmp_path), n_shards=shards, seed=9)
     tp_rank = tp - 1
     rv = layout.rank_view(tp_size=tp, tp_rank=tp_rank, ep_size=ep, ep_rank=tp_rank % ep, param_dtype=param_dtype)
     want = oracle_place(oracle, str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
     ck, plan = make_plan(str(tmp_path), rv, tp_size=tp, tp_rank=tp_rank, allow_cast=cast)
-    # default under direct I/O: whole row bands, gathered on the device; then strided rows packed by the readers
-    for pack in (None, True):
+    # default (strided rows packed by the readers out of large requests), then whole row bands gathered on the device
+    for pack in (None, False):
         eng = PlacementEngine(0, ring_slots=3, slot_bytes=1 << 17, reader_threads=2, streams=2, use_o_direct=True,
                               pack_strided_on_host=pack)
         dst = eng.allocate(plan, fill=0x11)
