@@ -442,6 +442,73 @@ def _other_config(config: int, rank: int, seed: int, steps: int = 5, warmup: int
         shutil.rmtree(hdr, ignore_errors=True)
 
 
+def _transpose_ops(eng) -> dict:
+    """The transposed-view operators (mxp_permute_copy / mxp_copy_view / mxp_copy_views): plain, converting and the MLA
+    W_UK_T shapes (engines/vllm/refit/receiver.py:252-261), each with its kernel time and its time per call."""
+    import torch
+
+    from modelexpress_amd.engine import CAST_CODES
+
+    ops = {}
+    small_note = ("one call moves %.0f MB: at this size a launch's fixed cost of a few microseconds is most of the time; the "
+                  "61-layer entries are the same transpose batched into one launch")
+    # plain: a square bf16 matrix, a batch of smaller ones and the MLA W_UK_T shape
+    for label, shape, perm in (("transpose_bf16_16384x16384", (16384, 16384), (1, 0)),
+                               ("transpose_bf16_16x4096x4096", (16, 4096, 4096), (0, 2, 1)),
+                               ("mla_w_uk_t_bf16_128x128x512", (128, 128, 512), (1, 2, 0))):
+        nbytes = 2
+        for v in shape:
+            nbytes *= v
+        a = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 256)
+        b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        ms, k_ms = _timed_op(eng, lambda: eng.permute_copy(a, b, shape, perm, 2, checksum=False))
+        ops[label] = {"bytes": nbytes, **_op_rates(2 * nbytes, ms, k_ms)}
+        if ms < 0.02:
+            ops[label]["note"] = small_note % (2 * nbytes / 1e6)
+        del a, b
+    # converting on the way: an fp32 master weight written transposed as bf16, a bf16 weight widened, and the MLA
+    # W_UK_T shape out of an fp8 kv_b_proj
+    for label, src_dt, dst_dt, shape, perm in (
+            ("transpose_f32_bf16_16384x16384", "F32", "BF16", (16384, 16384), (1, 0)),
+            ("transpose_bf16_f32_16384x16384", "BF16", "F32", (16384, 16384), (1, 0)),
+            ("transpose_bf16_f32_4x8192x8192", "BF16", "F32", (4, 8192, 8192), (0, 2, 1)),
+            ("mla_w_uk_t_f8_bf16_128x128x512", "F8_E4M3", "BF16", (128, 128, 512), (1, 2, 0))):
+        se = {"F32": 4, "BF16": 2, "F8_E4M3": 1}[src_dt]
+        de = {"F32": 4, "BF16": 2}[dst_dt]
+        n_el = 1
+        for v in shape:
+            n_el *= v
+        st = [1] * len(shape)
+        for d in range(len(shape) - 2, -1, -1):
+            st[d] = st[d + 1] * shape[d + 1]
+        v_shape, v_strides = [shape[q] for q in perm], [st[q] for q in perm]
+        a = torch.empty(n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256)
+        b = torch.empty(n_el * de, dtype=torch.uint8, device="cuda")
+        code = CAST_CODES[(src_dt, dst_dt)]
+        ms, k_ms = _timed_op(eng, lambda: eng.copy_view(a, b, v_shape, de, src_strides=v_strides, cast=code, checksum=False))
+        ops[label] = {"elements": n_el, **_op_rates((se + de) * n_el, ms, k_ms)}
+        if ms < 0.02:
+            ops[label]["note"] = small_note % ((se + de) * n_el / 1e6)
+        del a, b
+    # the W_UK_T of every layer of a DeepSeek-V3-shaped model in one call (61 transposes, one launch); every layer's
+    # tensors are allocations of their own, as a model's are
+    H, nope, lat, layers = 128, 128, 512, 61
+    for label, src_dt, se in (("mla_w_uk_t_61_layers_bf16", "BF16", 2), ("mla_w_uk_t_61_layers_f8_bf16", "F8_E4M3", 1)):
+        n_el = H * nope * lat
+        srcs = [torch.empty(n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256) for _ in range(layers)]
+        dsts = [torch.empty(n_el * 2, dtype=torch.uint8, device="cuda") for _ in range(layers)]
+        code = 0 if src_dt == "BF16" else CAST_CODES[(src_dt, "BF16")]
+        views = [{"src": srcs[k], "dst": dsts[k], "shape": (nope, lat, H), "elem_size": 2,
+                  "src_strides": (lat, 1, nope * lat), "cast": code} for k in range(layers)]
+        arr = eng.views_array(views)  # built once: marshalling 61 views in Python takes longer than the launch
+        ms, k_ms = _timed_op(eng, lambda: eng.copy_views_array(arr, len(views)))
+        kind, tile_rows, tile_row_bytes = eng.describe_views(views)[0]
+        ops[label] = {"elements": layers * n_el, **_op_rates((se + 2) * layers * n_el, ms, k_ms),
+                      "form": kind + (f" ({tile_rows} rows x {tile_row_bytes} B)" if tile_rows else "")}
+        del srcs, dsts, views, arr
+    return ops
+
+
 def _op_rates(traffic_bytes: int, ms: float, kernel_ms) -> dict:
     """Figures of one stand-alone operator: `ms` is a call as the stream saw it (descriptor upload and
     dispatch gaps included), `kernel_ms` the launch itself; `frac_of_hbm_peak` is the kernel's, like
@@ -519,6 +586,10 @@ def main() -> int:
                          "gathers from the checkpoint's pitch and from a padded one, reads alone, writes alone)")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the block of the other four configurations that the default run appends")
+    ap.add_argument("--transposes", action="store_true",
+                    help="run only the transposed-view operators, once in the forms the library picks and once with every "
+                         "transpose forced into the wavefront-autonomous form, and print both (the command the transpose "
+                         "profiles under profiles/ are taken with)")
     ap.add_argument("--seed", type=int, default=20240229)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -535,6 +606,18 @@ def main() -> int:
     from modelexpress_amd.engine import CAST_CODES, Checkpoint, PlacementEngine, PlacementPlan
 
     _lib.lib()  # fail loudly if the HIP library is missing
+    if args.transposes:
+        from modelexpress_amd.engine import set_transpose_form
+
+        eng = PlacementEngine(0)
+        res = {}
+        for label, form in (("library_choice", 0), ("wavefront_autonomous_forced", 1)):
+            set_transpose_form(form)
+            res[label] = _transpose_ops(eng)
+        set_transpose_form(0)
+        eng.close()
+        print(json.dumps({"transposes": res, "hbm_peak_gbps": HBM_PEAK_GBPS}), flush=True)
+        return 0
     w = _workload(args.config, args.rank, layers=args.layers, rank_local=args.rank_local)
     layout, tp, ep, n_shards, cast = w["layout"], w["tp"], w["ep"], w["n_shards"], w["cast"]
     tensors, total_bytes, rank, ep_rank, rv = w["tensors"], w["total_bytes"], w["rank"], w["ep_rank"], w["rv"]
@@ -686,21 +769,6 @@ def main() -> int:
                                             "frac_of_hbm_peak": round(2 * placed / ms / 1e6 / HBM_PEAK_GBPS, 4),
                                             "note": "torch.Tensor.copy_ between two contiguous device buffers; not part of the path"}
             del a, b
-            # LDS transpose (permuted copies): a square bf16 matrix, a batch of smaller ones and the MLA W_UK_T shape
-            for label, shape, perm in (("transpose_bf16_16384x16384", (16384, 16384), (1, 0)),
-                                       ("transpose_bf16_16x4096x4096", (16, 4096, 4096), (0, 2, 1)),
-                                       ("mla_w_uk_t_bf16_128x128x512", (128, 128, 512), (1, 2, 0))):
-                nbytes = 2
-                for v in shape:
-                    nbytes *= v
-                a = torch.empty(nbytes, dtype=torch.uint8, device="cuda").random_(0, 256)
-                b = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
-                ms, k_ms = _timed_op(eng, lambda: eng.permute_copy(a, b, shape, perm, 2, checksum=False))
-                ops[label] = {"bytes": nbytes, **_op_rates(2 * nbytes, ms, k_ms)}
-                if ms < 0.02:
-                    ops[label]["note"] = ("one call moves %.0f MB: at this size a launch's fixed cost of a few microseconds is most of "
-                                          "the time; the 61-layer entries are the same transpose batched into one launch" % (2 * nbytes / 1e6))
-                del a, b
             # the other conversions of copy_ on 2^28 elements (6 bytes of traffic per element)
             n_el = 1 << 28
             for src_dt, dst_dt in (("BF16", "F32"), ("F32", "F16")):
@@ -713,44 +781,7 @@ def main() -> int:
                 ms, k_ms = _timed_op(eng, lambda: eng.cast(a, b, n_el, src_dt, dst_dt, checksum=False))
                 ops[f"cast_{src_dt.lower()}_{dst_dt.lower()}"] = {"elements": n_el, **_op_rates(6 * n_el, ms, k_ms)}
                 del a, b
-            # transposes that convert on the way: an fp32 master weight written transposed as bf16, a bf16
-            # weight widened, and the MLA W_UK_T shape out of an fp8 kv_b_proj
-            for label, src_dt, dst_dt, shape, perm in (
-                    ("transpose_f32_bf16_16384x16384", "F32", "BF16", (16384, 16384), (1, 0)),
-                    ("transpose_bf16_f32_16384x16384", "BF16", "F32", (16384, 16384), (1, 0)),
-                    ("mla_w_uk_t_f8_bf16_128x128x512", "F8_E4M3", "BF16", (128, 128, 512), (1, 2, 0))):
-                se = {"F32": 4, "BF16": 2, "F8_E4M3": 1}[src_dt]
-                de = {"F32": 4, "BF16": 2}[dst_dt]
-                n_el = 1
-                for v in shape:
-                    n_el *= v
-                st = [1] * len(shape)
-                for d in range(len(shape) - 2, -1, -1):
-                    st[d] = st[d + 1] * shape[d + 1]
-                v_shape, v_strides = [shape[q] for q in perm], [st[q] for q in perm]
-                a = torch.empty(n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256)
-                b = torch.empty(n_el * de, dtype=torch.uint8, device="cuda")
-                code = CAST_CODES[(src_dt, dst_dt)]
-                ms, k_ms = _timed_op(eng, lambda: eng.copy_view(a, b, v_shape, de, src_strides=v_strides, cast=code, checksum=False))
-                ops[label] = {"elements": n_el, **_op_rates((se + de) * n_el, ms, k_ms)}
-                if ms < 0.02:
-                    ops[label]["note"] = ("one call moves %.0f MB: at this size a launch's fixed cost of a few microseconds is most of "
-                                          "the time; the 61-layer entries below are the same transposes batched into one launch"
-                                          % ((se + de) * n_el / 1e6))
-                del a, b
-            # the W_UK_T of every layer of a DeepSeek-V3-shaped model in one call (61 transposes, one launch)
-            H, nope, lat, layers = 128, 128, 512, 61
-            for label, src_dt, se in (("mla_w_uk_t_61_layers_bf16", "BF16", 2), ("mla_w_uk_t_61_layers_f8_bf16", "F8_E4M3", 1)):
-                n_el = H * nope * lat
-                a = torch.empty(layers * n_el * se, dtype=torch.uint8, device="cuda").random_(0, 256)
-                b = torch.empty(layers * n_el * 2, dtype=torch.uint8, device="cuda")
-                code = 0 if src_dt == "BF16" else CAST_CODES[(src_dt, "BF16")]
-                views = [{"src": a[k * n_el * se:], "dst": b[k * n_el * 2:], "shape": (nope, lat, H), "elem_size": 2,
-                          "src_strides": (lat, 1, nope * lat), "cast": code} for k in range(layers)]
-                arr = eng.views_array(views)  # built once: marshalling 61 views in Python takes longer than the launch
-                ms, k_ms = _timed_op(eng, lambda: eng.copy_views_array(arr, len(views)))
-                ops[label] = {"elements": layers * n_el, **_op_rates((se + 2) * layers * n_el, ms, k_ms)}
-                del a, b, views, arr
+            ops.update(_transpose_ops(eng))
             # a refit's re-slice of per-expert sources into fused w13 buffers (48 layers x 128 experts x gate/up,
             # fp32 -> bf16): resolved and lowered once, then each step only launches
             from modelexpress_amd.reshard import RecordedCopy, ReslicePlan

@@ -50,6 +50,18 @@ int mxp_measure_read(const char* const* paths, int64_t n_paths, int32_t threads,
 int mxp_measure_gather(mxp_engine* engine, uint64_t rows, uint32_t row_bytes, uint64_t src_pitch, uint32_t col_offset,
                        int32_t cast, int32_t repeats, double* bytes_per_second);
 
+/* How mxp_copy_views would run each of `views` (nothing is launched): kinds[k] = 0 row or element
+ * boxes through the placement kernel, 1 a transpose in which every wavefront moves its own sub-tile,
+ * 2 a transpose in which a workgroup stages a whole tile of tile_rows[k] source rows x
+ * tile_row_bytes[k] source bytes (both 0 otherwise).  For tests and measurements: the choice between
+ * the two transpose forms is a heuristic of the library, not part of its contract. */
+int mxp_describe_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, int32_t* kinds, int32_t* tile_rows,
+                       int32_t* tile_row_bytes);
+
+/* Process-wide measurement switch: 1 makes every transposed view run in the wavefront-autonomous form, 0
+ * (the default) lets the library pick between that and the staged-tile form.  Results are identical. */
+int mxp_set_transpose_form(int32_t form);
+
 /* Seeded synthetic contents (test and benchmark inputs; same bytes on host and device).
  * kind: 0 ~N(0,0.02), 1 ones, 2 zeros, 3 normal with denormal/inf/NaN/tie edge cases at
  * 1e-6 density, 4 fp8 bytes over the finite e4m3 codes, 5 fp32 scales in [1e-4,1e-2],

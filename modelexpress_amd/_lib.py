@@ -181,6 +181,8 @@ BENCH_SIGNATURES = {
     "mxp_engine_set_launch_timing": (C.c_int, [_P, C.c_int32]),
     "mxp_engine_launch_times": (C.c_int, [_P, C.POINTER(C.c_float), C.c_int32, C.POINTER(C.c_int32)]),
     "mxp_measure_h2d": (C.c_int, [_P, C.c_uint64, C.c_int32, C.POINTER(C.c_double)]),
+    "mxp_describe_views": (C.c_int, [_P, C.POINTER(ViewCopy), C.c_int64, C.POINTER(C.c_int32), C.POINTER(C.c_int32), C.POINTER(C.c_int32)]),
+    "mxp_set_transpose_form": (C.c_int, [C.c_int32]),
     "mxp_measure_read": (C.c_int, [C.POINTER(C.c_char_p), C.c_int64, C.c_int32, C.c_uint64, C.c_int32, _U64P, C.POINTER(C.c_double)]),
     "mxp_synth_host": (C.c_int, [_P, C.c_uint64, C.c_int32, C.c_uint32, C.c_uint64, C.c_int32]),
     "mxp_synth_device": (C.c_int, [_P, C.c_uint64, C.c_int32, C.c_uint32, C.c_uint64, _P]),

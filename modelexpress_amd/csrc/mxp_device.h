@@ -195,13 +195,32 @@ struct TransposeDesc {
   uint32_t csum_bias;
   uint32_t waves_i;           // wavefronts of a workgroup along i (power of two, divides waves)
   uint32_t group_j;           // tiles along j that consecutive workgroups visit before stepping along i (>= 1)
-  uint32_t waves;             // wavefronts of a workgroup (1, 2, 4 or 8)
+  uint32_t waves;             // wavefronts of a workgroup (1, 2, 4 or 8; up to 16 for a panel)
+  // Panel form (panel_rows_log2 != 0): the workgroup stages a whole tile of 2^panel_rows_log2 source rows
+  // x 2^panel_chunks_log2 16-byte chunks in LDS, waits at a barrier and writes the transposed tile; the
+  // extents are whole multiples of the tile, both sides 16-byte aligned, waves = rows * chunks / 512.
+  uint32_t panel_rows_log2, panel_chunks_log2;
 };
+constexpr uint32_t kPanelLoads = 8;             // 16-byte loads per lane of a panel workgroup
+constexpr uint32_t kPanelMaxBytes = 128 * 1024; // staged tile
 // What the kernels assume of a descriptor (index arithmetic in 32 bits, workgroup shape).
 inline bool transpose_desc_ok(const TransposeDesc& d) {
+  if (d.panel_rows_log2) return d.n_tiles <= 0x7FFFFFFFull && (uint64_t)d.tiles_i * d.tiles_j <= 0x7FFFFFFFull;  // shape: panel_desc_ok
   return d.n_tiles <= 0x7FFFFFFFull && d.waves != 0 && d.waves <= (uint32_t)kTransposeWaves && (d.waves & (d.waves - 1)) == 0 &&
          d.waves_i != 0 && d.waves % d.waves_i == 0 && d.group_j != 0 && (uint64_t)d.tiles_i * d.tiles_j <= 0x7FFFFFFFull &&
          (uint64_t)d.tiles_i * d.group_j <= 0x7FFFFFFFull;
+}
+// What the panel kernels assume of a descriptor, for source / destination element sizes es / eo: they
+// have no edge handling, so whole tiles and 16-byte accesses everywhere are checked here, on the host.
+inline bool panel_desc_ok(const TransposeDesc& d, uint32_t es, uint32_t eo) {
+  if (!d.panel_rows_log2 || d.panel_rows_log2 > 10 || d.panel_chunks_log2 < 3 || d.panel_chunks_log2 > 13) return false;
+  if (es != 1 && es != 2 && es != 4) return false;
+  if (eo != 1 && eo != 2 && eo != 4) return false;
+  const uint64_t rows = 1ull << d.panel_rows_log2, chunks = 1ull << d.panel_chunks_log2, cols = chunks * 16 / es;
+  const uint64_t threads = rows * chunks / kPanelLoads;
+  return rows * chunks * 16 <= kPanelMaxBytes && threads >= 64 && threads <= 1024 && d.waves * 64ull == threads &&
+         rows >= 16 / eo && d.align_src >= 16 && d.align_dst >= 16 && d.ni == (uint64_t)d.tiles_i * rows &&
+         d.nj == (uint64_t)d.tiles_j * cols && d.n_tiles <= 0x7FFFFFFFull;
 }
 // One transpose of a batched launch: `first_tile` is the number of workgroups of the items
 // before it (items sorted by it; every item has d.n_tiles >= 1 and the same d.waves).
@@ -221,8 +240,26 @@ hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, 
                             uint32_t nan_bits, uint32_t* sum_out, Fan fan, hipStream_t stream);
 // `n_items` transposes of one (elem_size, op, waves) in a launch of `total_tiles` workgroups; the
 // host checks each descriptor as launch_transpose would (transpose_desc_ok).
+// `panel`: 0, or (panel_rows_log2 << 8 | panel_chunks_log2) shared by every item; `uniform_tiles`: 0, or - for
+// a panel batch whose items all have the descriptor `*common` - the number of tiles of each
+// (total_tiles == n_items * uniform_tiles); the kernel then takes the descriptor as an argument, and with
+// `items_host` (the same items, on the host) and at most kPanelArgItems of them their pointers as well.
 hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_items, uint64_t total_tiles, uint32_t waves,
-                                  int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream);
+                                  int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream, uint32_t panel = 0,
+                                  uint32_t uniform_tiles = 0, const TransposeDesc* common = nullptr,
+                                  const TransposeItem* items_host = nullptr);
+// Items of a uniform panel batch whose pointers fit the kernel argument block (`items_host` given).
+constexpr int kPanelArgItems = 96;
+// Field by field (the struct may hold padding).
+inline bool same_transpose_desc(const TransposeDesc& a, const TransposeDesc& b) {
+  bool eq = a.ni == b.ni && a.nj == b.nj && a.si == b.si && a.dj == b.dj && a.tiles_i == b.tiles_i && a.tiles_j == b.tiles_j &&
+            a.n_tiles == b.n_tiles && a.align_src == b.align_src && a.align_dst == b.align_dst && a.csum_bias == b.csum_bias &&
+            a.waves_i == b.waves_i && a.group_j == b.group_j && a.waves == b.waves && a.panel_rows_log2 == b.panel_rows_log2 &&
+            a.panel_chunks_log2 == b.panel_chunks_log2;
+  for (int k = 0; k < kMaxBatchDims; ++k)
+    eq = eq && a.batch_size[k] == b.batch_size[k] && a.batch_sstride[k] == b.batch_sstride[k] && a.batch_dstride[k] == b.batch_dstride[k];
+  return eq;
+}
 
 // Synthetic-checkpoint generator (mxp_synth.hip), same arithmetic on host and device.
 enum SynthKind : uint32_t {

@@ -1446,6 +1446,10 @@ int mxp_place_boxes(mxp_engine* engine, const mxp_box* in, int64_t n, uint32_t n
 extern "C++" {
 namespace {
 
+// Measurement switch (mxp_set_transpose_form): 0 = the library picks the form of a transpose, 1 = always the
+// wavefront-autonomous form.
+std::atomic<int> g_transpose_form{0};
+
 // dst_view[...] = src_view[...] for two strided views of one shape (strides in elements).
 // Dimensions are put in destination order (largest destination stride first) and merged
 // where both sides allow; then
@@ -1470,9 +1474,12 @@ enum ViewKind {
 };
 
 // Lowers one view copy.  Boxes are appended to `boxes` with their base pointers in `srcs` / `dsts`.
+// `call_bytes`: destination bytes of all the views of the call this view belongs to (0 = this view alone);
+// a transpose sizes its workgroups by whether the whole call, not this view, fills the chip.
 ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std::vector<uint64_t> ss,
                     std::vector<uint64_t> ds, int elem_size, int cast, uint32_t csum_slot, std::vector<BoxCopy>& boxes,
-                    std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, const char* what) {
+                    std::vector<const void*>& srcs, std::vector<void*>& dsts, TransposeJob& tr, const char* what,
+                    uint64_t call_bytes = 0) {
   const uint32_t op = seg_op_of_cast(cast);
   const uint64_t es = (uint64_t)elem_size;          // destination element
   const uint64_t es_s = op_src_bytes(op, es);       // source element
@@ -1611,6 +1618,42 @@ ViewKind lower_view(const void* src, void* dst, std::vector<uint64_t> size, std:
     }
     td.align_src = (uint32_t)vs;
     td.align_dst = (uint32_t)vd;
+    // Panel form (mxp_permute.hip) where it measured faster than the wavefront-autonomous one; it has no edge
+    // handling, so only whole tiles with 16-byte accesses on both sides qualify.
+    if (vs >= 16 && vd >= 16 && eb <= 4 && es <= 4 && g_transpose_form.load(std::memory_order_relaxed) != 1) {
+      auto is_pow2 = [](uint64_t v) { return v && !(v & (v - 1)); };
+      auto log2u = [](uint64_t v) { uint32_t l = 0; while ((1ull << l) < v) ++l; return l; };
+      const uint64_t row_src = td.nj * eb;  // bytes of one source row of the view
+      const uint64_t src_pitch = td.si * eb, dst_pitch = td.dj * es, v_rows = 16 / es;
+      uint64_t rows = 0, row_bytes = 0;
+      if (td.dj == td.ni && is_pow2(td.ni) && td.ni >= v_rows && td.ni <= 1024 && td.ni * es <= 1024) {
+        // short destination rows that abut: all of i in one tile, whose output is then one contiguous block
+        rows = td.ni;
+        row_bytes = 128;
+        while (row_bytes * 2 <= 4096 && rows * row_bytes * 2 <= kPanelMaxBytes && row_src % (row_bytes * 2) == 0) row_bytes *= 2;
+        // smaller tiles while the call would leave compute units without a workgroup
+        const uint64_t all_bytes = std::max<uint64_t>(call_bytes, batches * td.ni * td.nj * es);
+        while (row_bytes > 128 && rows * row_bytes / 2 >= 8192 && all_bytes / (rows * row_bytes / eb * es) < 2ull * kChipCus) row_bytes /= 2;
+      } else if (eb == 2 && es == 2 && src_pitch >= 32768 && dst_pitch >= 32768) {
+        rows = 512;      // 2-byte matrices with long pitches on both sides: 1 KiB destination runs, 256-byte source runs
+        row_bytes = 256;
+      } else if (eb == 2 && es == 4 && src_pitch >= 16384 && dst_pitch >= 32768) {
+        rows = 256;      // widening: 1 KiB destination runs out of 512-byte source runs
+        row_bytes = 512;
+      }
+      if (rows && td.ni % rows == 0 && row_src % row_bytes == 0 && rows * row_bytes >= 8192) {
+        TransposeDesc pd = td;
+        pd.panel_rows_log2 = log2u(rows);
+        pd.panel_chunks_log2 = log2u(row_bytes / 16);
+        pd.waves = (uint32_t)(rows * row_bytes / 16 / kPanelLoads / 64);
+        pd.waves_i = 1;
+        pd.group_j = 1;
+        pd.tiles_i = (uint32_t)(td.ni / rows);
+        pd.tiles_j = (uint32_t)(row_src / row_bytes);
+        pd.n_tiles = (uint64_t)pd.tiles_i * pd.tiles_j * batches;
+        if (panel_desc_ok(pd, (uint32_t)eb, (uint32_t)es)) td = pd;
+      }
+    }
     td.n_tiles = (uint64_t)td.tiles_i * td.tiles_j;
     for (int q = 0; q < kMaxBatchDims; ++q) td.n_tiles *= td.batch_size[q];
     if (!transpose_desc_ok(td)) fail(MXP_ERR_UNSUPPORTED, "the transposed view needs more workgroups than one launch holds");
@@ -1674,7 +1717,11 @@ struct TransposeGroup {
   uint32_t waves;
   int elem_size;
   uint32_t op;
+  uint32_t panel;  // 0, or panel_rows_log2 << 8 | panel_chunks_log2 of every item
+  uint32_t uniform_tiles;  // != 0: a panel group whose items all have the descriptor `common` and this many tiles
+  TransposeDesc common;
 };
+inline uint32_t panel_code(const TransposeDesc& d) { return d.panel_rows_log2 ? (d.panel_rows_log2 << 8 | d.panel_chunks_log2) : 0u; }
 
 // Sorts `jobs` into launch groups (`items` receives their descriptor table) and `singles`
 // (a kind of its own: launched with the descriptor as a kernel argument).
@@ -1684,7 +1731,9 @@ void group_transposes(const std::vector<TransposeJob>& jobs, std::vector<Transpo
   for (size_t k = 0; k < jobs.size(); ++k) {
     if (jobs[k].td.n_tiles) order.push_back(k);  // descriptors were checked when the views were lowered
   }
-  auto key = [&](size_t k) { return ((uint64_t)jobs[k].op << 16) | ((uint64_t)jobs[k].elem_size << 8) | jobs[k].td.waves; };
+  auto key = [&](size_t k) {
+    return ((uint64_t)panel_code(jobs[k].td) << 32) | ((uint64_t)jobs[k].op << 16) | ((uint64_t)jobs[k].elem_size << 8) | jobs[k].td.waves;
+  };
   std::stable_sort(order.begin(), order.end(), [&](size_t x, size_t y) { return key(x) < key(y); });
   for (size_t q = 0; q < order.size();) {
     size_t r = q;
@@ -1695,13 +1744,16 @@ void group_transposes(const std::vector<TransposeJob>& jobs, std::vector<Transpo
       singles.push_back(jobs[order[q]]);
     } else {
       const TransposeJob& j0 = jobs[order[q]];
-      groups.push_back(TransposeGroup{items.size(), r - q, tiles, j0.td.waves, j0.elem_size, j0.op});
+      bool uniform = j0.td.panel_rows_log2 != 0 && j0.td.n_tiles <= 0xFFFFFFFFull;
       uint64_t first = 0;
       for (size_t k = q; k < r; ++k) {
         const TransposeJob& j = jobs[order[k]];
+        uniform = uniform && same_transpose_desc(j.td, j0.td);
         items.push_back(TransposeItem{static_cast<const uint8_t*>(j.src), static_cast<uint8_t*>(j.dst), first, 0, j.td});
         first += j.td.n_tiles;
       }
+      groups.push_back(TransposeGroup{items.size() - (r - q), r - q, tiles, j0.td.waves, j0.elem_size, j0.op, panel_code(j0.td),
+                                      uniform ? (uint32_t)j0.td.n_tiles : 0u, j0.td});
     }
     q = r;
   }
@@ -1737,7 +1789,7 @@ void run_transposes(mxp_engine& e, const std::vector<TransposeJob>& jobs, hipStr
   for (const TransposeGroup& g : groups) {
     LaunchTimer timer(e, stream);
     HIP_OK(launch_transpose_batch(tab.dev.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
-                                  e.opt.nan_bits, stream));
+                                  e.opt.nan_bits, stream, g.panel, g.uniform_tiles, &g.common, items.data() + g.first));
     timer.done();
   }
   HIP_OK(hipEventRecord(tab.busy, stream));
@@ -1769,6 +1821,13 @@ void check_view_args(const mxp_engine* engine, int32_t ndim, const int64_t* shap
 void lower_views(const mxp_engine* engine, const mxp_view_copy* views, int64_t n, std::vector<BoxCopy>& boxes,
                  std::vector<const void*>& srcs, std::vector<void*>& dsts, std::vector<TransposeJob>& transposes,
                  const char* what) {
+  uint64_t call_bytes = 0;  // what the whole call writes: sizes the transposes' workgroups
+  for (int64_t k = 0; k < n; ++k) {
+    if (views[k].ndim < 0 || views[k].ndim > MXP_MAX_DIMS || views[k].elem_size <= 0) continue;  // refused below
+    uint64_t el = 1;
+    for (int d = 0; d < views[k].ndim; ++d) el *= views[k].shape[d] > 0 ? (uint64_t)views[k].shape[d] : 0;
+    call_bytes += el * (uint64_t)views[k].elem_size;
+  }
   for (int64_t k = 0; k < n; ++k) {
     const mxp_view_copy& v = views[k];
     check_view_args(engine, v.ndim, v.shape, v.elem_size, what);
@@ -1780,7 +1839,8 @@ void lower_views(const mxp_engine* engine, const mxp_view_copy* views, int64_t n
     TransposeJob tr{};
     const auto s_st = strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, what);
     const auto d_st = strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, what);
-    const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts, tr, what);
+    const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts, tr, what,
+                                     call_bytes);
     if (kind == kViewTranspose) transposes.push_back(tr);
   }
 }
@@ -1798,6 +1858,7 @@ struct mxp_view_plan {
   std::vector<TransposeJob> singles;
   std::vector<TransposeGroup> groups;
   DevBuf<TransposeItem> items;
+  std::vector<TransposeItem> items_host;  // the same table: small uniform batches pass their pointers as kernel arguments
   uint64_t bytes = 0;  // destination bytes one run writes
 };
 
@@ -2004,6 +2065,44 @@ int mxp_copy_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, vo
   });
 }
 
+int mxp_set_transpose_form(int32_t form) {
+  return guard([&] {
+    if (form != 0 && form != 1) throw Error(MXP_ERR_ARG, "mxp_set_transpose_form: 0 (the library picks) or 1 (wavefront-autonomous)");
+    g_transpose_form.store(form, std::memory_order_relaxed);
+  });
+}
+
+int mxp_describe_views(mxp_engine* engine, const mxp_view_copy* views, int64_t n, int32_t* kinds, int32_t* tile_rows,
+                       int32_t* tile_row_bytes) {
+  return guard([&] {
+    if (!engine || n < 0 || (n && (!views || !kinds))) throw Error(MXP_ERR_ARG, "mxp_describe_views: bad argument");
+    uint64_t call_bytes = 0;
+    for (int64_t k = 0; k < n; ++k) {
+      uint64_t el = 1;
+      for (int d = 0; d < views[k].ndim && d < MXP_MAX_DIMS; ++d) el *= views[k].shape[d] > 0 ? (uint64_t)views[k].shape[d] : 0;
+      call_bytes += el * (uint64_t)(views[k].elem_size > 0 ? views[k].elem_size : 0);
+    }
+    for (int64_t k = 0; k < n; ++k) {  // each view lowered as mxp_copy_views would lower it among the others
+      std::vector<BoxCopy> boxes;
+      std::vector<const void*> srcs;
+      std::vector<void*> dsts;
+      const mxp_view_copy& v = views[k];
+      check_view_args(engine, v.ndim, v.shape, v.elem_size, "mxp_describe_views");
+      std::vector<uint64_t> size;
+      for (int d = 0; d < v.ndim; ++d) size.push_back((uint64_t)v.shape[d]);
+      TransposeJob tr{};
+      const auto s_st = strides_or_row_major(v.contiguous_src ? nullptr : v.src_strides, v.shape, v.ndim, "mxp_describe_views");
+      const auto d_st = strides_or_row_major(v.contiguous_dst ? nullptr : v.dst_strides, v.shape, v.ndim, "mxp_describe_views");
+      const ViewKind kind = lower_view(v.src, v.dst, size, s_st, d_st, v.elem_size, v.cast, 0xFFFFFFFFu, boxes, srcs, dsts, tr,
+                                       "mxp_describe_views", call_bytes);
+      const bool panel = kind == kViewTranspose && tr.td.panel_rows_log2 != 0;
+      kinds[k] = kind == kViewTranspose ? (panel ? 2 : 1) : 0;
+      if (tile_rows) tile_rows[k] = panel ? (int32_t)(1u << tr.td.panel_rows_log2) : 0;
+      if (tile_row_bytes) tile_row_bytes[k] = panel ? (int32_t)(16u << tr.td.panel_chunks_log2) : 0;
+    }
+  });
+}
+
 int mxp_view_plan_create(mxp_engine* engine, const mxp_view_copy* views, int64_t n, mxp_view_plan** out) {
   return guard([&] {
     if (!out) throw Error(MXP_ERR_ARG, "mxp_view_plan_create: null out");
@@ -2041,6 +2140,7 @@ int mxp_view_plan_create(mxp_engine* engine, const mxp_view_copy* views, int64_t
     std::vector<TransposeItem> items;
     group_transposes(transposes, items, vp->groups, vp->singles);
     if (!items.empty()) vp->items.upload(items.data(), items.size());
+    vp->items_host = items;
     for (const auto& t : transposes) {
       uint64_t elems = t.td.ni * t.td.nj;
       for (int q = 0; q < kMaxBatchDims; ++q) elems *= t.td.batch_size[q];
@@ -2066,7 +2166,8 @@ int mxp_view_plan_run(mxp_engine* engine, mxp_view_plan* plan, void* stream_v) {
       HIP_OK(launch_transpose(t.src, t.dst, t.td, t.elem_size, t.op, engine->opt.nan_bits, nullptr, Fan{}, stream));
     for (const auto& g : plan->groups)
       HIP_OK(launch_transpose_batch(plan->items.p + g.first, (uint32_t)g.count, g.tiles, g.waves, g.elem_size, g.op,
-                                    engine->opt.nan_bits, stream));
+                                    engine->opt.nan_bits, stream, g.panel, g.uniform_tiles, &g.common,
+                                    plan->items_host.empty() ? nullptr : plan->items_host.data() + g.first));
   });
 }
 

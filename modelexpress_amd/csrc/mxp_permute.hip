@@ -366,6 +366,168 @@ __global__ __launch_bounds__(kThreads) void transpose_batch_kernel(const Transpo
   transpose_tile<ES, OP>(it.src, it.dst, it.d, (uint64_t)blockIdx.x - it.first_tile, nan_bits, lds, wave, cs);
 }
 
+
+// ---- panel form ------------------------------------------------------------------------------
+// The whole workgroup stages one tile of A = 2^a source rows (i) x C = 2^c 16-byte chunks (j) in LDS
+// in the source's format, waits at a barrier, and writes the transposed tile: every lane issues its
+// eight 16-byte loads first (a wavefront load covers whole rows or whole 1 KiB pieces of a row), the
+// tile lands in LDS with the chunk index XOR-swizzled by the row group, and after the barrier a lane
+// gathers the V = 16 / (destination element) rows of one destination chunk as dwords down one LDS
+// column - 4 / (source element) destination rows per gather - regroups bytes with v_perm_b32,
+// converts, and stores; consecutive lanes take consecutive chunks along i, so a wavefront store is one
+// contiguous KiB of a destination row (or of several abutting rows).  A compute unit alternates
+// between a read burst and a write burst of up to 128 KiB, like the placement kernel.
+//
+// Where it pays (measured against the wavefront-autonomous form on the same box): destinations whose
+// rows are short and abut, so that a tile's output is one contiguous block (the MLA W_UK_T batch out of
+// bf16: 0.346 against 0.383 ms); 2-byte matrices with both pitches of 32 KiB or more (16384 x 16384:
+// 0.178 against 0.198 ms); widening transposes, two thirds of whose traffic is stores (8192 x 8192
+// bf16 -> fp32 x 4: 0.267 against 0.317 ms).  Tall, wide and small-pitch matrices stay with the
+// wavefront-autonomous form, which reads their rows better.  The host picks (mxp_engine.cpp).
+// No edge handling: whole tiles, 16-byte aligned on both sides (panel_desc_ok).
+template <int ES, int OP>
+__device__ __forceinline__ void panel_tile(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst, const TransposeDesc& d,
+                                           uint64_t tile, uint32_t nan_bits, uint8_t* lds, Csum& cs) {
+  constexpr int EO = out_elem(ES, OP);
+  constexpr uint32_t V = 16 / EO;        // source rows in one 16-byte destination chunk
+  constexpr uint32_t CPR = 4 / ES;       // destination rows fed by one LDS dword column
+  constexpr int KT = 2 * EO;             // gathers per lane: (columns / CPR) * (rows / V) / lanes
+  static_assert(ES == 1 || ES == 2 || ES == 4, "panel transposes read 1-, 2- or 4-byte elements");
+  static_assert(Sub<ES, OP>::NW == (int)V && Sub<ES, OP>::CPR == (int)CPR, "one dword per gathered row");
+  const uint32_t a = d.panel_rows_log2, c = d.panel_chunks_log2;
+  const uint32_t C = 1u << c, row_bytes = C << 4, sw = 7u;  // C >= 8
+  const uint32_t threads = blockDim.x, t = threadIdx.x;
+  const uint32_t nic_log2 = a - (uint32_t)__builtin_ctz(V), nic_mask = (1u << nic_log2) - 1u;
+  // tile -> (batch, tile_j, tile_i), tile_i fastest; workgroup-uniform
+  const uint64_t per_batch = (uint64_t)d.tiles_i * d.tiles_j;
+  uint64_t b = tile / per_batch;
+  const uint32_t within = (uint32_t)(tile % per_batch);
+  const uint32_t ti = within % d.tiles_i, tj = within / d.tiles_i;
+  uint64_t s_off = 0, d_off = 0;
+#pragma unroll
+  for (int k = kMaxBatchDims - 1; k >= 0; --k) {
+    const uint64_t n = d.batch_size[k];
+    const uint64_t idx = b % n;
+    b /= n;
+    s_off += idx * d.batch_sstride[k];
+    d_off += idx * d.batch_dstride[k];
+  }
+  const uint64_t i0 = (uint64_t)ti << a, j0 = (uint64_t)tj * (row_bytes / ES);
+  const uint64_t d_el = d_off + j0 * d.dj + i0;
+  const uint8_t* sp = src + (s_off + i0 * d.si + j0) * ES;
+  uint8_t* dp = dst + d_el * EO;
+  const uint64_t si_b = d.si * ES, dj_b = d.dj * EO;
+  const uint32_t csum_base = (uint32_t)(d_el * EO) + d.csum_bias;
+  {
+    uint4 x[kPanelLoads];
+#pragma unroll
+    for (uint32_t k = 0; k < kPanelLoads; ++k) {
+      const uint32_t q = k * threads + t, row = q >> c, cc = q & (C - 1u);
+      x[k] = ld16_nt(sp + (uint64_t)row * si_b + (cc << 4));
+    }
+#pragma unroll
+    for (uint32_t k = 0; k < kPanelLoads; ++k) {
+      const uint32_t q = k * threads + t, row = q >> c, cc = q & (C - 1u);
+      *reinterpret_cast<uint4*>(lds + row * row_bytes + ((cc ^ ((row / V) & sw)) << 4)) = x[k];
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < KT; ++k) {
+    const uint32_t q = (uint32_t)k * threads + t, ic = q & nic_mask, jg = q >> nic_log2;
+    const uint32_t bytecol = jg << 2;
+    const uint8_t* l = lds + (ic * V) * row_bytes + (((bytecol >> 4) ^ (ic & sw)) << 4) + (bytecol & 15u);
+    uint32_t w[V];
+#pragma unroll
+    for (uint32_t kk = 0; kk < V; ++kk) w[kk] = *reinterpret_cast<const uint32_t*>(l + kk * row_bytes);
+    const uint64_t off = (uint64_t)(jg * CPR) * dj_b + (ic << 4);
+    const uint32_t pos = csum_base + (uint32_t)off;
+    {
+      const uint4 v = make_chunk<ES, OP, 0>(w, nan_bits);
+      st16_nt(dp + off, v);
+      cs.add16(v, pos);
+    }
+    if constexpr (CPR >= 2) {
+      const uint4 v = make_chunk<ES, OP, 1>(w, nan_bits);
+      st16_nt(dp + off + dj_b, v);
+      cs.add16(v, pos + (uint32_t)dj_b);
+    }
+    if constexpr (CPR == 4) {
+      const uint4 v2 = make_chunk<ES, OP, 2>(w, nan_bits);
+      st16_nt(dp + off + 2 * dj_b, v2);
+      cs.add16(v2, pos + (uint32_t)(2 * dj_b));
+      const uint4 v3 = make_chunk<ES, OP, 3>(w, nan_bits);
+      st16_nt(dp + off + 3 * dj_b, v3);
+      cs.add16(v3, pos + (uint32_t)(3 * dj_b));
+    }
+  }
+}
+
+template <int ES, int OP>
+__global__ __launch_bounds__(1024) void panel_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                      const TransposeDesc d, uint32_t nan_bits, uint32_t* __restrict__ sum_out,
+                                                      Fan fan) {
+  extern __shared__ __align__(16) uint8_t lds[];  // the staged tile
+  __shared__ uint32_t wave_sums[16];
+  Csum cs;
+  panel_tile<ES, OP>(src, dst, d, blockIdx.x, nan_bits, lds, cs);
+  if (sum_out) {
+    const uint32_t w = wave_sum_u32(cs.fold());
+    if ((threadIdx.x & 63) == 0) wave_sums[threadIdx.x >> 6] = w;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      uint32_t t = 0;
+      for (uint32_t k = 0; k < (blockDim.x >> 6); ++k) t += wave_sums[k];
+      atomicAdd(&sum_out[(blockIdx.x & fan.mask) * fan.pitch], t);
+    }
+  }
+}
+
+// `uniform_tiles` != 0: every item has that many tiles and the same descriptor (the usual batch: one transpose
+// of one shape per layer), which then travels as the kernel argument `common`; the item is a division away
+// and only its two pointers are loaded.  A panel workgroup has a compute unit to itself, so what it waits for
+// before its first data load is not hidden by other workgroups: the bisection and the 224-byte descriptor load
+// cost the 61-layer MLA batch 8 % (0.378 against 0.350 ms).
+template <int ES, int OP>
+__global__ __launch_bounds__(1024) void panel_batch_kernel(const TransposeItem* __restrict__ items, uint32_t n_items,
+                                                            uint32_t nan_bits, uint32_t uniform_tiles, const TransposeDesc common) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  uint32_t lo = 0;
+  if (uniform_tiles) {
+    lo = blockIdx.x / uniform_tiles;
+    const TransposeItem& it = items[lo];
+    Csum cs;
+    panel_tile<ES, OP>(it.src, it.dst, common, (uint64_t)(blockIdx.x - lo * uniform_tiles), nan_bits, lds, cs);
+    return;
+  } else {
+    uint32_t hi = n_items;  // the last item with first_tile <= blockIdx.x
+    while (hi - lo > 1) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (items[mid].first_tile <= (uint64_t)blockIdx.x) lo = mid;
+      else hi = mid;
+    }
+  }
+  const TransposeItem& it = items[lo];
+  Csum cs;
+  panel_tile<ES, OP>(it.src, it.dst, it.d, (uint64_t)blockIdx.x - it.first_tile, nan_bits, lds, cs);
+}
+
+// The same for a uniform batch of at most kPanelArgItems items, whose pointers travel in the kernel argument
+// block as well: a workgroup's two pointers are then loaded together with the descriptor when the wavefront
+// starts, instead of after it (a table in memory is addressed through a pointer that is itself an argument).
+struct PanelPtrTable {
+  const uint8_t* src[kPanelArgItems];
+  uint8_t* dst[kPanelArgItems];
+};
+template <int ES, int OP>
+__global__ __launch_bounds__(1024) void panel_batch_args_kernel(const PanelPtrTable ptrs, uint32_t nan_bits, uint32_t uniform_tiles,
+                                                                 const TransposeDesc common) {
+  extern __shared__ __align__(16) uint8_t lds[];
+  const uint32_t item = blockIdx.x / uniform_tiles;
+  Csum cs;
+  panel_tile<ES, OP>(ptrs.src[item], ptrs.dst[item], common, (uint64_t)(blockIdx.x - item * uniform_tiles), nan_bits, lds, cs);
+}
+
 }  // namespace
 
 namespace {
@@ -425,6 +587,21 @@ struct LaunchOne {
   mutable hipError_t err = hipSuccess;
   template <int ES, int OP>
   void operator()() const {
+    if (d.panel_rows_log2) {
+      if constexpr (ES <= 4) {
+        if (!panel_desc_ok(d, ES, out_elem(ES, OP)) || block.x * (uint32_t)kPanelLoads != (1u << (d.panel_rows_log2 + d.panel_chunks_log2))) {
+          err = hipErrorInvalidValue;
+          return;
+        }
+        const uint32_t lds = 16u << (d.panel_rows_log2 + d.panel_chunks_log2);
+        err = allow_lds<panel_kernel<ES, OP>>(lds);
+        if (err != hipSuccess) return;
+        hipLaunchKernelGGL((panel_kernel<ES, OP>), grid, block, lds, stream, s, t, d, nan_bits, sum_out, fan);
+      } else {
+        err = hipErrorInvalidValue;
+      }
+      return;
+    }
     const uint32_t lds = (block.x / 64u) * Sub<ES, OP>::kLdsBytes;
     err = allow_lds<transpose_kernel<ES, OP>>(lds);
     if (err != hipSuccess) return;
@@ -437,9 +614,41 @@ struct LaunchBatch {
   hipStream_t stream;
   const TransposeItem* items;
   uint32_t n_items, nan_bits;
+  uint32_t panel;  // 0, or panel_rows_log2 << 8 | panel_chunks_log2 of every item
+  uint32_t uniform_tiles;  // != 0: every item has this many tiles and the descriptor `common`
+  const TransposeDesc* common;
+  const TransposeItem* items_host;  // may be null
   mutable hipError_t err = hipSuccess;
   template <int ES, int OP>
   void operator()() const {
+    if (panel) {
+      if constexpr (ES <= 4) {
+        const uint32_t bits = (panel >> 8) + (panel & 0xFFu);
+        if (bits < 9 || (16ull << bits) > kPanelMaxBytes || block.x * (uint32_t)kPanelLoads != (1u << bits)) {
+          err = hipErrorInvalidValue;
+          return;
+        }
+        const uint32_t lds = 16u << bits;
+        if (uniform_tiles && items_host && n_items <= (uint32_t)kPanelArgItems) {
+          PanelPtrTable ptrs{};
+          for (uint32_t k = 0; k < n_items; ++k) {
+            ptrs.src[k] = items_host[k].src;
+            ptrs.dst[k] = items_host[k].dst;
+          }
+          err = allow_lds<panel_batch_args_kernel<ES, OP>>(lds);
+          if (err != hipSuccess) return;
+          hipLaunchKernelGGL((panel_batch_args_kernel<ES, OP>), grid, block, lds, stream, ptrs, nan_bits, uniform_tiles, *common);
+          return;
+        }
+        err = allow_lds<panel_batch_kernel<ES, OP>>(lds);
+        if (err != hipSuccess) return;
+        hipLaunchKernelGGL((panel_batch_kernel<ES, OP>), grid, block, lds, stream, items, n_items, nan_bits, uniform_tiles,
+                           common ? *common : TransposeDesc{});
+      } else {
+        err = hipErrorInvalidValue;
+      }
+      return;
+    }
     const uint32_t lds = (block.x / 64u) * Sub<ES, OP>::kLdsBytes;
     err = allow_lds<transpose_batch_kernel<ES, OP>>(lds);
     if (err != hipSuccess) return;
@@ -461,10 +670,16 @@ hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, 
 }
 
 hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_items, uint64_t total_tiles, uint32_t waves,
-                                  int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream) {
+                                  int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream, uint32_t panel,
+                                  uint32_t uniform_tiles, const TransposeDesc* common, const TransposeItem* items_host) {
   if (n_items == 0 || total_tiles == 0) return hipSuccess;
-  if (total_tiles > 0x7FFFFFFFull || waves == 0 || waves > (uint32_t)kWaves || (waves & (waves - 1))) return hipErrorInvalidValue;
-  const LaunchBatch many{dim3((uint32_t)total_tiles), dim3(waves * 64u), stream, items_dev, n_items, nan_bits};
+  if (total_tiles > 0x7FFFFFFFull || waves == 0 || waves > (panel ? 16u : (uint32_t)kWaves) || (waves & (waves - 1)))
+    return hipErrorInvalidValue;
+  if (uniform_tiles && ((uint64_t)uniform_tiles * n_items != total_tiles || !common || common->n_tiles != uniform_tiles ||
+                        !panel || panel != (common->panel_rows_log2 << 8 | common->panel_chunks_log2)))
+    return hipErrorInvalidValue;
+  const LaunchBatch many{dim3((uint32_t)total_tiles), dim3(waves * 64u), stream, items_dev, n_items, nan_bits, panel, uniform_tiles,
+                         common, items_host};
   if (!with_instance(elem_size, op, many)) return hipErrorInvalidValue;
   if (many.err != hipSuccess) return many.err;
   return hipGetLastError();

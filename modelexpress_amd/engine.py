@@ -496,6 +496,14 @@ class PlacementEngine:
                     getattr(o, key)[d] = int(x)
         return arr
 
+    def describe_views(self, views: Sequence[dict]) -> list:
+        """How ``copy_views`` would run each view (nothing is launched): ``("boxes" | "transpose" | "staged_tile",
+        tile rows, tile row bytes)`` per view."""
+        n = len(views)
+        kinds, rows, row_bytes = ((C.c_int32 * max(1, n))() for _ in range(3))
+        L.check(L.lib().mxp_describe_views(self._h, self.views_array(views), n, kinds, rows, row_bytes))
+        return [(("boxes", "transpose", "staged_tile")[kinds[k]], rows[k], row_bytes[k]) for k in range(n)]
+
     def copy_views_array(self, arr, n: int, *, stream: int = 0) -> None:
         """``copy_views`` on an ``_lib.ViewCopy`` array the caller built (and may keep between calls)."""
         L.check(L.lib().mxp_copy_views(self._h, arr, n, C.c_void_p(stream)))
@@ -531,6 +539,11 @@ class PlacementEngine:
         out = C.c_double()
         L.check(L.lib().mxp_measure_h2d(self._h, nbytes, repeats, C.byref(out)))
         return float(out.value)
+
+
+def set_transpose_form(form: int) -> None:
+    """Measurement switch: 1 = every transposed view runs in the wavefront-autonomous form, 0 = the library picks."""
+    L.check(L.lib().mxp_set_transpose_form(int(form)))
 
 
 def measure_read(paths: Sequence[str], *, threads: int = 16, request_bytes: int = 16 << 20, direct: bool = True) -> dict:

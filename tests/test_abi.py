@@ -19,8 +19,8 @@ def _declared(header="mxp.h"):
     return sorted(set(re.findall(r"\b(mxp_[a-z0-9_]+)\s*\(", text)))
 
 
-BENCH_ONLY = ["mxp_engine_launch_times", "mxp_engine_set_launch_timing", "mxp_measure_gather", "mxp_measure_h2d",
-              "mxp_measure_read", "mxp_synth_device", "mxp_synth_host"]
+BENCH_ONLY = ["mxp_describe_views", "mxp_engine_launch_times", "mxp_engine_set_launch_timing", "mxp_measure_gather", "mxp_measure_h2d",
+              "mxp_measure_read", "mxp_set_transpose_form", "mxp_synth_device", "mxp_synth_host"]
 
 
 def test_library_exports_every_declared_symbol(mxp):

@@ -457,6 +457,80 @@ def test_converting_transposes_match_oracle(gpu_engine, oracle, oracle_c, src_dt
         assert int(csum, 16) == ref, (src_dtype, dst_dtype, nb, r, c)
 
 
+_PANEL_PAIRS = [("U8", "U8"), ("BF16", "BF16"), ("F32", "F32"), ("F32", "BF16"), ("BF16", "F32"), ("F16", "F32"), ("F32", "F16"),
+                ("F8_E4M3", "BF16"), ("F16", "BF16"), ("BF16", "F16")]
+_WORD = {"U8": np.uint8, "F32": np.uint32, "BF16": np.uint16, "F16": np.uint16, "F8_E4M3": np.uint8}
+
+
+def _panel_cases(se, de):
+    """(batch dims, rows r = destination innermost, columns c, source row pitch, destination row pitch) in elements,
+    chosen so that the transposes take the staged-tile ("panel") form: whole tiles, 16-byte aligned, and either short
+    abutting destination rows or long pitches on both sides."""
+    cases = [((3,), 128, 1024 // se, 1024 // se, 128),         # destination rows abut: one tile = one contiguous block
+             ((2, 3), 16, 2048 // se, 2048 // se + 16 // se, 16),   # very short rows, two batch dimensions, padded source pitch
+             ((1,), 1024 // de, 512, 512, 1024 // de),         # the longest rows of that branch (1 KiB)
+             ((600,), 32, 256 // se, 256 // se, 32)]           # many small tiles: enough for full-size workgroups
+    if se == 2 and de == 2:
+        cases.append(((1,), 1024, 512, 16384, 16384))          # 32 KiB pitches on both sides
+    if se == 2 and de == 4:
+        cases.append(((2,), 512, 512, 8192, 8192))             # widening: 16 KiB source pitch, 32 KiB destination pitch
+    return cases
+
+
+@pytest.mark.parametrize("src_dtype,dst_dtype", _PANEL_PAIRS)
+def test_staged_tile_transposes_match_oracle(gpu_engine, oracle, oracle_c, src_dtype, dst_dtype):
+    """The transposes that run as whole staged tiles (a workgroup's read burst, a barrier, a write burst; no edge
+    handling in the kernel): every element type and conversion, single launches with their checksum and batched
+    launches (mxp_copy_views), against convert-then-transpose on the host."""
+    rng = np.random.default_rng(78)
+    code = 0 if src_dtype == dst_dtype else oracle.CAST_CODES[(src_dtype, dst_dtype)]
+    sw, dw = _WORD[src_dtype], _WORD[dst_dtype]
+    se, de = np.dtype(sw).itemsize, np.dtype(dw).itemsize
+    fill = {1: 0xEE, 2: 0xEEEE, 4: 0xEEEEEEEE}[de]
+    batch_views, batch_wants = [], []
+    for (bdims, r, c, sp, dp) in _panel_cases(se, de):
+        nb = int(np.prod(bdims))
+        raw = rng.integers(0, 1 << (8 * se), nb * r * sp, dtype=np.uint64).astype(sw)
+        k = min(raw.size, 1 << 16)
+        raw[:k] = np.arange(k, dtype=np.uint64).astype(sw) if se < 4 else (np.arange(k, dtype=np.uint32) << 16) | 0x8000
+        src = raw.reshape(nb, r, sp)[:, :, :c]
+        conv = src if code == 0 else oracle_c.cast(code, np.ascontiguousarray(src).reshape(-1)).reshape(nb, r, c)
+        want = np.full(nb * c * dp, fill, dtype=dw)
+        want.reshape(nb, c, dp)[:, :, :r] = conv.transpose(0, 2, 1)
+        d = torch.from_numpy(np.full(want.size * de, 0xEE, dtype=np.uint8)).cuda()
+        dev = _dev(raw.view(np.uint8))
+        # batch dimensions outermost, then (c, r): dst[b..., c, r] = convert(src[b..., r, c])
+        shape = tuple(bdims) + (c, r)
+        b_src = [int(np.prod(bdims[i + 1:])) * r * sp for i in range(len(bdims))]
+        b_dst = [int(np.prod(bdims[i + 1:])) * c * dp for i in range(len(bdims))]
+        view = dict(src=dev, dst=d, shape=shape, elem_size=de, src_strides=tuple(b_src) + (1, sp), dst_strides=tuple(b_dst) + (dp, 1), cast=code)
+        kind, tile_rows, tile_row_bytes = gpu_engine.describe_views([view])[0]
+        assert kind == "staged_tile" and r % tile_rows == 0 and (c * se) % tile_row_bytes == 0, (kind, tile_rows, tile_row_bytes, bdims, r, c)
+        csum = gpu_engine.copy_view(dev, d, shape, de, src_strides=view["src_strides"], dst_strides=view["dst_strides"], cast=code)
+        got = d.cpu().numpy().view(dw)
+        assert np.array_equal(got, want), (src_dtype, dst_dtype, bdims, r, c, sp, dp)
+        mask = np.zeros(nb * c * dp, dtype=bool)
+        mask.reshape(nb, c, dp)[:, :, :r] = True
+        pos = np.flatnonzero(np.repeat(mask, de))
+        b = want.view(np.uint8)[pos].astype(np.uint64)
+        ref = int((b * ((pos.astype(np.uint64) * np.uint64(2654435761) + np.uint64(1)) & np.uint64(0xFFFFFFFF))).sum() & np.uint64(0xFFFFFFFF))
+        assert int(csum, 16) == ref, (src_dtype, dst_dtype, bdims, r, c)
+        d2 = torch.from_numpy(np.full(want.size * de, 0xEE, dtype=np.uint8)).cuda()
+        batch_views.append(dict(view, dst=d2))
+        batch_wants.append((d2, want))
+    # the same views again as one call: transposes that share a tile shape go out as one launch - with one descriptor
+    # for all when they are alike (the first view twice), each with its own otherwise (its first two batches alone)
+    first, (_d, want0) = batch_views[0], batch_wants[0]
+    part = torch.from_numpy(np.full(want0.size * de, 0xEE, dtype=np.uint8)).cuda()
+    shorter = dict(first, dst=part, shape=(2,) + tuple(first["shape"][1:]))
+    gpu_engine.copy_views(batch_views + [dict(first), shorter])
+    for d2, want in batch_wants:
+        assert np.array_equal(d2.cpu().numpy().view(want.dtype), want), (src_dtype, dst_dtype, want.size)
+    per_batch = want0.size // 3
+    got = part.cpu().numpy().view(dw)
+    assert np.array_equal(got[: 2 * per_batch], want0[: 2 * per_batch]) and np.all(got[2 * per_batch:] == fill)
+
+
 def _random_layout(rng, shape):
     """Strides (in elements) of a view of `shape` inside a padded buffer whose dimensions are stored in a random order."""
     order = list(rng.permutation(len(shape)))  # storage order, outermost first
