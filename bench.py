@@ -873,6 +873,9 @@ def main() -> int:
                     paths = [f["path"] for f in ck_c.files()]
                     # the denominator: the same files read whole by the same number of threads with the same request
                     # size and O_DIRECT, no GPU work - before and after each ingest leg (a shared virtual disk drifts)
+                    # (the first pass over freshly written files is served faster than any later one on these virtual disks -
+                    # 7.6 against 5-6.5 GB/s - so one pass is spent before the comparison starts)
+                    first_pass = measure_read(paths, threads=readers, request_bytes=args.slot_mib << 20, direct=True)
                     probes = [measure_read(paths, threads=readers, request_bytes=args.slot_mib << 20, direct=True)]
                     legs = {}
                     for label, pack in (("packed_rows", True), ("row_bands", False)):
@@ -902,7 +905,8 @@ def main() -> int:
                         "storage_peak_is": f"plain O_DIRECT read of the same {len(paths)} shard files ({probes[0]['bytes'] / 1e9:.2f} GB), {readers} threads, "
                                            f"{args.slot_mib} MiB requests, no GPU work; one pass before the first leg and one after each leg ("
                                            + " / ".join(f"{p['bytes_per_second'] / 1e9:.2f}" for p in probes) + " GB/s); a leg's fraction is "
-                                           "against the better of the two passes around it",
+                                           "against the better of the two passes around it; the very first pass over the freshly written files "
+                                           f"({first_pass['bytes_per_second'] / 1e9:.2f} GB/s) is not used",
                         "strided_slices_under_direct_io": "packed_rows is the default: the readers fetch a band's rows with large requests into "
                                                           "their own buffers and copy only the rows into the ring (a third of the bytes cross "
                                                           "PCIe); row_bands stages whole bands and gathers on the device - each reader then "

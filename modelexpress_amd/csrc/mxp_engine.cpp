@@ -384,7 +384,14 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
       // strided source, packed by the readers: only the needed bytes cross PCIe and the
       // slot holds the rows back to back, so the device sees a plain copy
       if (row_src > slot) throw Error(MXP_ERR_UNSUPPORTED, "a source row of '" + t.name + "' does not fit a staging slot");
-      const uint64_t max_rows = slot / std::max<uint64_t>(row_src, kPackedRowCost);
+      uint64_t max_rows = slot / std::max<uint64_t>(row_src, kPackedRowCost);
+      // Direct I/O reads the file span the rows lie in: a piece is what one request covers, so that a chunk costs
+      // its reader one request like any other (a piece of 4096 rows of a 28 KiB pitch would be seven requests in
+      // a row for one reader while the others run out of work).
+      if (L->direct_io) {
+        const uint64_t per = direct_rows_per_read(eng.opt.slot_bytes, w.src_pitch, row_src);
+        if (per > 1) max_rows = std::min(max_rows, per);  // per == 1: rows far apart, read one by one
+      }
       for (uint64_t r = 0; r < w.rows; r += max_rows) {
         const uint64_t nr = std::min(max_rows, w.rows - r);
         Piece p{t.file_index, t0 + r * w.src_pitch, row_src, b, nr, w.src_pitch};
@@ -495,7 +502,9 @@ void lower_plan(mxp_plan& pl, const mxp_engine& eng) {
           p.nbytes = a1 - a0;
         }
         const uint64_t in_slot = p.nbytes * p.rows;
-        const uint64_t piece_cost = p.rows > 1 ? p.rows * std::max<uint64_t>(p.nbytes, kPackedRowCost) : in_slot;
+        const uint64_t piece_cost = p.rows > 1 ? (L->direct_io ? direct_rows_file_bytes(eng.opt.slot_bytes, p.file_off, p.rows, p.file_pitch, p.nbytes)
+                                                              : p.rows * std::max<uint64_t>(p.nbytes, kPackedRowCost))
+                                               : in_slot;
         if (!cur.ranges.empty() && (at + in_slot > cap || cur_cost + piece_cost > cap)) {
           close();
           at = 0;
