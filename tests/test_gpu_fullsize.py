@@ -232,42 +232,47 @@ def _room_for(n_bytes: int):
     return None
 
 
-def _whole_checkpoint_against_cpu_oracle(config: int, rank: int, n_files_expected: int, placed_expected: int, oracle, oracle_c):
-    """Writes one benchmark configuration's checkpoint files at full size, places the whole rank share on the CPU with
-    the oracle (numpy planner + C executor over the same files) and on the GPU twice - ingested from the files and
-    from the staged copy - and compares EVERY parameter buffer byte for byte, every checksum with the oracle's
-    safe_checksum and every digest with the oracle's tensor_digest (engines/vllm/refit/installer.py:419-424,
-    tensor_utils.py:27-44, refit/reshard/verify.py:79-155)."""
+def _whole_checkpoint_against_cpu_oracle(layout, tp, ep, rank, n_shards, n_files_expected, placed_expected, oracle, oracle_c, *,
+                                         ck_kw=None, cast=False, resident_from_generator=False):
+    """Writes a checkpoint's files at full size, places the whole rank share on the CPU with the oracle (numpy planner + C
+    executor over the same files) and on the GPU twice - ingested from the files and from the staged copy - and compares
+    EVERY parameter buffer byte for byte, every checksum with the oracle's safe_checksum and every digest with the
+    oracle's tensor_digest (engines/vllm/refit/installer.py:419-424, tensor_utils.py:27-44, refit/reshard/verify.py:79-155).
+    ``resident_from_generator``: the staged copy comes from the device-side generator (the same bytes as the files)
+    instead of reading the files back, for checkpoints too large to read twice."""
     import shutil
 
     from oracle import cpu_path
 
-    layout, tp, ep, n_shards, ck_dtype, ck_kind = models.baseline_config(config)
-    kw = {"dtype": ck_dtype, "edge_cases": ck_kind} if ck_dtype and config in (2, 3) else {}
-    tensors = layout.checkpoint(**kw)
+    tensors = layout.checkpoint(**(ck_kw or {}))
     total = sum(t.nbytes for t in tensors)
     workdir = _room_for(total)
     if workdir is None:
-        pytest.skip(f"no file system with room for the {total / 1e9:.1f} GB checkpoint of configuration {config}")
+        pytest.skip(f"no file system with room for the {total / 1e9:.1f} GB checkpoint")
     try:
         synth.write_checkpoint(tensors, workdir, n_shards=n_shards, seed=SEED, threads=16)
         ck = Checkpoint(workdir)
         assert len(ck.files()) == n_files_expected and sum(t.nbytes for t in ck.tensors()) == total
-        rv = layout.rank_view(tp_size=tp, tp_rank=rank, ep_size=ep, ep_rank=rank % ep)
+        rv = layout.rank_view(tp_size=tp, tp_rank=rank, ep_size=ep, ep_rank=rank % ep, param_dtype="BF16" if cast else None)
         plan = PlacementPlan(ck, rv.params, tp_size=tp, tp_rank=rank, stacked_params_mapping=rv.stacked_params_mapping,
-                             expert_mapping=rv.expert_mapping)
+                             expert_mapping=rv.expert_mapping, allow_cast=cast)
         assert plan.totals()["placed_bytes"] == placed_expected
+        local_of = {int(r[2]): int(r[4]) for r in (rv.expert_mapping or [])}
+        nan_bits = 0x7FC0
         cpu = cpu_path.run(workdir, [(p.name, p.dtype, p.shape) for p in rv.params], tp_size=tp, tp_rank=rank,
-                           stacked=rv.stacked_params_mapping, threads=16)
+                           stacked=rv.stacked_params_mapping,
+                           expert_mapping=[r[:4] for r in rv.expert_mapping] if rv.expert_mapping else None,
+                           expert_local=(lambda _f, g: local_of.get(g, g)) if rv.expert_mapping else None,
+                           allow_cast=cast, nan_bits=nan_bits, threads=16)
         assert cpu["placed_bytes"] == placed_expected
         want = {n: np.frombuffer(t.tobytes(), dtype=np.uint8) for n, t in cpu["params"].items()}
         want_sums = [cpu["checksums"][p.name] for p in plan.params]
         # the C executor's checksums are the oracle's own, checked against the numpy statement on the smaller buffers
-        for p in plan.params:
-            if p.nbytes <= (8 << 20):
-                assert cpu["checksums"][p.name] == oracle.safe_checksum_bytes(want[p.name]), p.name
+        small = [p for p in plan.params if p.nbytes <= (8 << 20)]
+        for p in small[:: max(1, len(small) // 200)]:
+            assert cpu["checksums"][p.name] == oracle.safe_checksum_bytes(want[p.name]), p.name
         want_digests = [oracle.tensor_digest_bytes(want[p.name]) for p in plan.params]
-        eng = PlacementEngine(0)
+        eng = PlacementEngine(0, nan_bits=nan_bits)
         eng.set_fused_digests(True)
         for mode in ("ingest", "resident"):
             dst = eng.allocate(plan, fill=0xE7)
@@ -275,13 +280,19 @@ def _whole_checkpoint_against_cpu_oracle(config: int, rank: int, n_files_expecte
                 stats = eng.execute(plan, dst)
                 assert stats["placed_bytes"] == placed_expected
             else:
-                staged = [torch.from_numpy(np.fromfile(f["path"], dtype=np.uint8)).cuda() for f in ck.files()]
+                if resident_from_generator:
+                    staged = synth.stage_on_device(ck, tensors, seed=SEED)
+                else:
+                    staged = [torch.from_numpy(np.fromfile(f["path"], dtype=np.uint8)).cuda() for f in ck.files()]
                 eng.execute_resident(plan, staged, dst)
                 del staged
             sums, digests = eng.checksums(plan), eng.digests(plan)
             assert sums == want_sums, (mode, [p.name for p, a, b in zip(plan.params, sums, want_sums) if a != b][:5])
             assert digests == want_digests, (mode, [p.name for p, a, b in zip(plan.params, digests, want_digests) if a != b][:5])
-            assert eng.digest(dst) == want_digests  # the stand-alone pass over the finished buffers
+            alone = []
+            for i in range(0, len(dst), 1024):
+                alone += eng.digest(dst[i:i + 1024])
+            assert alone == want_digests  # the stand-alone pass over the finished buffers
             for p, d in zip(plan.params, dst):
                 assert np.array_equal(d.view(torch.uint8).reshape(-1).cpu().numpy(), want[p.name]), (mode, p.name)
             del dst
@@ -294,12 +305,39 @@ def _whole_checkpoint_against_cpu_oracle(config: int, rank: int, n_files_expecte
 
 def test_gpt2_small_whole_checkpoint_at_real_shapes(oracle, oracle_c, mxp):
     """Configuration 1 at its real shapes: one file, 148 fp16 tensors, 248,879,616 bytes, TP=1 - all buffers."""
-    _whole_checkpoint_against_cpu_oracle(1, 0, 1, 248_879_616, oracle, oracle_c)
+    layout, tp, ep, n_shards, _dt, _kind = models.baseline_config(1)
+    _whole_checkpoint_against_cpu_oracle(layout, tp, ep, 0, n_shards, 1, 248_879_616, oracle, oracle_c)
 
 
 def test_llama3_8b_whole_rank_share_against_the_cpu_oracle(oracle, oracle_c, mxp):
     """Configuration 2: the 16 GB checkpoint in 4 shard files, rank 5 of 8 - all 195 buffers byte for byte."""
-    _whole_checkpoint_against_cpu_oracle(2, RANK, 4, 2_008_031_232, oracle, oracle_c)
+    layout, tp, ep, n_shards, _dt, _kind = models.baseline_config(2)
+    _whole_checkpoint_against_cpu_oracle(layout, tp, ep, RANK, n_shards, 4, 2_008_031_232, oracle, oracle_c)
+
+
+def test_llama3_8b_refit_whole_rank_share_against_the_cpu_oracle(oracle, oracle_c, mxp):
+    """Configuration 3: the 32 GB fp32 checkpoint (denormals, infinities and NaNs at 1e-6 density each) refitted into the
+    bf16 rank share - all 195 buffers byte for byte, ingested (PCIe carries fp32, cast in flight) and resident."""
+    layout, tp, ep, n_shards, dt, kind = models.baseline_config(3)
+    _whole_checkpoint_against_cpu_oracle(layout, tp, ep, RANK, n_shards, 8, 2_008_031_232, oracle, oracle_c,
+                                         ck_kw={"dtype": dt, "edge_cases": kind}, cast=True, resident_from_generator=True)
+
+
+def test_mixtral_two_layers_whole_against_the_cpu_oracle(oracle, oracle_c, mxp):
+    """Configuration 4's family at real shapes, two layers: every expert of both layers stacked into w13 [8, 28672, 4096]
+    / w2 [8, 4096, 14336], QKV fused - every buffer byte for byte."""
+    layout = models.Mixtral(layers=2)
+    placed = sum(p.nbytes for p in layout.rank_view().params)
+    _whole_checkpoint_against_cpu_oracle(layout, 1, 1, 0, 2, 2, placed, oracle, oracle_c)
+
+
+def test_deepseek_v3_four_layers_whole_rank_share_against_the_cpu_oracle(oracle, oracle_c, mxp):
+    """Configuration 5's family at real shapes (three dense layers and one MoE layer of 256 routed experts, TP=8 / EP=8):
+    fp8 weights with their fp32 128x128 scale tiles, the rank's 32 local experts stacked - every buffer of the rank."""
+    layout = models.DeepSeekV3(layers=4, dense_layers=3)
+    rv = layout.rank_view(tp_size=8, tp_rank=5, ep_size=8, ep_rank=5)
+    placed = sum(p.nbytes for p in rv.params)
+    _whole_checkpoint_against_cpu_oracle(layout, 8, 8, 5, 6, 6, placed, oracle, oracle_c, resident_from_generator=True)
 
 
 def test_buffer_beyond_4_gib_wraps_positions_like_the_reference(oracle_c, gpu_engine):
