@@ -315,12 +315,14 @@ def _ingest_leg(plan, dst, resident_sums, h2d_peak: float, source: str, *, pack:
     # At least `runs` ingests, and for a small checkpoint as many as fit into 0.6 s (at most 60): for a few hundred
     # milliseconds after a large free of device memory every ingest runs slower, and a 5 ms ingest would be measured
     # entirely inside that window.
-    best, i, t_begin = None, 0, time.perf_counter()
+    best, i, t_begin, walls = None, 0, time.perf_counter(), []
     while i < runs or (i < 60 and time.perf_counter() - t_begin < 0.6):
         st = e2.execute(plan, dst)
+        walls.append(round(st["wall_seconds"] * 1e3, 2))
         if i and (best is None or st["wall_seconds"] < best["wall_seconds"]):
             best = st
         i += 1
+    _log(f"ingest runs (ms): {walls}")
     sums = e2.checksums(plan)
     e2.close()
     w = best["wall_seconds"]

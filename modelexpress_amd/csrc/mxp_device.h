@@ -243,12 +243,12 @@ hipError_t launch_transpose(const void* src, void* dst, const TransposeDesc& d, 
 // `panel`: 0, or (panel_rows_log2 << 8 | panel_chunks_log2) shared by every item; `uniform_tiles`: 0, or - for
 // a panel batch whose items all have the descriptor `*common` - the number of tiles of each
 // (total_tiles == n_items * uniform_tiles); the kernel then takes the descriptor as an argument, and with
-// `items_host` (the same items, on the host) and at most kPanelArgItems of them their pointers as well.
+// `items_host` (the same items, on the host) their pointers as well, kPanelArgItems items to a launch.
 hipError_t launch_transpose_batch(const TransposeItem* items_dev, uint32_t n_items, uint64_t total_tiles, uint32_t waves,
                                   int elem_size, uint32_t op, uint32_t nan_bits, hipStream_t stream, uint32_t panel = 0,
                                   uint32_t uniform_tiles = 0, const TransposeDesc* common = nullptr,
                                   const TransposeItem* items_host = nullptr);
-// Items of a uniform panel batch whose pointers fit the kernel argument block (`items_host` given).
+// Items of a uniform panel batch whose pointers fit the kernel argument block of one launch (`items_host` given).
 constexpr int kPanelArgItems = 96;
 // Field by field (the struct may hold padding).
 inline bool same_transpose_desc(const TransposeDesc& a, const TransposeDesc& b) {

@@ -512,7 +512,7 @@ __global__ __launch_bounds__(1024) void panel_batch_kernel(const TransposeItem* 
   panel_tile<ES, OP>(it.src, it.dst, it.d, (uint64_t)blockIdx.x - it.first_tile, nan_bits, lds, cs);
 }
 
-// The same for a uniform batch of at most kPanelArgItems items, whose pointers travel in the kernel argument
+// The same for kPanelArgItems items of a uniform batch at a time, whose pointers travel in the kernel argument
 // block as well: a workgroup's two pointers are then loaded together with the descriptor when the wavefront
 // starts, instead of after it (a table in memory is addressed through a pointer that is itself an argument).
 struct PanelPtrTable {
@@ -629,15 +629,20 @@ struct LaunchBatch {
           return;
         }
         const uint32_t lds = 16u << bits;
-        if (uniform_tiles && items_host && n_items <= (uint32_t)kPanelArgItems) {
-          PanelPtrTable ptrs{};
-          for (uint32_t k = 0; k < n_items; ++k) {
-            ptrs.src[k] = items_host[k].src;
-            ptrs.dst[k] = items_host[k].dst;
-          }
+        if (uniform_tiles && items_host) {
+          // kPanelArgItems items to a launch: a few microseconds between launches cost less than a pointer table in memory
           err = allow_lds<panel_batch_args_kernel<ES, OP>>(lds);
           if (err != hipSuccess) return;
-          hipLaunchKernelGGL((panel_batch_args_kernel<ES, OP>), grid, block, lds, stream, ptrs, nan_bits, uniform_tiles, *common);
+          for (uint32_t first = 0; first < n_items; first += (uint32_t)kPanelArgItems) {
+            const uint32_t n = n_items - first < (uint32_t)kPanelArgItems ? n_items - first : (uint32_t)kPanelArgItems;
+            PanelPtrTable ptrs{};
+            for (uint32_t k = 0; k < n; ++k) {
+              ptrs.src[k] = items_host[first + k].src;
+              ptrs.dst[k] = items_host[first + k].dst;
+            }
+            hipLaunchKernelGGL((panel_batch_args_kernel<ES, OP>), dim3(n * uniform_tiles), block, lds, stream, ptrs, nan_bits,
+                               uniform_tiles, *common);
+          }
           return;
         }
         err = allow_lds<panel_batch_kernel<ES, OP>>(lds);

@@ -531,6 +531,27 @@ def test_staged_tile_transposes_match_oracle(gpu_engine, oracle, oracle_c, src_d
     assert np.array_equal(got[: 2 * per_batch], want0[: 2 * per_batch]) and np.all(got[2 * per_batch:] == fill)
 
 
+def test_staged_tile_uniform_batch_longer_than_one_argument_block(gpu_engine):
+    """230 transposes of one shape in one mxp_copy_views call: their pointers travel as kernel arguments, 96 items to
+    a launch, so the call is three launches; every item must land in its own destination and nowhere else."""
+    rng = np.random.default_rng(79)
+    n_items, nb, r, c = 230, 4, 128, 256     # per item: [4, 128, 256] bf16 -> [4, 256, 128]
+    raw = rng.integers(0, 1 << 16, (n_items, nb, r, c), dtype=np.uint16)
+    src = _dev(raw.reshape(-1).view(np.uint8))
+    dst = torch.from_numpy(np.full(raw.size * 2 + 4096, 0xEE, dtype=np.uint8)).cuda()
+    per = nb * r * c * 2
+    order = rng.permutation(n_items)           # item k writes the order[k]-th slot of the destination
+    views = [dict(src=src[k * per:(k + 1) * per], dst=dst[int(order[k]) * per:(int(order[k]) + 1) * per], shape=(nb, c, r), elem_size=2,
+                  src_strides=(r * c, 1, c), dst_strides=(c * r, r, 1)) for k in range(n_items)]
+    kinds = gpu_engine.describe_views(views)
+    assert all(kind == "staged_tile" for kind, _r, _b in kinds), kinds[0]
+    gpu_engine.copy_views(views)
+    got = dst.cpu().numpy()
+    assert np.all(got[n_items * per:] == 0xEE)
+    got = got[: n_items * per].view(np.uint16).reshape(n_items, nb, c, r)
+    assert np.array_equal(got[order], raw.transpose(0, 1, 3, 2))
+
+
 def _random_layout(rng, shape):
     """Strides (in elements) of a view of `shape` inside a padded buffer whose dimensions are stored in a random order."""
     order = list(rng.permutation(len(shape)))  # storage order, outermost first
