@@ -7,7 +7,15 @@ inputs are the ones most likely to break host code: a session of the parser prop
 and structured headers), the reference's planner vectors, the random planner models, the Megatron layouts and
 the full-scale DeepSeek-V3 plan is run once with every host-side ABI call recorded (tests/abi_trace.py), and
 the trace is replayed through the sanitized build, which must return what the product build returned, report
-nothing and leak nothing."""
+nothing and leak nothing.
+
+The engine itself (csrc/mxp_engine.cpp: reader threads, pinned ring, slot events, stream ordering, error path) is
+the one concurrent piece of the library.  It is built for the CPU against a stand-in for the HIP runtime
+(tests/c/cpu_hip: streams are worker threads, events complete when their worker reaches them, "device" memory is
+host memory, the kernel launches are executed by meaning) and driven by tests/c/engine_hosttest.cpp through every
+ingest mode under ``-fsanitize=thread`` and again under ``-fsanitize=address,undefined``.  That the harness sees
+what it is there to see is checked too: with events that claim completion early the same run must end in a data
+race report."""
 
 import os
 import subprocess
@@ -77,3 +85,60 @@ def test_lowering_and_overlap_checkers_under_sanitizers():
     r = subprocess.run([str(overlap), "0", "4000"], capture_output=True, text=True, env=_env(), timeout=600)
     _clean(r)
     assert "4000 pairs clipped and replayed" in r.stdout
+
+
+HIP_ON_CPU = CDIR / "cpu_hip"
+ENGINE_SOURCES = [CDIR / "engine_hosttest.cpp", HIP_ON_CPU / "cpu_hip.cpp", HIP_ON_CPU / "cpu_kernels.cpp", CSRC / "mxp_engine.cpp",
+                  CSRC / "mxp_ckpt.cpp", CSRC / "mxp_plan.cpp", CSRC / "mxp_crc32c.cpp"]
+TSAN = ["-fsanitize=thread", "-fno-omit-frame-pointer", "-g", "-O1"]
+
+
+@pytest.fixture(scope="module")
+def engine_binaries():
+    """engine_hosttest built twice (ThreadSanitizer; AddressSanitizer + UndefinedBehaviorSanitizer), side by side."""
+    deps = [*CSRC.glob("*.hpp"), *CSRC.glob("*.h"), *(ROOT / "include").glob("*.h"), HIP_ON_CPU / "hip" / "hip_runtime.h", Path(__file__)]
+    newest = max(p.stat().st_mtime for p in [*ENGINE_SOURCES, *deps])
+    base = ["g++", "-std=c++17", "-Wall", f"-I{HIP_ON_CPU}", f"-I{ROOT / 'include'}", f"-I{CSRC}"]  # the stand-in's hip/hip_runtime.h, not ROCm's
+    outs = {"tsan": (CDIR / "engine_hosttest_tsan", TSAN), "asan": (CDIR / "engine_hosttest_asan", SAN)}
+    running = []
+    for out, flags in outs.values():
+        if not out.exists() or out.stat().st_mtime < newest:
+            running.append(subprocess.Popen([*base, *flags, *map(str, ENGINE_SOURCES), "-o", str(out), "-lpthread"],
+                                            stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True))
+    for proc in running:
+        _o, err = proc.communicate(timeout=900)
+        assert proc.returncode == 0, err[-4000:]
+    return {k: v[0] for k, v in outs.items()}
+
+
+def _tsan_env(**extra):
+    return dict(os.environ, TSAN_OPTIONS="halt_on_error=0:second_deadlock_stack=1", **extra)
+
+
+def _skip_if_tsan_cannot_map(r):
+    if "unexpected memory mapping" in r.stderr:  # the sanitizer's own start-up check against the kernel's address layout
+        pytest.skip("ThreadSanitizer cannot run on this kernel's address-space layout")
+
+
+def test_engine_ring_and_streams_under_thread_sanitizer(engine_binaries, tmp_path):
+    r = subprocess.run([str(engine_binaries["tsan"]), str(tmp_path)], capture_output=True, text=True, env=_tsan_env(), timeout=900)
+    _skip_if_tsan_cannot_map(r)
+    assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-6000:])
+    assert "ThreadSanitizer" not in r.stderr, r.stderr[-6000:]
+    assert r.stdout.startswith("ok: 63 placements checked"), r.stdout
+
+
+def test_engine_ring_and_streams_under_address_sanitizer(engine_binaries, tmp_path):
+    r = subprocess.run([str(engine_binaries["asan"]), str(tmp_path)], capture_output=True, text=True, env=_env(), timeout=900)
+    _clean(r)
+    assert r.stdout.startswith("ok: 63 placements checked"), r.stdout
+
+
+def test_thread_sanitizer_reports_a_ring_slot_reused_too_early(engine_binaries, tmp_path):
+    """The harness's own check: events that claim completion before their stream got there let the readers overwrite
+    slots whose copies are still queued; the run must not pass."""
+    r = subprocess.run([str(engine_binaries["tsan"]), str(tmp_path)], capture_output=True, text=True,
+                       env=_tsan_env(CPU_HIP_EVENTS_COMPLETE_EARLY="1"), timeout=900)
+    _skip_if_tsan_cannot_map(r)
+    assert r.returncode != 0
+    assert "ThreadSanitizer: data race" in r.stderr and "pread" in r.stderr, r.stderr[-3000:]
