@@ -331,7 +331,8 @@ def _ingest_leg(plan, dst, resident_sums, h2d_peak: float, source: str, *, pack:
             "wall_s": round(w, 4), "file_bytes": best["file_bytes"], "h2d_bytes": best["h2d_bytes"],
             "strided_slices": "rows packed into the pinned slot by the readers" if pack else
                               "whole row bands staged, gathered on the device",
-            "reader_threads": readers, "ring": f"{ring_slots} x {slot_mib} MiB pinned", "source": source,
+            "reader_threads": readers, "readers_busy_frac": round(best["read_seconds"] / (readers * w), 3),
+            "ring": f"{ring_slots} x {slot_mib} MiB pinned", "source": source,
             "checksums_match_resident": sums == resident_sums}
 
 
@@ -897,6 +898,7 @@ def main() -> int:
                                        "file_gbps": round(st["file_bytes"] / st["wall_seconds"] / 1e9, 3),
                                        "h2d_gbps": round(st["h2d_bytes"] / st["wall_seconds"] / 1e9, 3),
                                        "wall_s": round(st["wall_seconds"], 3), "file_bytes": st["file_bytes"],
+                                       "readers_busy_frac": round(st["read_seconds"] / (readers * st["wall_seconds"]), 3),
                                        "checksums_match_resident": cold_sums == resident_sums}
                         probes.append(measure_read(paths, threads=readers, request_bytes=args.slot_mib << 20, direct=True))
                         around = max(probes[-2]["bytes_per_second"], probes[-1]["bytes_per_second"]) / 1e9

@@ -254,7 +254,7 @@ typedef struct mxp_engine_options {
 
 typedef struct mxp_exec_stats {
   double wall_seconds;     /* entry to last stream idle */
-  double read_seconds;     /* summed over reader threads */
+  double read_seconds;     /* reading and packing, summed over reader threads (waiting for a slot not included) */
   double kernel_ms;        /* HIP-event time of placement kernels (resident mode) */
   uint64_t file_bytes;     /* read from storage */
   uint64_t h2d_bytes;      /* copied host -> device */

@@ -960,7 +960,8 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
           if (turn > 0) HIP_OK(hipEventSynchronize(sl.done));
           return true;
         };
-        const double t0 = now_s();
+        // read_s: time spent reading and packing, not waiting for a slot
+        double t0 = now_s();
         if (direct_buf) {
           // Direct I/O: the whole chunk is read into the reader's own block-aligned copy of the slot BEFORE
           // the slot is waited for, so the number of storage requests in flight is the number of readers,
@@ -984,10 +985,13 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
                             static_cast<uint8_t*>(direct_buf) + (o0 - a0) + k * r.file_pitch, r.nbytes);
             }
           }
+          read_s[tid] += now_s() - t0;
           if (!wait_for_slot()) break;
+          t0 = now_s();
           std::memcpy(sl.host, stage, ch.used_bytes);
         } else {
           if (!wait_for_slot()) break;
+          t0 = now_s();
           for (const auto& r : ch.ranges)
             for (uint64_t row = 0; row < r.rows; ++row)
               pread_full(fds[r.file], sl.host + r.slot_off + row * r.nbytes, r.nbytes, r.file_off + row * r.file_pitch,
