@@ -8,13 +8,16 @@
 // more readers than slots, one stream, a delay in front of every copy - several times each on one engine; the
 // bytes that arrive and their checksums are compared with what the driver computes from the tensors itself.
 // Then: a caller stream with work pending on the destinations, the resident path, the stand-alone checksum,
-// a shard file truncated between plan and execute (the ingest must fail cleanly and work again afterwards).
+// a shard file truncated between plan and execute (the ingest must fail cleanly and work again afterwards); last,
+// 96 random strided views (storage orders, paddings, element sizes, two conversions) as single recorded copies,
+// as batched calls back to back on two streams and as view plans run repeatedly, and the small stand-alone operators.
 //
 // usage: engine_hosttest <empty working directory>      prints "ok" and exits 0 on success
 #include <hip/hip_runtime.h>
 #include <sys/stat.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <chrono>
 #include <cinttypes>
 #include <cstdio>
@@ -27,6 +30,7 @@
 #include <vector>
 
 #include "mxp.h"
+#include "mxp_bench.h"
 
 namespace {
 
@@ -252,6 +256,225 @@ mxp_engine* make_engine(int slots, uint64_t slot_bytes, int readers, int streams
   return e;
 }
 
+// ---- recorded copies between strided views (mxp_copy_view, mxp_copy_views, mxp_view_plan_*) ----
+struct View {
+  std::vector<int64_t> shape, ss, ds;  // strides in elements
+  int es = 1, eo = 1, cast = MXP_CAST_NONE;
+  std::vector<uint8_t> src, want;       // host images of the whole source / destination buffers
+  uint8_t* dsrc = nullptr;              // "device" copies
+  uint8_t* ddst = nullptr;
+  size_t src_off = 0;                   // elements the view starts into its source buffer
+  uint32_t csum = 0;                    // checksum of the written bytes, positions counted from ddst
+};
+
+// Strides of a view of `shape` inside a buffer whose dimensions are stored in a random order, sometimes padded.
+int64_t random_layout(std::mt19937& rng, const std::vector<int64_t>& shape, std::vector<int64_t>& strides) {
+  std::vector<size_t> order(shape.size());
+  for (size_t i = 0; i < order.size(); ++i) order[i] = i;
+  std::shuffle(order.begin(), order.end(), rng);
+  strides.assign(shape.size(), 0);
+  int64_t run = 1;
+  for (size_t k = order.size(); k-- > 0;) {
+    strides[order[k]] = run;
+    run *= shape[order[k]] + (rng() % 3 == 0 ? (int64_t)(rng() % 3) : 0);
+  }
+  return run;
+}
+
+View make_view(std::mt19937& rng, int index) {
+  View v;
+  const int pick = index % 6;
+  if (pick == 4) { v.es = 4; v.eo = 2; v.cast = MXP_CAST_F32_BF16; }
+  else if (pick == 5) { v.es = 2; v.eo = 4; v.cast = MXP_CAST_BF16_F32; }
+  else v.es = v.eo = 1 << (pick % 4);
+  const int ndim = 1 + (int)(rng() % 4);
+  int64_t elems = 1;
+  static const int64_t sizes[] = {1, 2, 3, 5, 8, 16, 31, 64, 70, 128, 256};
+  do {
+    v.shape.clear();
+    for (int d = 0; d < ndim; ++d) v.shape.push_back(sizes[rng() % (ndim > 2 ? 8 : 11)]);
+    if (index % 5 == 0 && ndim >= 2) {  // whole tiles, so that the staged-tile transposes are met as well
+      v.shape[ndim - 1] = 128;
+      v.shape[ndim - 2] = 256;
+      for (int d = 0; d < ndim - 2; ++d) v.shape[d] = 1 + (int64_t)(rng() % 2);
+    }
+    elems = 1;
+    for (int64_t e : v.shape) elems *= e;
+  } while (elems > 140000);  // the whole run stays within seconds under ThreadSanitizer
+  int64_t s_total, d_total;
+  if (index % 5 == 0 && ndim >= 2) {
+    // the shape of the MLA W_UK_T rewrite: destination row-major, source with its last two dimensions swapped
+    v.ds.assign((size_t)ndim, 1);
+    for (int d = ndim - 2; d >= 0; --d) v.ds[(size_t)d] = v.ds[(size_t)d + 1] * v.shape[(size_t)d + 1];
+    v.ss = v.ds;
+    v.ss[(size_t)ndim - 1] = v.shape[(size_t)ndim - 2];
+    v.ss[(size_t)ndim - 2] = 1;
+    s_total = d_total = v.ds[0] * v.shape[0];
+  } else {
+    s_total = random_layout(rng, v.shape, v.ss);
+    d_total = random_layout(rng, v.shape, v.ds);
+  }
+  v.src_off = rng() % 4;
+  v.src.resize((size_t)(s_total + (int64_t)v.src_off) * v.es);
+  for (auto& b : v.src) b = (uint8_t)rng();
+  if (v.cast == MXP_CAST_F32_BF16)
+    for (size_t i = 3; i < v.src.size(); i += 4) v.src[i] &= 0x3F;  // no NaN
+  v.want.assign((size_t)d_total * v.eo, 0xEE);
+  std::vector<int64_t> idx(v.shape.size(), 0);
+  int64_t n = 1;
+  for (int64_t e : v.shape) n *= e;
+  for (int64_t k = 0; k < n; ++k) {
+    int64_t so = (int64_t)v.src_off, d_o = 0;
+    for (size_t d = 0; d < idx.size(); ++d) { so += idx[d] * v.ss[d]; d_o += idx[d] * v.ds[d]; }
+    const uint8_t* sp = v.src.data() + so * v.es;
+    uint8_t* dp = v.want.data() + d_o * v.eo;
+    if (v.cast == MXP_CAST_F32_BF16) {
+      uint32_t u;
+      std::memcpy(&u, sp, 4);
+      const uint16_t h = f32_to_bf16(u);
+      std::memcpy(dp, &h, 2);
+    } else if (v.cast == MXP_CAST_BF16_F32) {
+      uint16_t h;
+      std::memcpy(&h, sp, 2);
+      const uint32_t u = (uint32_t)h << 16;
+      std::memcpy(dp, &u, 4);
+    } else {
+      std::memcpy(dp, sp, (size_t)v.es);
+    }
+    for (int e = 0; e < v.eo; ++e) v.csum += dp[e] * ((uint32_t)(d_o * v.eo + e) * 2654435761u + 1u);
+    for (size_t d = idx.size(); d-- > 0;) {
+      if (++idx[d] < v.shape[d]) break;
+      idx[d] = 0;
+    }
+  }
+  if (hipMalloc(reinterpret_cast<void**>(&v.dsrc), v.src.size()) != hipSuccess || hipMalloc(reinterpret_cast<void**>(&v.ddst), v.want.size()) != hipSuccess)
+    die("hipMalloc");
+  std::memcpy(v.dsrc, v.src.data(), v.src.size());
+  return v;
+}
+
+mxp_view_copy as_abi(const View& v) {
+  mxp_view_copy c{};
+  c.src = v.dsrc + v.src_off * (size_t)v.es;
+  c.dst = v.ddst;
+  c.ndim = (int32_t)v.shape.size();
+  c.elem_size = v.eo;
+  c.cast = v.cast;
+  for (size_t d = 0; d < v.shape.size(); ++d) { c.shape[d] = v.shape[d]; c.src_strides[d] = v.ss[d]; c.dst_strides[d] = v.ds[d]; }
+  return c;
+}
+
+void check_views(std::vector<View>& views, const std::string& what) {
+  if (hipDeviceSynchronize() != hipSuccess) die("sync");
+  for (size_t k = 0; k < views.size(); ++k)
+    if (std::memcmp(views[k].ddst, views[k].want.data(), views[k].want.size()) != 0) die(what + ": wrong bytes in view " + std::to_string(k));
+}
+void scribble_views(std::vector<View>& views) {
+  for (auto& v : views) std::memset(v.ddst, 0xEE, v.want.size());
+}
+
+long exercise_views(mxp_engine* eng) {
+  std::mt19937 rng(77);
+  long checked = 0;
+  hipStream_t side;
+  if (hipStreamCreateWithFlags(&side, hipStreamNonBlocking) != hipSuccess) die("stream");
+  std::vector<std::vector<View>> groups(4);
+  int index = 0;
+  for (auto& g : groups)
+    for (int k = 0; k < 24; ++k) g.push_back(make_view(rng, index++));
+  int kinds[3] = {0, 0, 0};
+  for (auto& g : groups) {
+    std::vector<mxp_view_copy> abi;
+    for (const auto& v : g) abi.push_back(as_abi(v));
+    std::vector<int32_t> kind(abi.size());
+    OK(mxp_describe_views(eng, abi.data(), (int64_t)abi.size(), kind.data(), nullptr, nullptr));
+    for (int32_t k : kind) ++kinds[k];
+  }
+  if (!kinds[0] || !kinds[1] || !kinds[2])
+    die("the random views do not cover the three ways a view can run: " + std::to_string(kinds[0]) + " / " + std::to_string(kinds[1]) + " / " + std::to_string(kinds[2]));
+  // one view at a time, with its checksum
+  for (auto& g : groups) {
+    scribble_views(g);
+    for (auto& v : g) {
+      const mxp_view_copy c = as_abi(v);
+      uint32_t got = 0;
+      OK(mxp_copy_view(eng, c.src, c.dst, c.ndim, c.shape, c.src_strides, c.dst_strides, c.elem_size, c.cast, &got, nullptr));
+      if (got != v.csum) die("copy_view checksum");
+    }
+    check_views(g, "mxp_copy_view");
+    checked += (long)g.size();
+  }
+  // batched calls back to back on two streams, nothing waited for in between: the descriptor arenas are taken in turn
+  for (int rep = 0; rep < 2; ++rep) {
+    for (auto& g : groups) scribble_views(g);
+    for (size_t gi = 0; gi < groups.size(); ++gi) {
+      std::vector<mxp_view_copy> abi;
+      for (const auto& v : groups[gi]) abi.push_back(as_abi(v));
+      OK(mxp_copy_views(eng, abi.data(), (int64_t)abi.size(), gi % 2 ? side : nullptr));
+    }
+    for (auto& g : groups) { check_views(g, "mxp_copy_views"); checked += (long)g.size(); }
+  }
+  // lowered once, run many times
+  for (size_t gi = 0; gi < groups.size(); ++gi) {
+    auto& g = groups[gi];
+    std::vector<mxp_view_copy> abi;
+    for (const auto& v : g) abi.push_back(as_abi(v));
+    mxp_view_plan* vp = nullptr;
+    OK(mxp_view_plan_create(eng, abi.data(), (int64_t)abi.size(), &vp));
+    uint64_t bytes = 0, want_bytes = 0;
+    OK(mxp_view_plan_bytes(vp, &bytes));
+    for (const auto& v : g) { int64_t n = v.eo; for (int64_t e : v.shape) n *= e; want_bytes += (uint64_t)n; }
+    if (bytes != want_bytes) die("view plan byte count");
+    for (int rep = 0; rep < 3; ++rep) {
+      scribble_views(g);
+      OK(mxp_view_plan_run(eng, vp, rep == 1 ? side : nullptr));
+      check_views(g, "mxp_view_plan_run");
+      checked += (long)g.size();
+    }
+    mxp_view_plan_destroy(vp);
+  }
+  // boxes, whole-buffer copies, a cast and a pitched gather with their checksums
+  {
+    const size_t n = 70000;
+    std::vector<uint8_t> host(n * 4);
+    for (auto& b : host) b = (uint8_t)rng();
+    for (size_t i = 3; i < host.size(); i += 4) host[i] &= 0x3F;
+    uint8_t *a = nullptr, *b = nullptr;
+    if (hipMalloc(reinterpret_cast<void**>(&a), host.size()) != hipSuccess || hipMalloc(reinterpret_cast<void**>(&b), host.size()) != hipSuccess) die("hipMalloc");
+    std::memcpy(a, host.data(), host.size());
+    uint32_t got = 0;
+    OK(mxp_cast(eng, a, b, n, MXP_CAST_F32_BF16, &got, nullptr));
+    std::vector<uint8_t> want(n * 2);
+    for (size_t i = 0; i < n; ++i) { uint32_t u; std::memcpy(&u, host.data() + 4 * i, 4); const uint16_t h = f32_to_bf16(u); std::memcpy(want.data() + 2 * i, &h, 2); }
+    if (std::memcmp(b, want.data(), want.size()) != 0 || got != checksum(want)) die("mxp_cast");
+    OK(mxp_gather2d(eng, a + 48, 1000, b, 304, 200, 300, &got, side));
+    std::vector<uint8_t> rows;
+    uint32_t want_sum = 0;
+    for (size_t r = 0; r < 200; ++r)
+      for (size_t c = 0; c < 300; ++c) {
+        if (b[r * 304 + c] != host[48 + r * 1000 + c]) die("mxp_gather2d bytes");
+        want_sum += b[r * 304 + c] * ((uint32_t)(r * 304 + c) * 2654435761u + 1u);
+      }
+    if (got != want_sum) die("mxp_gather2d checksum");
+    const void* srcs[3] = {a, a + 4096, a + 100000};
+    void* dsts[3] = {b, b + 8192, b + 120000};
+    const uint64_t sizes[3] = {4000, 1, 65537};
+    uint32_t sums[3];
+    OK(mxp_copy_batch(eng, srcs, dsts, sizes, 3, sums, nullptr));
+    for (int k = 0; k < 3; ++k) {
+      const std::vector<uint8_t> piece(static_cast<const uint8_t*>(srcs[k]), static_cast<const uint8_t*>(srcs[k]) + sizes[k]);
+      if (std::memcmp(dsts[k], piece.data(), piece.size()) != 0 || sums[k] != checksum(piece)) die("mxp_copy_batch");
+    }
+    (void)hipFree(a);
+    (void)hipFree(b);
+    checked += 5;
+  }
+  for (auto& g : groups)
+    for (auto& v : g) { (void)hipFree(v.dsrc); (void)hipFree(v.ddst); }
+  (void)hipStreamDestroy(side);
+  return checked;
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -387,6 +610,9 @@ int main(int argc, char** argv) {
   m32.plan = nullptr;
   close_model(m16);
   close_model(m32);
-  std::printf("ok: %ld placements checked, %" PRIu64 " stream operations run\n", runs, cpu_hip::operations_run());
+  mxp_engine* e3 = make_engine(3, 1 << 16, 2, 2, 1, 0);
+  const long views = exercise_views(e3);
+  mxp_engine_destroy(e3);
+  std::printf("ok: %ld placements and %ld view copies checked, %" PRIu64 " stream operations run\n", runs, views, cpu_hip::operations_run());
   return 0;
 }

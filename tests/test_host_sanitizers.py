@@ -125,13 +125,13 @@ def test_engine_ring_and_streams_under_thread_sanitizer(engine_binaries, tmp_pat
     _skip_if_tsan_cannot_map(r)
     assert r.returncode == 0, (r.stdout[-2000:], r.stderr[-6000:])
     assert "ThreadSanitizer" not in r.stderr, r.stderr[-6000:]
-    assert r.stdout.startswith("ok: 63 placements checked"), r.stdout
+    assert r.stdout.startswith("ok: 63 placements and 581 view copies checked"), r.stdout
 
 
 def test_engine_ring_and_streams_under_address_sanitizer(engine_binaries, tmp_path):
     r = subprocess.run([str(engine_binaries["asan"]), str(tmp_path)], capture_output=True, text=True, env=_env(), timeout=900)
     _clean(r)
-    assert r.stdout.startswith("ok: 63 placements checked"), r.stdout
+    assert r.stdout.startswith("ok: 63 placements and 581 view copies checked"), r.stdout
 
 
 def test_thread_sanitizer_reports_a_ring_slot_reused_too_early(engine_binaries, tmp_path):
