@@ -15,6 +15,7 @@
 #include <atomic>
 #include <chrono>
 #include <condition_variable>
+#include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <memory>
@@ -920,6 +921,11 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
   unsigned long long* const dsums_dev = L.digest_sums(L.cur);
   HIP_OK(hipStreamSynchronize(e.streams[0]));
   for (auto& s : e.slots) s->submitted = 0;
+  // MXP_INGEST_TRACE (read by the library itself, once): one line per ingest on stderr with the times at which the
+  // first chunk had been read, the last one, the readers were done and the streams idle.
+  static const bool trace = std::getenv("MXP_INGEST_TRACE") != nullptr;
+  const double t_tables = now_s();
+  std::atomic<double> t_first_submit{0.0}, t_last_read{0.0};
 
   std::atomic<size_t> next{0};
   std::atomic<bool> abort{false};
@@ -998,6 +1004,13 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
                          ck.files[r.file].path, r.need);
         }
         read_s[tid] += now_s() - t0;
+        if (trace) {
+          const double t = now_s();
+          double seen = t_first_submit.load();
+          while (seen == 0.0 && !t_first_submit.compare_exchange_weak(seen, t)) {}
+          double last = t_last_read.load();
+          while (last < t && !t_last_read.compare_exchange_weak(last, t)) {}
+        }
         hipStream_t st = e.streams[(c % n_slots) % e.streams.size()];
         mutated.store(1);
         for (const auto& r : ch.bounce_runs)
@@ -1037,11 +1050,16 @@ void do_execute(mxp_engine& e, mxp_plan& pl, void* const* dst_ptrs, hipStream_t 
     for (int t = 0; t < n_thr; ++t) pool.emplace_back(worker, t);
     for (auto& t : pool) t.join();
   }
+  const double t_join = now_s();
   hipError_t sync_err = hipSuccess;
   for (auto st : e.streams) {
     const hipError_t r = hipStreamSynchronize(st);
     if (r != hipSuccess) sync_err = r;
   }
+  if (trace)
+    std::fprintf(stderr, "[mxp ingest] set-up %.3f ms, first chunk read %.3f ms later, last chunk read at %.3f ms, readers joined at %.3f ms, streams idle at %.3f ms (%zu chunks)\n",
+                 (t_tables - t_start) * 1e3, (t_first_submit.load() - t_tables) * 1e3, (t_last_read.load() - t_start) * 1e3,
+                 (t_join - t_start) * 1e3, (now_s() - t_start) * 1e3, n_chunks);
   if (stats) {
     stats->wall_seconds = now_s() - t_start;
     for (double r : read_s) stats->read_seconds += r;

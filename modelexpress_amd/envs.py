@@ -56,6 +56,9 @@ environment_variables: dict[str, Callable[[], Any]] = {
     "MXP_NAN_BITS": lambda: _env_int("MXP_NAN_BITS", 0),
     # Fail the load when a checksum differs from the manifest the caller supplied.
     "MXP_VERIFY_CHECKSUMS": lambda: _env_bool("MXP_VERIFY_CHECKSUMS", True),
+    # Read by the library itself (not through this registry), once per process: when set, every ingest prints one line
+    # on stderr with the times of its phases (first chunk read, last chunk read, readers done, streams idle).
+    "MXP_INGEST_TRACE": lambda: os.environ.get("MXP_INGEST_TRACE"),
     # Allow fp32 checkpoints to be cast into bf16 parameters (refit).
     "MXP_ALLOW_CAST": lambda: _env_bool("MXP_ALLOW_CAST", False),
     # Coverage gate of a refit, same names and defaults as the reference (modelexpress/envs.py:266-272):
